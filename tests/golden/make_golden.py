@@ -1,0 +1,50 @@
+"""Writes tests/golden/gemm_small.npz: small seeded inputs and expected outputs for both GEMMs.
+
+The reference cannot produce these (no FP8 entry point, CUDA-only kernels, no fixtures of its own), so the
+expected values come from the closed forms in oracle/gemm_oracle.py evaluated in fp64, cross-checked here against
+the C triple loop before anything is written. Run from the repository root: `python tests/golden/make_golden.py`.
+"""
+import os
+import sys
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+sys.path.insert(0, ROOT)
+import oracle                     # noqa: E402
+from oracle import c_oracle       # noqa: E402
+
+
+def main():
+    rng = np.random.default_rng(20240607)
+    out = {}
+    # FP8 block-scaled, 64 x 256 x 384 (3 K blocks, 2 weight-scale rows), N(0,1) sources
+    x = rng.standard_normal((64, 384)).astype(np.float32)
+    w = rng.standard_normal((256, 384)).astype(np.float32)
+    qa, sa = oracle.per_token_cast_to_fp8(x)
+    qb, sb = oracle.per_block_cast_to_fp8(w)
+    exp = oracle.gemm_fp8_block_scaled_ref(qa, sa, qb, sb, np.float64)
+    assert oracle.calc_diff(c_oracle.gemm_fp8_nt(qa, sa, qb, sb), exp) < 1e-14
+    out.update(fp8_lhs=qa, fp8_lhs_scales=sa, fp8_rhs=qb, fp8_rhs_scales=sb, fp8_expected_f64=exp)
+    # bf16, 96 x 80 x 136 (k is not a multiple of 64: exercises the K tail)
+    a = oracle.f32_to_bf16_bits(rng.standard_normal((96, 136)).astype(np.float32))
+    b = oracle.f32_to_bf16_bits(rng.standard_normal((80, 136)).astype(np.float32))
+    exp = oracle.gemm_bf16_tn_ref(oracle.bf16_bits_to_f32(a), oracle.bf16_bits_to_f32(b), np.float64)
+    assert np.allclose(c_oracle.gemm_bf16_tn(a, b), exp, rtol=1e-12, atol=1e-12)
+    out.update(bf16_a_bits=a, bf16_b_bits=b, bf16_expected_f64=exp)
+    # exact-integer FP8 case with power-of-two scales, 40 x 192 x 256: a kernel must reproduce it bit for bit
+    va = rng.integers(-4, 5, size=(40, 256)).astype(np.float32)
+    vb = rng.integers(-4, 5, size=(192, 256)).astype(np.float32)
+    isa = (2.0 ** rng.integers(-2, 3, size=(40, 2))).astype(np.float32)
+    isb = (2.0 ** rng.integers(-2, 3, size=(2, 2))).astype(np.float32)
+    ia, ib = oracle.e4m3fn_encode(va), oracle.e4m3fn_encode(vb)
+    iexp = oracle.gemm_fp8_block_scaled_ref(ia, isa, ib, isb)
+    assert np.array_equal(iexp, c_oracle.gemm_fp8_nt(ia, isa, ib, isb))
+    out.update(int_lhs=ia, int_lhs_scales=isa, int_rhs=ib, int_rhs_scales=isb, int_expected=iexp)
+    path = os.path.join(ROOT, 'tests', 'golden', 'gemm_small.npz')
+    np.savez_compressed(path, **out)
+    print('wrote', path, os.path.getsize(path), 'bytes')
+
+
+if __name__ == '__main__':
+    main()

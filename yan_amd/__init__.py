@@ -1,0 +1,7 @@
+"""MI355X-native GEMM hot path behind the JIT / operator surface of zoheth/yan (`yan/__init__.py:3-5`)."""
+import torch
+
+from . import jit
+from .jit_kernels import (gemm, gemm_bf16_tn, gemm_fp16_tn, gemm_fp8_fp8_bf16_nt, get_col_major_tensor,
+                          set_num_sms, get_num_sms, ceil_div, get_m_alignment_for_contiguous_layout)
+from .utils import bench_kineto, calc_diff, count_bytes

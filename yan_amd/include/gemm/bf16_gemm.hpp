@@ -1,0 +1,205 @@
+// C[m,n] = A[m,k] . B[n,k]^T for bf16 (or fp16) operands, fp32 accumulation, gfx950.
+//
+// Entry point `gemm_tn<BLOCK_M, BLOCK_N, NUM_STAGES>` keeps the signature and layout contract of the
+// reference's launcher (yan/include/gemm/cute_gemm.cuh:262-378: A [m,k] and B [n,k] row-major with K
+// contiguous, C [m,n] row-major written in place, work enqueued on `stream`), but none of its structure:
+// the reference kernel (cute_gemm.cuh:14-260) is a 128x128x32 cp.async/ldmatrix/mma.sync pipeline with fp16
+// accumulation and no bounds handling. Here:
+//   * macro tile BLOCK_M x BLOCK_N x 64 (128-byte rows), 8 waves (2 per SIMD) for big tiles, 4 otherwise;
+//   * HBM -> LDS with buffer_load ... lds into two static LDS stages (tile_io.hpp);
+//   * each wave owns a (BLOCK_N/WAVES_N) x (BLOCK_M/WAVES_M) slab computed with 32x32x16 MFMAs. B rows feed the
+//     MFMA row operand and A rows the column operand, so a lane's four consecutive accumulator registers are
+//     four consecutive n of one m: contiguous in C;
+//   * fp32 accumulators, round-to-nearest-even on the way out;
+//   * any m and n (n % 4 == 0), k % 8 == 0; rows beyond m / n and the k tail read as zero.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <hip/hip_bf16.h>
+#include <hip/hip_fp16.h>
+
+#include "utils.hpp"
+#include "mfma_utils.hpp"
+#include "scheduler.hpp"
+#include "tile_io.hpp"
+
+namespace yan {
+
+template <int BLOCK_M, int BLOCK_N>
+struct DenseTileConfig {
+    static constexpr int NUM_WAVES = get_num_waves(BLOCK_M, BLOCK_N);
+    // A slab of at most 128 x 64 outputs: 128 accumulator registers per lane.
+    static constexpr int WAVES_N   = pick_waves_n(BLOCK_M, BLOCK_N, NUM_WAVES, 32, 128 * 64);
+    static_assert(WAVES_N > 0, "no wave layout fits this tile");
+    static constexpr int WAVES_M   = NUM_WAVES / WAVES_N;
+    static constexpr int WTN = BLOCK_N / WAVES_N, WTM = BLOCK_M / WAVES_M;
+    static_assert(WTN % 32 == 0 && WTM % 32 == 0, "wave slab must be a whole number of 32x32 atoms");
+    static constexpr int LDS_BYTES = 2 * (BLOCK_M + BLOCK_N) * kRowBytes;
+    static_assert(LDS_BYTES <= 160 * 1024, "two stages must fit the 160 KB LDS");
+};
+
+template <typename Atom, typename Elem, int BLOCK_M, int BLOCK_N>
+__global__ void __launch_bounds__((get_num_waves(BLOCK_M, BLOCK_N) * kWaveSize))
+dense_gemm_mfma(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, Elem* __restrict__ C,
+                int m, int n, int k) {
+    using Cfg = DenseTileConfig<BLOCK_M, BLOCK_N>;
+    constexpr int NW = Cfg::NUM_WAVES, TN = Cfg::WTN / 32, TM = Cfg::WTM / 32;
+
+    __shared__ __attribute__((aligned(1024))) uint8_t lds_a0[BLOCK_M * kRowBytes];
+    __shared__ __attribute__((aligned(1024))) uint8_t lds_b0[BLOCK_N * kRowBytes];
+    __shared__ __attribute__((aligned(1024))) uint8_t lds_a1[BLOCK_M * kRowBytes];
+    __shared__ __attribute__((aligned(1024))) uint8_t lds_b1[BLOCK_N * kRowBytes];
+
+    const XcdTileScheduler<> sched(m, n, BLOCK_M, BLOCK_N);
+    const TileCoord tile = sched.tile_of(blockIdx.x);
+    if (!tile.valid) return;
+    const int m0 = tile.m_idx * BLOCK_M, n0 = tile.n_idx * BLOCK_N;
+
+    const int lane = get_lane_id();
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWaveSize);
+    const int wn = wave % Cfg::WAVES_N, wm = wave / Cfg::WAVES_N;
+
+    const uint32_t ld_bytes = uint32_t(k) * 2;
+    const __amdgpu_buffer_rsrc_t rsrc_a = make_rsrc(A, uint32_t(m) * ld_bytes);
+    const __amdgpu_buffer_rsrc_t rsrc_b = make_rsrc(B, uint32_t(n) * ld_bytes);
+    TileStager<BLOCK_M, NW> stage_a;
+    TileStager<BLOCK_N, NW> stage_b;
+    stage_a.init(m0, ld_bytes, wave, lane);
+    stage_b.init(n0, ld_bytes, wave, lane);
+
+    // k-tiles: `num_k_tiles` in all, the last one possibly partial (only `tail_bytes` of each row exist).
+    const int k_bytes = k * 2;
+    const int num_k_tiles = ceil_div(k_bytes, kRowBytes);
+    const int tail_tile = (k_bytes % kRowBytes) ? num_k_tiles - 1 : -1;
+    const uint32_t tail_a = stage_a.tail_voff(k_bytes % kRowBytes), tail_b = stage_b.tail_voff(k_bytes % kRowBytes);
+    auto prefetch = [&](int kt, uint8_t* la, uint8_t* lb) {
+        const bool tail = kt == tail_tile;
+        stage_a.issue_from(rsrc_a, la, kt * kRowBytes, wave, tail ? tail_a : stage_a.voff);
+        stage_b.issue_from(rsrc_b, lb, kt * kRowBytes, wave, tail ? tail_b : stage_b.voff);
+    };
+
+    // Lane-constant LDS offsets of the four 16-deep K steps inside a 64-deep tile.
+    const int g = lane / 32;
+    int koff[4];
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk) koff[kk] = frag_offset<32>(lane, 2 * kk + g);
+
+    typename Atom::Acc acc[TN][TM];
+#pragma unroll
+    for (int i = 0; i < TN; ++i)
+#pragma unroll
+        for (int j = 0; j < TM; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+    // One k-tile = four 16-deep steps; the fragments of step kk+1 are fetched before the MFMAs of step kk issue.
+    auto compute_tile = [&](const uint8_t* la, const uint8_t* lb) {
+        using Frag = typename Atom::Frag;
+        const uint8_t* pa = la + wm * Cfg::WTM * kRowBytes;
+        const uint8_t* pb = lb + wn * Cfg::WTN * kRowBytes;
+        Frag nf[2][TN], mf[2][TM];
+        auto fetch = [&](int kk) {
+#pragma unroll
+            for (int i = 0; i < TN; ++i) nf[kk & 1][i] = *reinterpret_cast<const Frag*>(pb + i * 32 * kRowBytes + koff[kk]);
+#pragma unroll
+            for (int j = 0; j < TM; ++j) mf[kk & 1][j] = *reinterpret_cast<const Frag*>(pa + j * 32 * kRowBytes + koff[kk]);
+        };
+        fetch(0);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int kk = 0; kk < 4; ++kk) {
+            if (kk + 1 < 4) fetch(kk + 1);
+#pragma unroll
+            for (int i = 0; i < TN; ++i)
+#pragma unroll
+                for (int j = 0; j < TM; ++j) acc[i][j] = Atom::mma(nf[kk & 1][i], mf[kk & 1][j], acc[i][j]);
+            // Issue order inside the step: one LDS read, one MFMA, ... so the reads ride under the MFMAs.
+            if (kk + 1 < 4) {
+#pragma unroll
+                for (int x = 0; x < TN + TM; ++x) {
+                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                }
+                __builtin_amdgcn_sched_group_barrier(0x008, TN * TM - (TN + TM), 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+
+    // Two LDS stages; the copy of tile kt+1 is in flight while tile kt is consumed. The barrier both publishes
+    // the tile that just landed and retires every wave's reads of the stage about to be overwritten. The
+    // steady-state body is branch-free: a copy started for a tile past the end is simply never consumed.
+    prefetch(0, lds_a0, lds_b0);
+    int kt = 0;
+    for (; kt + 1 < num_k_tiles; kt += 2) {
+        __syncthreads();
+        prefetch(kt + 1, lds_a1, lds_b1);
+        compute_tile(lds_a0, lds_b0);
+        __syncthreads();
+        prefetch(kt + 2, lds_a0, lds_b0);
+        compute_tile(lds_a1, lds_b1);
+    }
+    if (kt < num_k_tiles) {
+        __syncthreads();
+        compute_tile(lds_a0, lds_b0);
+    }
+
+    // Epilogue: registers 4*q .. 4*q+3 of an atom are n = 8*q + 4*g + {0,1,2,3} of column m = lane % 32.
+    const int m_lane = m0 + wm * Cfg::WTM + lane % 32;
+    const int n_lane = n0 + wn * Cfg::WTN + 4 * g;
+#pragma unroll
+    for (int j = 0; j < TM; ++j) {
+        const int mm = m_lane + j * 32;
+        if (mm >= m) continue;
+        Elem* row = C + size_t(mm) * n;
+#pragma unroll
+        for (int i = 0; i < TN; ++i)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int nn = n_lane + i * 32 + q * 8;
+                if (nn < n) {
+                    const f32x4 v = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
+                    *reinterpret_cast<decltype(pack4(v, Elem{}))*>(row + nn) = pack4(v, Elem{});
+                }
+            }
+    }
+}
+
+// Arguments every dense launcher checks before touching the GPU. Returns hipSuccess or hipErrorInvalidValue.
+inline hipError_t check_dense_args(int m, int n, int k, const void* a, const void* b, const void* c,
+                                   int block_m, int block_n) {
+    if (m < 0 || n < 0 || k <= 0 || (n % 4) != 0 || (k % 8) != 0) return hipErrorInvalidValue;
+    if (!a || !b || !c) return hipErrorInvalidValue;
+    // 32-bit descriptor offsets: every tile row, including the overhang of the last tile, must stay below 2 GiB
+    const uint64_t m_pad = uint64_t(ceil_div(m, block_m)) * block_m, n_pad = uint64_t(ceil_div(n, block_n)) * block_n;
+    if (m_pad * k * 2 >= kOutOfRange || n_pad * k * 2 >= kOutOfRange) return hipErrorInvalidValue;
+    return hipSuccess;
+}
+
+template <typename Atom, typename Elem, int BLOCK_M, int BLOCK_N>
+inline hipError_t launch_dense(int m, int n, int k, const void* a, const void* b, void* c, hipStream_t stream) {
+    if (m == 0 || n == 0) return hipSuccess;
+    if (hipError_t e = check_dense_args(m, n, k, a, b, c, BLOCK_M, BLOCK_N); e != hipSuccess) return e;
+    using Cfg = DenseTileConfig<BLOCK_M, BLOCK_N>;
+    const XcdTileScheduler<> sched(m, n, BLOCK_M, BLOCK_N);
+    hipLaunchKernelGGL((dense_gemm_mfma<Atom, Elem, BLOCK_M, BLOCK_N>), dim3(sched.grid_size()),
+                       dim3(Cfg::NUM_WAVES * kWaveSize), 0, stream, static_cast<const uint8_t*>(a),
+                       static_cast<const uint8_t*>(b), static_cast<Elem*>(c), m, n, k);
+    return hipGetLastError();
+}
+
+} // namespace yan
+
+// bf16 in, fp32 accumulate, bf16 out. NUM_STAGES is accepted for interface parity; the kernel always runs two
+// LDS stages (two 256x256x64 stages are 128 KB of the 160 KB).
+template <int BLOCK_M, int BLOCK_N, int NUM_STAGES>
+inline hipError_t gemm_tn(int m, int n, int k, const __hip_bfloat16* A, const __hip_bfloat16* B, __hip_bfloat16* C,
+                          hipStream_t stream) {
+    return yan::launch_dense<yan::MfmaBF16_32x32x16, __bf16, BLOCK_M, BLOCK_N>(m, n, k, A, B, C, stream);
+}
+
+// fp16 in, fp32 accumulate, fp16 out.
+template <int BLOCK_M, int BLOCK_N, int NUM_STAGES>
+inline hipError_t gemm_tn(int m, int n, int k, const __half* A, const __half* B, __half* C, hipStream_t stream) {
+    return yan::launch_dense<yan::MfmaF16_32x32x16, _Float16, BLOCK_M, BLOCK_N>(m, n, k, A, B, C, stream);
+}

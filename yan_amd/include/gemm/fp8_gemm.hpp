@@ -1,0 +1,249 @@
+// out[m,n] = sum_kb sA[m,kb] * sB[n/128,kb] * sum_{t<128} A8[m,128kb+t] * B8[n,128kb+t]   (e4m3 x e4m3 -> fp32 -> bf16)
+//
+// The block-scaled FP8 GEMM of the reference's yan/include/gemm/fp8_gemm.cuh (template parameters :32-39,
+// kernel signature :40-46, BLOCK_K == 128 :48, one A scale per row and K block and one or two B scales per tile
+// and K block :55-61), which in the reference is an unfinished Hopper kernel built on TMA descriptors, cluster
+// barriers and warpgroup MMAs. This is a different kernel for gfx950:
+//   * macro tile BLOCK_M x BLOCK_N x 128 (one scale block per k-tile, 128-byte rows); 8 waves, two per SIMD, so
+//     one wave's scale arithmetic and LDS traffic hide under the other's MFMAs;
+//   * HBM -> LDS with buffer_load ... lds into two static LDS stages (tile_io.hpp);
+//   * 16x16x128 e4m3 MFMAs: one instruction covers a whole scale block, starts from a zero accumulator and
+//     yields 4 partial sums per lane, which the VALU folds into the running fp32 sums as acc += partial * s,
+//     s = sA * sB. Weights feed the MFMA row operand and activations the column operand, so a lane only ever
+//     meets one activation row per atom: one sA per lane per atom per K block, and sB is wave-uniform;
+//   * the running sums stay in architectural VGPRs (the VALU cannot address AGPRs): 128 per wave;
+//   * m is a run-time argument with tails predicated; N and K are compile-time.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <hip/hip_bf16.h>
+#include <hip/hip_fp8.h>
+
+#include "utils.hpp"
+#include "mfma_utils.hpp"
+#include "scheduler.hpp"
+#include "tile_io.hpp"
+
+namespace yan {
+
+template <int BLOCK_M, int BLOCK_N>
+struct Fp8TileConfig {
+    static constexpr int NUM_WAVES = get_num_waves(BLOCK_M, BLOCK_N);
+    static constexpr int WAVES_N   = pick_waves_n(BLOCK_M, BLOCK_N, NUM_WAVES, 16, 128 * 64);
+    static_assert(WAVES_N > 0, "no wave layout fits this tile");
+    static constexpr int WAVES_M   = NUM_WAVES / WAVES_N;
+    static constexpr int WTN = BLOCK_N / WAVES_N, WTM = BLOCK_M / WAVES_M;
+    static_assert(WTN % 16 == 0 && WTM % 16 == 0, "wave slab must be a whole number of 16x16 atoms");
+    static_assert(WTN * WTM <= 128 * 64, "running sums must fit 128 VGPRs per lane");
+    // A slab that divides a 128-wide scale block never straddles two of them.
+    static constexpr bool UNIFORM_SCALE_B = (128 % WTN == 0);
+    // Number of 128-wide scale blocks a slab of 16-aligned start can touch.
+    static constexpr int  SCALE_B_PER_SLAB = UNIFORM_SCALE_B ? 1 : (WTN + 112) / 128 + 1;
+    static constexpr int  LDS_BYTES = 2 * (BLOCK_M + BLOCK_N) * kRowBytes;
+    static_assert(LDS_BYTES <= 160 * 1024, "two stages must fit the 160 KB LDS");
+};
+
+template <int SHAPE_N, int SHAPE_K, int BLOCK_M, int BLOCK_N>
+__global__ void __launch_bounds__((get_num_waves(BLOCK_M, BLOCK_N) * kWaveSize))
+fp8_gemm_kernel(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_scales,
+                const uint8_t* __restrict__ rhs, const float* __restrict__ rhs_scales,
+                __bf16* __restrict__ out, int m, int n_rt, int k_rt, int sa_stride_m, int sa_stride_k) {
+    using Cfg  = Fp8TileConfig<BLOCK_M, BLOCK_N>;
+    using Atom = MfmaFP8_16x16x128;
+    constexpr int NW = Cfg::NUM_WAVES, TN = Cfg::WTN / 16, TM = Cfg::WTM / 16;
+    constexpr int NB = Cfg::SCALE_B_PER_SLAB;
+    static_assert(SHAPE_K % 128 == 0 && SHAPE_N % 4 == 0);
+    // SHAPE_N / SHAPE_K == 0 selects the run-time sizes (ahead-of-time library); the JIT bakes them in.
+    const int N = SHAPE_N ? SHAPE_N : n_rt, K = SHAPE_K ? SHAPE_K : k_rt;
+    const int NUM_K_BLOCKS = K / 128, NUM_N_BLOCKS = ceil_div(N, 128);
+
+    __shared__ __attribute__((aligned(1024))) uint8_t lds_a0[BLOCK_M * kRowBytes];
+    __shared__ __attribute__((aligned(1024))) uint8_t lds_b0[BLOCK_N * kRowBytes];
+    __shared__ __attribute__((aligned(1024))) uint8_t lds_a1[BLOCK_M * kRowBytes];
+    __shared__ __attribute__((aligned(1024))) uint8_t lds_b1[BLOCK_N * kRowBytes];
+
+    const XcdTileScheduler<> sched(m, N, BLOCK_M, BLOCK_N);
+    const TileCoord tile = sched.tile_of(blockIdx.x);
+    if (!tile.valid) return;
+    const int m0 = tile.m_idx * BLOCK_M, n0 = tile.n_idx * BLOCK_N;
+
+    const int lane = get_lane_id();
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWaveSize);
+    const int wn = wave % Cfg::WAVES_N, wm = wave / Cfg::WAVES_N;
+    const int g = lane / 16, col = lane % 16;
+    const int m_slab = m0 + wm * Cfg::WTM, n_slab = n0 + wn * Cfg::WTN;
+
+    const __amdgpu_buffer_rsrc_t rsrc_a = make_rsrc(lhs, uint32_t(m) * K);
+    const __amdgpu_buffer_rsrc_t rsrc_b = make_rsrc(rhs, uint32_t(N) * K);
+    TileStager<BLOCK_M, NW> stage_a;
+    TileStager<BLOCK_N, NW> stage_b;
+    stage_a.init(m0, K, wave, lane);
+    stage_b.init(n0, K, wave, lane);
+
+    // Activation scales through a descriptor as well: element (row, kb) at (row*stride_m + kb*stride_k) floats.
+    // Atom j of the slab covers rows m_slab + 16j + col; rows past m read as 0 or as some other row's scale,
+    // either of which only ever multiplies the zero partial sums of a row that is never stored.
+    const uint32_t sa_bytes = (uint32_t(m - 1) * sa_stride_m + uint32_t(NUM_K_BLOCKS - 1) * sa_stride_k + 1) * 4;
+    const __amdgpu_buffer_rsrc_t rsrc_sa = make_rsrc(lhs_scales, sa_bytes);
+    const uint32_t sa_voff = uint32_t(m_slab + col) * sa_stride_m * 4;
+    // Weight scales: rows base_blk .. base_blk+NB-1 of the [N/128, K/128] table cover the slab.
+    const int base_blk = n_slab / 128;
+
+    const int off0 = frag_offset<16>(lane, 2 * g), off1 = frag_offset<16>(lane, 2 * g + 1);
+    auto read_frag = [&](const uint8_t* atom_rows) {
+        const i32x4 lo = *reinterpret_cast<const i32x4*>(atom_rows + off0);
+        const i32x4 hi = *reinterpret_cast<const i32x4*>(atom_rows + off1);
+        return i32x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    };
+
+    f32x4 acc[TN][TM];
+#pragma unroll
+    for (int i = 0; i < TN; ++i)
+#pragma unroll
+        for (int j = 0; j < TM; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    float sa_next[TM];     // activation scales of the k-tile in flight
+    float sb_next[NB];     // weight scales of the k-tile in flight (wave-uniform)
+    auto load_scales = [&](int kb) {
+#pragma unroll
+        for (int j = 0; j < TM; ++j)
+            sa_next[j] = buffer_load_f32(rsrc_sa, sa_voff, (kb * sa_stride_k + j * 16 * sa_stride_m) * 4);
+#pragma unroll
+        for (int b = 0; b < NB; ++b) sb_next[b] = rhs_scales[min(base_blk + b, NUM_N_BLOCKS - 1) * NUM_K_BLOCKS + kb];
+    };
+
+    // One k-tile: TN x TM atoms, software-pipelined by hand. Step t issues the MFMA of atom t (fresh zero
+    // accumulator) and folds in the partial sums of atom t - DEPTH, whose MFMA has retired by then; the fragment of
+    // weight rows i+1 is fetched while rows i are being multiplied. sched_barrier keeps the compiler from
+    // regrouping the steps (it would otherwise hoist every MFMA and need a register per partial sum).
+    auto compute_tile = [&](const uint8_t* la, const uint8_t* lb, const float (&sa)[TM], const float (&sb)[NB]) {
+        constexpr int T = TN * TM, DEPTH = 2, RING = 4;
+        const uint8_t* pa = la + wm * Cfg::WTM * kRowBytes;
+        const uint8_t* pb = lb + wn * Cfg::WTN * kRowBytes;
+        i32x8 mf[TM], nf[2];
+        nf[0] = read_frag(pb);
+#pragma unroll
+        for (int j = 0; j < TM; ++j) mf[j] = read_frag(pa + j * 16 * kRowBytes);
+        float s[TM];
+        f32x4 p[RING];
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int t = 0; t < T + DEPTH; ++t) {
+            if (t < T) {
+                const int i = t / TM, j = t % TM;
+                if (j == 0 && i + 1 < TN) nf[(i + 1) & 1] = read_frag(pb + (i + 1) * 16 * kRowBytes);
+                p[t % RING] = Atom::mma(nf[i & 1], mf[j], f32x4{0.f, 0.f, 0.f, 0.f});
+            }
+            if (t >= DEPTH) {
+                const int u = t - DEPTH, i = u / TM, j = u % TM;
+                if (j == 0) {
+                    // (re)compute s = sA * sB on entering the slab and whenever rows i cross into the next 128-block
+                    const bool fresh = (i == 0) || (!Cfg::UNIFORM_SCALE_B && ((n_slab + i * 16) & 127) == 0);
+                    if (fresh) {
+                        float sbv = sb[0];
+                        if constexpr (NB > 1) {
+                            const int rel = (n_slab + i * 16) / 128 - base_blk;
+#pragma unroll
+                            for (int b = 1; b < NB; ++b) sbv = (rel == b) ? sb[b] : sbv;
+                        }
+#pragma unroll
+                        for (int jj = 0; jj < TM; ++jj) s[jj] = sa[jj] * sbv;
+                    }
+                }
+#pragma unroll
+                for (int r = 0; r < 4; ++r) acc[i][j][r] = __builtin_fmaf(p[u % RING][r], s[j], acc[i][j][r]);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+
+    // Two LDS stages, one k-tile (= one scale block) of prefetch; the scales of the next block travel in
+    // registers alongside. The steady-state body is branch-free (a copy past the last k-tile is out of range
+    // for the descriptor and moves zeros), which keeps each MFMA/FMA step where it was written.
+    float sa_cur[TM], sb_cur[NB];
+    auto rotate_scales = [&]() {
+#pragma unroll
+        for (int j = 0; j < TM; ++j) sa_cur[j] = sa_next[j];
+#pragma unroll
+        for (int b = 0; b < NB; ++b) sb_cur[b] = sb_next[b];
+    };
+    auto prefetch = [&](int kb, uint8_t* la, uint8_t* lb) {
+        stage_a.issue(rsrc_a, la, kb * kRowBytes, wave);
+        stage_b.issue(rsrc_b, lb, kb * kRowBytes, wave);
+        load_scales(min(kb, NUM_K_BLOCKS - 1));
+    };
+    prefetch(0, lds_a0, lds_b0);
+    for (int kb = 0; kb + 1 < NUM_K_BLOCKS; kb += 2) {
+        rotate_scales();
+        __syncthreads();
+        prefetch(kb + 1, lds_a1, lds_b1);
+        compute_tile(lds_a0, lds_b0, sa_cur, sb_cur);
+        rotate_scales();
+        __syncthreads();
+        prefetch(kb + 2, lds_a0, lds_b0);
+        compute_tile(lds_a1, lds_b1, sa_cur, sb_cur);
+    }
+    if (NUM_K_BLOCKS % 2 == 1) {
+        rotate_scales();
+        __syncthreads();
+        compute_tile(lds_a0, lds_b0, sa_cur, sb_cur);
+    }
+
+    // Epilogue: the 4 registers of atom (i, j) are n = n_slab + 16i + 4g + {0..3} of row m = m_slab + 16j + col.
+#pragma unroll
+    for (int j = 0; j < TM; ++j) {
+        const int mm = m_slab + j * 16 + col;
+        if (mm >= m) continue;
+        __bf16* row = out + size_t(mm) * N;
+#pragma unroll
+        for (int i = 0; i < TN; ++i) {
+            const int nn = n_slab + i * 16 + 4 * g;
+            if (nn < N) *reinterpret_cast<bf16x4*>(row + nn) = pack4(acc[i][j], __bf16{});
+        }
+    }
+}
+
+// Host side of the kernel, shaped after the class the reference's JIT template instantiates
+// (yan/jit_kernels/gemm.py:20-30: Gemm<N, K, BLOCK_M, BLOCK_N, 128, 1, kNumStages, kNumTMAMulticast, Normal>::run).
+// BLOCK_K is fixed at 128; kNumGroups, kNumStages and kNumTMAMulticast are accepted and unused: the kernel always
+// runs two LDS stages and gfx950 has no multicast copy. `num_sms` and `smem_size` are accepted likewise (one
+// workgroup per tile, static LDS).
+template <uint32_t SHAPE_N, uint32_t SHAPE_K, uint32_t BLOCK_M, uint32_t BLOCK_N, uint32_t BLOCK_K,
+          uint32_t kNumGroups, uint32_t kNumStages, uint32_t kNumTMAMulticast, GemmType kGemmType>
+class Gemm {
+    static_assert(BLOCK_K == 128, "one k-tile is one 128-deep scale block");
+    static_assert(kGemmType == GemmType::Normal && kNumGroups == 1, "grouped layouts are not implemented");
+
+public:
+    // lhs [m, K] e4m3 row-major; lhs_scales fp32, element (i, kb) at i * stride_m + kb * stride_k;
+    // rhs [N, K] e4m3 row-major; rhs_scales fp32 [ceil(N/128), K/128] row-major; out [m, N] bf16 row-major.
+    static hipError_t run(__hip_bfloat16* out, const void* lhs, const float* lhs_scales, int lhs_scales_stride_m,
+                          int lhs_scales_stride_k, const void* rhs, const float* rhs_scales, int m,
+                          hipStream_t stream, int num_sms, uint32_t smem_size) {
+        return run_sized(out, lhs, lhs_scales, lhs_scales_stride_m, lhs_scales_stride_k, rhs, rhs_scales, m,
+                         int(SHAPE_N), int(SHAPE_K), stream, num_sms, smem_size);
+    }
+
+    // Same with explicit n and k, which must equal SHAPE_N / SHAPE_K unless those are 0 (sizes known at run time).
+    static hipError_t run_sized(__hip_bfloat16* out, const void* lhs, const float* lhs_scales, int lhs_scales_stride_m,
+                                int lhs_scales_stride_k, const void* rhs, const float* rhs_scales, int m, int n, int k,
+                                hipStream_t stream, int num_sms, uint32_t smem_size) {
+        (void)num_sms, (void)smem_size;
+        if (m == 0 || n == 0) return hipSuccess;
+        if (m < 0 || n < 0 || k <= 0 || (n % 4) != 0 || (k % 128) != 0) return hipErrorInvalidValue;
+        if ((SHAPE_N && n != int(SHAPE_N)) || (SHAPE_K && k != int(SHAPE_K))) return hipErrorInvalidValue;
+        if (!out || !lhs || !lhs_scales || !rhs || !rhs_scales) return hipErrorInvalidValue;
+        // 32-bit descriptor offsets: every tile row, including the overhang of the last tile, must stay below 2 GiB
+        const uint64_t m_pad = uint64_t(ceil_div<uint32_t>(m, BLOCK_M)) * BLOCK_M, n_pad = uint64_t(ceil_div<uint32_t>(n, BLOCK_N)) * BLOCK_N;
+        if (m_pad * k >= kOutOfRange || n_pad * k >= kOutOfRange) return hipErrorInvalidValue;
+        using Cfg = Fp8TileConfig<BLOCK_M, BLOCK_N>;
+        const XcdTileScheduler<> sched(m, n, BLOCK_M, BLOCK_N);
+        hipLaunchKernelGGL((fp8_gemm_kernel<SHAPE_N, SHAPE_K, BLOCK_M, BLOCK_N>), dim3(sched.grid_size()),
+                           dim3(Cfg::NUM_WAVES * kWaveSize), 0, stream, static_cast<const uint8_t*>(lhs), lhs_scales,
+                           static_cast<const uint8_t*>(rhs), rhs_scales, reinterpret_cast<__bf16*>(out), m, n, k,
+                           lhs_scales_stride_m, lhs_scales_stride_k);
+        return hipGetLastError();
+    }
+};
+
+} // namespace yan

@@ -1,0 +1,94 @@
+// Moving K-major operand tiles HBM -> LDS -> MFMA fragments on gfx950, and writing accumulators back.
+//
+// Both GEMMs in this directory stage tiles whose rows are 128 bytes along K (64 bf16 or 128 e4m3 values).
+// This file is what stands in for the reference's TMA descriptors and swizzled shared-memory layouts
+// (yan/include/gemm/fp8_gemm.cuh:55-113, yan/include/gemm/cute_gemm.cuh:278-316).
+//
+// HBM -> LDS: `buffer_load_dwordx4 ... lds`. One wave instruction moves 64 x 16 bytes and the hardware places
+// lane i's 16 bytes at LDS address M0 + 16*i, i.e. one instruction fills 8 consecutive tile rows. The LDS side
+// is therefore fixed; the swizzle is applied on the global side by choosing WHICH 16-byte chunk of the row
+// each lane fetches. Rows past the end of the matrix get an offset beyond the descriptor's num_records, for
+// which the hardware returns zeros, so tails need no branches.
+//
+// LDS layout: row r of a tile starts at byte 128*r; its logical chunk c (16 bytes) sits in slot
+// c ^ swizzle_of_row(r). An MFMA operand read has lanes of consecutive rows fetch the same logical chunk; the
+// XOR spreads any 8 consecutive rows over the 8 slots and rows r, r+8 over different slots, so neither a
+// 32-bank nor a 64-bank LDS sees a conflict for ds_read_b128.
+#pragma once
+
+#include "utils.hpp"
+#include "mfma_utils.hpp"
+
+namespace yan {
+
+__device__ __forceinline__ int swizzle_of_row(int row) { return (row & 7) ^ ((row >> 3) & 1); }
+
+// Offsets at or above this fail the bounds check of every descriptor this code builds (all < 2 GiB).
+constexpr uint32_t kOutOfRange = 0x80000000u;
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, uint32_t bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, bytes, 0x00020000);
+}
+
+// One fp32 through a descriptor: per-lane byte offset + wave-uniform byte offset; out of range reads 0.0f.
+__device__ __forceinline__ float buffer_load_f32(__amdgpu_buffer_rsrc_t rsrc, uint32_t voffset, uint32_t soffset) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsrc, voffset, soffset, 0));
+}
+
+// Per-thread state for staging a ROWS x 128-byte tile with NUM_WAVES waves: one VGPR. Everything that varies
+// per pass or per k-tile is wave-uniform and rides in the instruction's scalar offset, which the hardware adds
+// before its bounds check; a row past the end of the matrix lands at or beyond num_records and reads as zero.
+template <int ROWS, int NUM_WAVES>
+struct TileStager {
+    static_assert(ROWS % 16 == 0 && NUM_WAVES % 2 == 0);
+    static constexpr int GROUPS = ROWS / 8;                       // 8-row groups, one instruction each
+    static constexpr int PASSES = ceil_div(GROUPS, NUM_WAVES);
+
+    uint32_t voff;        // byte offset of this lane's chunk for pass 0 at K = 0
+    uint32_t pass_pitch;  // bytes between the rows of consecutive passes (uniform)
+    int      logical;     // logical chunk index this lane fetches
+
+    // The tile starts at matrix row `tile_row0`; rows have a pitch of `ld_bytes`.
+    __device__ __forceinline__ void init(int tile_row0, uint32_t ld_bytes, int wave, int lane) {
+        const int sub = lane >> 3, slot = lane & 7;
+        logical    = slot ^ sub ^ (wave & 1);     // == slot ^ swizzle_of_row(8*q + sub) for every q = wave (mod 2)
+        voff       = uint32_t(tile_row0 + wave * 8 + sub) * ld_bytes + logical * kChunk;
+        pass_pitch = uint32_t(NUM_WAVES * 8) * ld_bytes;
+    }
+
+    // Start the copy of the k-tile at byte `k_byte0` of every row into `lds_tile`.
+    __device__ __forceinline__ void issue(__amdgpu_buffer_rsrc_t rsrc, uint8_t* lds_tile, int k_byte0, int wave) const {
+        issue_from(rsrc, lds_tile, k_byte0, wave, voff);
+    }
+
+    // Lane offset to use for a last k-tile of which only `valid_bytes` (a multiple of 16) per row exist: lanes
+    // whose chunk lies beyond the row end are sent out of range and move zeros.
+    __device__ __forceinline__ uint32_t tail_voff(int valid_bytes) const {
+        return logical * kChunk < valid_bytes ? voff : kOutOfRange;
+    }
+
+    __device__ __forceinline__ void issue_from(__amdgpu_buffer_rsrc_t rsrc, uint8_t* lds_tile, int k_byte0, int wave,
+                                               uint32_t lane_voff) const {
+#pragma unroll
+        for (int j = 0; j < PASSES; ++j) {
+            const int q = j * NUM_WAVES + wave;
+            if (GROUPS % NUM_WAVES == 0 || q < GROUPS)
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, YAN_LDS_PTR(lds_tile + q * 8 * kRowBytes), kChunk,
+                                                         lane_voff, k_byte0 + j * pass_pitch, 0, 0);
+        }
+    }
+};
+
+// Byte offset, relative to the first row of an R-row atom that starts at a multiple of 16 tile rows, of logical
+// chunk `chunk` of the row this lane owns.
+template <int R>
+__device__ __forceinline__ int frag_offset(int lane, int chunk) {
+    const int i = lane % R;
+    return i * kRowBytes + ((chunk ^ swizzle_of_row(i)) * kChunk);
+}
+
+// fp32 -> bf16 / f16, round to nearest even, four at a time.
+__device__ __forceinline__ bf16x4 pack4(f32x4 v, __bf16) { return __builtin_convertvector(v, bf16x4); }
+__device__ __forceinline__ f16x4  pack4(f32x4 v, _Float16) { return __builtin_convertvector(v, f16x4); }
+
+} // namespace yan

@@ -1,0 +1,4 @@
+from .bf16_gemm import gemm_bf16_tn, gemm_fp16_tn, accuracy_test as bf16_gemm_accuracy_test
+from .gemm import gemm_fp8_fp8_bf16_nt
+from .utils import ceil_div, set_num_sms, get_num_sms, get_col_major_tensor, get_m_alignment_for_contiguous_layout
+from .tuner import jit_tuner

@@ -1,0 +1,77 @@
+"""Dense 16-bit GEMM entry points: `c[m,n] = a[m,k] @ b[n,k]^T`, written in place, returns None.
+
+Same contract as the reference's `gemm_fp16_tn` (`yan/jit_kernels/cute_gemm.py:21-64`): `a` is `[m,k]`, `b` is
+`[n,k]`, `c` is `[m,n]`, all row-major on the current device; the call is asynchronous on the current stream;
+`m == 0` or `n == 0` returns at once. The reference only has the fp16 flavour and accumulates in fp16; here both
+bf16 and fp16 exist and both accumulate in fp32. Keys and argument order of the JIT kernel are the reference's:
+keys `BLOCK_M, BLOCK_N, NUM_STAGES`, args `(m, n, k, A, B, C, stream)`.
+"""
+import torch
+
+from .heuristics import get_best_dense_config
+from .tuner import jit_tuner
+from .utils import get_num_sms
+
+includes = ('"gemm/bf16_gemm.hpp"', )
+template = """
+// Templated args from Python JIT call
+constexpr auto BLOCK_M = {BLOCK_M};
+constexpr auto BLOCK_N = {BLOCK_N};
+constexpr auto kNumStages = {NUM_STAGES};
+
+__return_code = static_cast<int>(gemm_tn<BLOCK_M, BLOCK_N, kNumStages>(m, n, k, A, B, C, stream));
+"""
+
+
+def _arg_defs(dtype: torch.dtype):
+    return (('m', int), ('n', int), ('k', int), ('A', dtype), ('B', dtype), ('C', dtype), ('stream', torch.cuda.Stream))
+
+
+def dense_kernel_plan(m: int, n: int, k: int, dtype: torch.dtype, num_cus: int):
+    """(name, keys, arg_defs) of the JIT kernel a call with these sizes uses; needs no GPU."""
+    block_m, block_n = get_best_dense_config(m, n, k, num_cus)
+    name = 'gemm_bf16_tn' if dtype == torch.bfloat16 else 'gemm_fp16_tn'
+    return name, {'BLOCK_M': block_m, 'BLOCK_N': block_n, 'NUM_STAGES': 2}, _arg_defs(dtype)
+
+
+def _gemm_16bit_tn(a: torch.Tensor, b: torch.Tensor, c: torch.Tensor, dtype: torch.dtype) -> None:
+    m, k = a.shape
+    n, k_ = b.shape
+    m_, n_ = c.shape
+    assert m == m_ and n == n_ and k == k_
+    assert a.dtype == dtype and b.dtype == dtype and c.dtype == dtype
+    assert a.is_contiguous() and b.is_contiguous() and c.is_contiguous()
+    assert n % 4 == 0 and k % 8 == 0, 'n must be a multiple of 4 and k a multiple of 8'
+    if m == 0 or n == 0:
+        return
+
+    stream = torch.cuda.current_stream()
+    args = (m, n, k, a, b, c, stream)
+    name, keys, arg_defs = dense_kernel_plan(m, n, k, dtype, get_num_sms())
+    runtime = jit_tuner.compile_and_tune(name=name, keys=keys, space=(), includes=includes,
+                                         arg_defs=arg_defs, template=template, args=args)
+    rc = runtime(*args)
+    assert rc == 0, f'{name} failed with HIP error {rc}'
+
+
+def gemm_bf16_tn(a: torch.Tensor, b: torch.Tensor, c: torch.Tensor) -> None:
+    _gemm_16bit_tn(a, b, c, torch.bfloat16)
+
+
+def gemm_fp16_tn(a: torch.Tensor, b: torch.Tensor, c: torch.Tensor) -> None:
+    _gemm_16bit_tn(a, b, c, torch.half)
+
+
+def accuracy_test():
+    """The reference's smoke check (`cute_gemm.py:67-86`): seed 42, 4096 x 7168 x 2048, against `a @ b.t()`."""
+    from ..utils import calc_diff
+    torch.manual_seed(42)
+    m, n, k = 4096, 7168, 2048
+    for dtype, fn in ((torch.bfloat16, gemm_bf16_tn), (torch.half, gemm_fp16_tn)):
+        a = torch.randn(m, k, dtype=dtype, device='cuda')
+        b = torch.randn(n, k, dtype=dtype, device='cuda')
+        c = torch.zeros(m, n, dtype=dtype, device='cuda')
+        fn(a, b, c)
+        diff = calc_diff(c, a.float() @ b.float().t())
+        print(f'{fn.__name__}: calc_diff = {diff:.3e}')
+        assert diff < 1e-5

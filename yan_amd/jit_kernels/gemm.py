@@ -1,0 +1,90 @@
+"""FP8 e4m3 block-scaled GEMM, DeepGEMM convention: per-token 1x128 activation scales, 128x128 weight scales.
+
+The reference ships only the JIT template of this op (`yan/jit_kernels/gemm.py:8-31`: keys `N, K, BLOCK_M,
+BLOCK_N, NUM_STAGES, NUM_TMA_MULTICAST`; run-time names `lhs, lhs_scales, rhs, rhs_scales, out, m, stream,
+num_sms, smem_size`) and no Python entry. The template below keeps those keys and names; TMA descriptors have no
+gfx950 counterpart, so the operands go to `Gemm::run` as plain pointers and the strides of the activation scales
+are passed explicitly, which lets the kernel read them row-major or token-contiguous without a transposing copy.
+
+    out[i, j] = bf16( sum_kb lhs_scales[i, kb] * rhs_scales[j // 128, kb]
+                              * sum_{t < 128} f32(lhs[i, 128 kb + t]) * f32(rhs[j, 128 kb + t]) )
+"""
+from typing import Tuple
+
+import torch
+
+from .heuristics import get_best_fp8_config
+from .tuner import jit_tuner
+from .utils import get_num_sms, ceil_div, get_col_major_tensor
+
+# C++ code templates
+includes = ('"gemm/fp8_gemm.hpp"', )
+template = """
+using namespace yan;
+
+// Templated args from Python JIT call
+constexpr auto N = {N}, K = {K};
+constexpr auto BLOCK_M = {BLOCK_M};
+constexpr auto BLOCK_N = {BLOCK_N};
+constexpr auto kNumStages = {NUM_STAGES};
+constexpr auto kNumTMAMulticast = {NUM_TMA_MULTICAST};
+
+// Make a templated GEMM
+using GemmType = Gemm<N, K, BLOCK_M, BLOCK_N, 128, 1, kNumStages, kNumTMAMulticast, GemmType::Normal>;
+
+// Launch kernel
+__return_code = static_cast<int>(GemmType::run(out, lhs, lhs_scales, lhs_scales_stride_m, lhs_scales_stride_k,
+                                               rhs, rhs_scales, m, stream, num_sms, smem_size));
+"""
+
+arg_defs = (('lhs', torch.float8_e4m3fn), ('lhs_scales', torch.float),
+            ('rhs', torch.float8_e4m3fn), ('rhs_scales', torch.float),
+            ('out', torch.bfloat16), ('m', int),
+            ('stream', torch.cuda.Stream), ('num_sms', int), ('smem_size', int),
+            ('lhs_scales_stride_m', int), ('lhs_scales_stride_k', int))
+
+
+def fp8_kernel_plan(m: int, n: int, k: int, num_cus: int):
+    """(name, keys, arg_defs, smem_size) of the JIT kernel a call with these sizes uses; needs no GPU."""
+    block_m, block_n = get_best_fp8_config(m, n, k, num_cus)
+    keys = {'N': n, 'K': k, 'BLOCK_M': block_m, 'BLOCK_N': block_n, 'NUM_STAGES': 2, 'NUM_TMA_MULTICAST': 1}
+    smem_size = 2 * (block_m + block_n) * 128
+    return 'gemm_fp8_fp8_bf16_nt', keys, arg_defs, smem_size
+
+
+def gemm_fp8_fp8_bf16_nt(lhs: Tuple[torch.Tensor, torch.Tensor],
+                         rhs: Tuple[torch.Tensor, torch.Tensor],
+                         out: torch.Tensor) -> None:
+    """
+    lhs: (e4m3fn `[m, k]` row-major, fp32 scales `[m, ceil(k/128)]` in any strided layout)
+    rhs: (e4m3fn `[n, k]` row-major, fp32 scales `[ceil(n/128), ceil(k/128)]` row-major)
+    out: bf16 `[m, n]` row-major, written in place; the call is asynchronous on the current stream.
+    Requires k % 128 == 0 and n % 4 == 0; m is arbitrary.
+    """
+    lhs, lhs_scales = lhs
+    rhs, rhs_scales = rhs
+    m, k = lhs.shape
+    n, k_ = rhs.shape
+    m_, n_ = out.shape
+
+    assert n % 4 == 0 and k % 128 == 0
+    assert m == m_ and n == n_ and k == k_
+    assert lhs_scales.shape == (m, ceil_div(k, 128))
+    assert rhs_scales.shape == (ceil_div(n, 128), ceil_div(k, 128))
+    assert lhs.dtype == torch.float8_e4m3fn and lhs_scales.dtype == torch.float32
+    assert rhs.dtype == torch.float8_e4m3fn and rhs_scales.dtype == torch.float32
+    assert out.dtype == torch.bfloat16
+    assert lhs.is_contiguous() and rhs.is_contiguous() and out.is_contiguous() and rhs_scales.is_contiguous()
+
+    # Do nothing if `m` is zero
+    if m == 0:
+        return
+
+    num_sms = get_num_sms()
+    name, keys, defs, smem_size = fp8_kernel_plan(m, n, k, num_sms)
+    args = (lhs, lhs_scales, rhs, rhs_scales, out, m, torch.cuda.current_stream(), num_sms, smem_size,
+            lhs_scales.stride(0), lhs_scales.stride(1))
+    runtime = jit_tuner.compile_and_tune(name=name, keys=keys, space=(), includes=includes,
+                                         arg_defs=defs, template=template, args=args)
+    rc = runtime(*args)
+    assert rc == 0, f'{name} failed with HIP error {rc}'

@@ -1,0 +1,34 @@
+"""Macro-tile selection for a 256-CU part.
+
+The reference leaves this open: its dense entry hard-codes one tile and an empty tuning space
+(`yan/jit_kernels/cute_gemm.py:39-53`) and its FP8 template takes BLOCK_M / BLOCK_N as keys without saying who
+picks them (`yan/jit_kernels/gemm.py:13-16`). Here a small cost model ranks the tiles the kernels support:
+one workgroup per tile, one workgroup per CU at a time, so a launch costs
+`ceil(tiles / num_cus)` rounds of one tile time, and a tile's time grows with its MFMA work but shrinks per
+flop as the tile gets larger (fewer operand bytes fetched per flop).
+"""
+from typing import List, Tuple
+
+from .utils import ceil_div
+
+# (BLOCK_M, BLOCK_N): relative time per unit of tile area. Bigger tiles reuse operands better.
+_DENSE_TILES = {(256, 256): 1.00, (256, 128): 1.12, (128, 256): 1.12, (128, 128): 1.30, (64, 128): 1.7, (64, 64): 2.4}
+_FP8_TILES = {(256, 256): 1.00, (256, 128): 1.12, (128, 256): 1.12, (128, 128): 1.30, (64, 128): 1.7, (64, 64): 2.2,
+              (64, 32): 3.0, (64, 16): 4.5}
+
+
+def rank_tiles(m: int, n: int, num_cus: int, table) -> List[Tuple[float, Tuple[int, int]]]:
+    ranked = []
+    for (bm, bn), per_area in table.items():
+        tiles = ceil_div(m, bm) * ceil_div(n, bn)
+        rounds = ceil_div(tiles, num_cus)
+        ranked.append((rounds * bm * bn * per_area, (bm, bn)))
+    return sorted(ranked)
+
+
+def get_best_dense_config(m: int, n: int, k: int, num_cus: int) -> Tuple[int, int]:
+    return rank_tiles(m, n, num_cus, _DENSE_TILES)[0][1]
+
+
+def get_best_fp8_config(m: int, n: int, k: int, num_cus: int) -> Tuple[int, int]:
+    return rank_tiles(m, n, num_cus, _FP8_TILES)[0][1]

@@ -1,0 +1,132 @@
+"""Harness-side helpers shared by tests, the smoke entry and the benchmark: FP8 quantisers in the DeepGEMM
+convention and seeded constructors for the benchmark configurations. The reference defines neither (its FP8 path
+has no Python entry or test); the recipes are the ones the benchmark configurations name:
+per-token 1x128 / per-block 128x128 amax, clamp 1e-4, x * 448 / amax -> e4m3fn, scale = amax / 448.
+"""
+from typing import Tuple
+
+import torch
+
+FP8_MAX = 448.0
+
+
+def per_token_cast_to_fp8(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """x [m, k] (k % 128 == 0) -> (e4m3fn [m, k], fp32 scales [m, k/128])."""
+    assert x.dim() == 2 and x.size(1) % 128 == 0
+    m, k = x.shape
+    xv = x.float().view(m, k // 128, 128)
+    amax = xv.abs().amax(dim=2).clamp(1e-4)
+    q = (xv * (FP8_MAX / amax).unsqueeze(2)).to(torch.float8_e4m3fn)
+    return q.view(m, k), amax / FP8_MAX
+
+
+def per_block_cast_to_fp8(w: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """w [n, k] (k % 128 == 0) -> (e4m3fn [n, k], fp32 scales [ceil(n/128), k/128])."""
+    assert w.dim() == 2 and w.size(1) % 128 == 0
+    n, k = w.shape
+    n_pad = (n + 127) // 128 * 128
+    wp = torch.zeros((n_pad, k), dtype=torch.float32, device=w.device)
+    wp[:n] = w
+    wv = wp.view(n_pad // 128, 128, k // 128, 128)
+    amax = wv.abs().amax(dim=(1, 3)).clamp(1e-4)
+    q = (wv * (FP8_MAX / amax)[:, None, :, None]).to(torch.float8_e4m3fn)
+    return q.view(n_pad, k)[:n].contiguous(), amax / FP8_MAX
+
+
+def dequant_lhs(q: torch.Tensor, scales: torch.Tensor) -> torch.Tensor:
+    return q.float() * scales.repeat_interleave(128, dim=1)
+
+
+def dequant_rhs(q: torch.Tensor, scales: torch.Tensor) -> torch.Tensor:
+    n = q.size(0)
+    return q.float() * scales.repeat_interleave(128, dim=0)[:n].repeat_interleave(128, dim=1)
+
+
+def _source(rows: int, cols: int, dist: str, gen: torch.Generator, device) -> torch.Tensor:
+    if dist == 'normal':
+        return torch.randn(rows, cols, generator=gen, device=device)
+    if dist == 'outlier':     # uniform[-4, 4] with 1% of the entries multiplied by 50
+        x = torch.rand(rows, cols, generator=gen, device=device) * 8 - 4
+        hot = torch.rand(rows, cols, generator=gen, device=device) < 0.01
+        return torch.where(hot, x * 50, x)
+    raise ValueError(dist)
+
+
+def make_bf16_case(m: int, n: int, k: int, seed: int = 42, scale: float = 1.0, dtype=torch.bfloat16,
+                   device='cpu', gen_device='cpu'):
+    """A [m,k], B [n,k] ~ N(0,1)*scale in `dtype`, plus a zeroed C [m,n]. Values are drawn on `gen_device`
+    (CPU by default so that host and GPU paths see the same bits) and moved to `device`."""
+    gen = torch.Generator(device=gen_device).manual_seed(seed)
+    a = (torch.randn(m, k, generator=gen, device=gen_device) * scale).to(dtype).to(device)
+    b = (torch.randn(n, k, generator=gen, device=gen_device) * scale).to(dtype).to(device)
+    return a, b, torch.zeros(m, n, dtype=dtype, device=device)
+
+
+def make_fp8_case(m: int, n: int, k: int, seed: int = 42, dist: str = 'normal', device='cpu', gen_device='cpu',
+                  col_major_scales: bool = False):
+    """((A8, sA), (B8, sB), out) for the block-scaled GEMM, quantised from seeded fp32 sources.
+    Sources are drawn and quantised in row slabs so that the 16384^3 case never holds two fp32 matrices."""
+    gen = torch.Generator(device=gen_device).manual_seed(seed)
+
+    def build(rows, quantise, align):
+        qs, ss = [], []
+        step = max(align, (1 << 26) // k // align * align)
+        for r0 in range(0, rows, step):
+            r = min(step, rows - r0)
+            q, s = quantise(_source(r, k, dist, gen, gen_device).to(device))
+            qs.append(q), ss.append(s)
+        return torch.cat(qs), torch.cat(ss)
+
+    a8, sa = build(m, per_token_cast_to_fp8, 1)
+    b8, sb = build(n, per_block_cast_to_fp8, 128)
+    if col_major_scales:
+        from .jit_kernels.utils import get_col_major_tensor
+        sa = get_col_major_tensor(sa)
+    return (a8, sa), (b8, sb), torch.zeros(m, n, dtype=torch.bfloat16, device=device)
+
+
+# ----------------------------------------------------------------------------- shapes exercised on the GPU
+# (m, n, k). Listed here so that every JIT kernel they need can be compiled ahead of time, without a GPU.
+BASELINE_BF16 = {'cfg1': (1024, 1024, 1024), 'cfg2': (8192, 8192, 8192)}
+BASELINE_FP8 = {'cfg3': (4096, 7168, 7168), 'cfg4': (64, 4096, 7168), 'cfg5': (16384, 16384, 16384)}
+
+DENSE_TEST_SHAPES = [
+    (1024, 1024, 1024), (8192, 8192, 8192),
+    (128, 256, 256), (64, 64, 64), (1, 64, 64), (255, 132, 72), (300, 520, 8), (33, 4, 200), (257, 1028, 1096),
+    (256, 5120, 5120), (4096, 2048, 7168), (4096, 7168, 2048), (256, 24576, 1536),
+]
+FP8_TEST_SHAPES = [
+    (4096, 7168, 7168), (64, 4096, 7168), (16384, 16384, 16384),
+    (64, 256, 384), (512, 1024, 1024), (1, 128, 128), (63, 192, 256), (129, 320, 128), (300, 96, 640), 
+    (257, 2112, 1024), (128, 7168, 2048), (4096, 2048, 7168),
+]
+
+
+def prebuild_jit_kernels(num_cus: int = 256, verbose: bool = False) -> int:
+    """Compile every JIT kernel the shapes above select (hipcc cross-compiles for gfx950 without a GPU) into the
+    current kernel cache. Returns the number of distinct kernels."""
+    from .jit import build, cpp_format, generate
+    from .jit_kernels import bf16_gemm, gemm
+    seen = set()
+    for m, n, k in DENSE_TEST_SHAPES:
+        for dtype in (torch.bfloat16, torch.half):
+            if m == 0 or n == 0:
+                continue
+            name, keys, arg_defs = bf16_gemm.dense_kernel_plan(m, n, k, dtype, num_cus)
+            code = generate(bf16_gemm.includes, arg_defs, cpp_format(bf16_gemm.template, keys))
+            if (name, code) not in seen:
+                seen.add((name, code))
+                rt = build(name, arg_defs, code)
+                if verbose:
+                    print(f'built {name} {keys} -> {rt.path}')
+    for m, n, k in FP8_TEST_SHAPES:
+        if m == 0:
+            continue
+        name, keys, arg_defs, _ = gemm.fp8_kernel_plan(m, n, k, num_cus)
+        code = generate(gemm.includes, arg_defs, cpp_format(gemm.template, keys))
+        if (name, code) not in seen:
+            seen.add((name, code))
+            rt = build(name, arg_defs, code)
+            if verbose:
+                print(f'built {name} {keys} -> {rt.path}')
+    return len(seen)
