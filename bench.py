@@ -1,0 +1,166 @@
+#!/usr/bin/env python3
+"""Benchmark of the GEMM hot path on one MI355X.
+
+A step is one FP8 e4m3 block-scaled GEMM at M=4096, N=7168, K=7168 (per-token 1x128 activation scales, 128x128
+weight scales, bf16 output) through the JIT entry point, inputs resident in HBM before the timed region.
+Prints ONE JSON line: whole-job TFLOPS, the roofline position of the GEMM kernel (HIP-event time of the launches
+on the stream they run on) and a torch-CPU baseline on a bounded slab of the same workload.
+`--also` adds the other baseline configurations (bf16 8192^3, the M=64 decode shape) as extra fields.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+os.environ.setdefault('YAN_CACHE_DIR', os.path.join(ROOT, '.yan_cache'))
+
+METRIC = 'TFLOPS & % of MFMA peak, fp8 block-scaled GEMM 4096x7168x7168, 1 MI355X'
+# MI355X vendor peaks (dense): the one place these constants live.
+PEAK_FP8_TFLOPS = 5000.0
+PEAK_BF16_TFLOPS = 2500.0
+PEAK_HBM_GBPS = 8000.0
+
+
+def _event_time_ms(fn, steps, warmup):
+    """Average device time of one call over `steps` back-to-back calls, from events on the current stream."""
+    import torch
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    start.record()
+    for _ in range(steps):
+        fn()
+    end.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    return start.elapsed_time(end) / steps, wall_ms / steps
+
+
+def _cpu_baseline_fp8(a8, sa, b8, sb, budget_s=12.0):
+    """The reference's CPU path for this metric: torch CPU matmul of the dequantised operands (fp32), timed on a
+    slab of rows sized for about `budget_s` seconds, scaled to the full M by the flop count."""
+    import torch
+    import oracle
+    from yan_amd import testing
+    m, k = a8.shape
+    n = b8.shape[0]
+    b_cpu, sb_cpu = b8.cpu(), sb.cpu()
+    wd = testing.dequant_rhs(b_cpu, sb_cpu)
+
+    def run(rows):
+        t0 = time.perf_counter()
+        x = testing.dequant_lhs(a8[:rows].cpu(), sa[:rows].cpu())
+        out = x @ wd.t()
+        return time.perf_counter() - t0, out
+
+    t_probe, _ = run(32)
+    t_probe, _ = run(32)
+    rows = int(min(m, max(64, 32 * budget_s / max(t_probe, 1e-4) // 64 * 64)))
+    reps = []
+    for _ in range(2):
+        t, out = run(rows)
+        reps.append(t)
+    t = min(reps)
+    # the slab is also the oracle's check of the baseline itself
+    ref = oracle.gemm_fp8_block_scaled_ref(a8[:64].view(torch.uint8).cpu().numpy(), sa[:64].cpu().numpy(),
+                                           b_cpu.view(torch.uint8).numpy(), sb_cpu.numpy())
+    assert oracle.calc_diff(out[:64].numpy(), ref) < 1e-9
+    return {'value': round(2.0 * rows * n * k / t / 1e12, 4), 'unit': 'TFLOPS', 'cores': torch.get_num_threads(),
+            'kind': 'port', 'sample': f'torch CPU fp32 matmul of dequantised operands, first {rows} of {m} rows x N={n} x K={k}, '
+                                      f'best of 2, {t:.2f} s, os.cpu_count()={os.cpu_count()}'}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument('--gpus', type=int, default=1)
+    ap.add_argument('--steps', type=int, default=200)
+    ap.add_argument('--warmup', type=int, default=20)
+    ap.add_argument('--also', action='store_true', help='also time bf16 8192^3, the decode shape and 16384^3 (extra fields)')
+    ap.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline leg')
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f'bench.py: this build runs on one GPU; --gpus {args.gpus} is not supported (every figure is a 1-GPU figure)',
+              file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    import yan_amd as yan
+    from yan_amd import testing
+    from yan_amd.jit_kernels.gemm import fp8_kernel_plan
+    assert torch.cuda.is_available(), 'bench.py needs a GPU'
+    torch.cuda.set_device(0)
+
+    m, n, k = testing.BASELINE_FP8['cfg3']
+    (a8, sa), (b8, sb), out = testing.make_fp8_case(m, n, k, seed=42, device='cuda', gen_device='cuda')
+    sa = yan.get_col_major_tensor(sa)      # token-contiguous scales, the layout DeepGEMM-style callers hand over
+    step = lambda: yan.gemm_fp8_fp8_bf16_nt((a8, sa), (b8, sb), out)
+
+    # validity of what is being timed: sampled rows against an fp32 matmul of the dequantised operands
+    step()
+    rows = torch.randperm(m, device='cuda')[:256]
+    ref = testing.dequant_lhs(a8[rows], sa[rows]) @ testing.dequant_rhs(b8, sb).t()
+    diff = float(yan.calc_diff(out[rows].float(), ref))
+    assert diff < 1e-3, f'parity lost: calc_diff={diff}'
+    del ref
+
+    kernel_ms, wall_ms = _event_time_ms(step, args.steps, args.warmup)
+    flops = 2.0 * m * n * k
+    tflops_job = flops / (wall_ms * 1e-3) / 1e12
+    tflops_kernel = flops / (kernel_ms * 1e-3) / 1e12
+    bytes_alg = m * k + n * k + 4 * m * (k // 128) + 4 * ((n + 127) // 128) * (k // 128) + 2 * m * n
+    _, keys, _, _ = fp8_kernel_plan(m, n, k, yan.get_num_sms())
+
+    line = {
+        'metric': METRIC, 'value': round(tflops_job, 1), 'unit': 'TFLOPS', 'n_gpus': 1,
+        'steps': args.steps, 'warmup': args.warmup, 'ms_per_step': round(wall_ms, 5),
+        'higher_is_better': True, 'scaling': 'weak', 'vs_baseline': None, 'dtype': 'fp8_e4m3 (fp32 accumulate, bf16 out)',
+        'data': 'synthetic: N(0,1) sources, seed 42, quantised per-token 1x128 / per-block 128x128',
+        'config': {'workload': 'configs[2]: FP8 e4m3 block-scaled GEMM M=4096 N=7168 K=7168, bf16 out',
+                   'tile': f"{keys['BLOCK_M']}x{keys['BLOCK_N']}x128", 'cache_state': 'warm (same operands every step)',
+                   'calc_diff_sampled_rows': diff},
+        'roofline': {'bound': 'mfma', 'achieved': round(tflops_kernel, 1), 'peak': PEAK_FP8_TFLOPS, 'unit': 'TFLOP/s',
+                     'frac': round(tflops_kernel / PEAK_FP8_TFLOPS, 4), 'traffic': None,
+                     'kernel': 'fp8_gemm_kernel', 'kernel_us': round(kernel_ms * 1e3, 2),
+                     'algorithmic_flop_per_launch': flops, 'algorithmic_bytes_per_launch': bytes_alg},
+    }
+
+    if args.also:
+        extra = {}
+        mm, nn, kk = testing.BASELINE_BF16['cfg2']
+        a, b, c = testing.make_bf16_case(mm, nn, kk, seed=42, scale=kk ** -0.5, device='cuda', gen_device='cuda')
+        ms, _ = _event_time_ms(lambda: yan.gemm_bf16_tn(a, b, c), 50, 10)
+        extra['bf16_8192'] = {'us': round(ms * 1e3, 1), 'tflops': round(2.0 * mm * nn * kk / ms / 1e9, 1),
+                              'frac_of_bf16_peak': round(2.0 * mm * nn * kk / ms / 1e9 / PEAK_BF16_TFLOPS, 4)}
+        ms, _ = _event_time_ms(lambda: torch.matmul(a, b.t(), out=c), 50, 10)
+        extra['bf16_8192_torch_hipblaslt'] = {'us': round(ms * 1e3, 1), 'tflops': round(2.0 * mm * nn * kk / ms / 1e9, 1)}
+        del a, b, c
+        mm, nn, kk = testing.BASELINE_FP8['cfg4']
+        (x8, sx), (w8, sw), o = testing.make_fp8_case(mm, nn, kk, seed=42, device='cuda')
+        sx = yan.get_col_major_tensor(sx)
+        ms, wall = _event_time_ms(lambda: yan.gemm_fp8_fp8_bf16_nt((x8, sx), (w8, sw), o), 200, 20)
+        byt = mm * kk + nn * kk + 4 * mm * (kk // 128) + 4 * (nn // 128) * (kk // 128) + 2 * mm * nn
+        extra['fp8_decode_64x4096x7168'] = {'us': round(ms * 1e3, 2), 'wall_us': round(wall * 1e3, 2), 'gb_per_s': round(byt / ms / 1e6, 1),
+                                            'frac_of_hbm_peak': round(byt / ms / 1e6 / PEAK_HBM_GBPS, 4)}
+        mm, nn, kk = testing.BASELINE_FP8['cfg5']
+        (x8, sx), (w8, sw), o = testing.make_fp8_case(mm, nn, kk, seed=42, dist='outlier', device='cuda', gen_device='cuda')
+        sx = yan.get_col_major_tensor(sx)
+        ms, _ = _event_time_ms(lambda: yan.gemm_fp8_fp8_bf16_nt((x8, sx), (w8, sw), o), 10, 2)
+        extra['fp8_16384_outliers'] = {'us': round(ms * 1e3, 1), 'tflops': round(2.0 * mm * nn * kk / ms / 1e9, 1),
+                                       'frac_of_fp8_peak': round(2.0 * mm * nn * kk / ms / 1e9 / PEAK_FP8_TFLOPS, 4)}
+        del x8, sx, w8, sw, o
+        line['extra'] = extra
+
+    if not args.no_cpu:
+        line['cpu_baseline'] = _cpu_baseline_fp8(a8, sa, b8, sb)
+    else:
+        line['cpu_baseline'] = None
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == '__main__':
+    main()

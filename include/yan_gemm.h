@@ -1,0 +1,78 @@
+/* C ABI of the MI355X (gfx950) GEMM hot path: bf16 / fp16 dense GEMM and FP8 e4m3 block-scaled GEMM.
+ *
+ * Two ways in, both plain C with raw device pointers and sizes:
+ *
+ * 1. The ahead-of-time library libyan_gemm.so (yan_amd/csrc), declared below: every tile variant precompiled,
+ *    sizes taken at run time. This is what a host that is not Python (or does not want a compiler at run time)
+ *    binds.
+ * 2. A JIT-built kernel.so, which exports exactly one symbol,
+ *        void launch(<one parameter per argument>, int* __return_code);
+ *    with tensors and streams passed as void* and bool/int/float by value. This is the boundary of the reference
+ *    (yan/jit/template.py:121-149 generates it, yan/jit/runtime.py:54-68 calls it through ctypes). The two
+ *    instantiations this path uses are spelled out as function-pointer types at the end of this header.
+ *
+ * Conventions shared by every entry point:
+ *   - all matrices are row-major with the K dimension contiguous ("TN"/"NT": both operands K-major);
+ *   - pointers are device pointers owned by the caller; nothing is allocated, freed or retained;
+ *   - work is enqueued on `stream` (a hipStream_t, NULL for the default stream) and NOT synchronised;
+ *   - the return value is a hipError_t as int: 0 on success, hipErrorInvalidValue (1) for sizes the kernels do
+ *     not take (they never fault on a bad size), or whatever the launch reported;
+ *   - m == 0 or n == 0 is a successful no-op.
+ */
+#ifndef YAN_GEMM_H
+#define YAN_GEMM_H
+
+#if defined(__GNUC__)
+#define YAN_API __attribute__((visibility("default")))
+#else
+#define YAN_API
+#endif
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* c[m,n] = a[m,k] . b[n,k]^T, bf16 in, fp32 accumulate, bf16 out (round to nearest even).
+ * Requires n % 4 == 0, k % 8 == 0, and (m rounded up to 256) * k * 2 < 2^31 bytes, same for n.
+ * Replaces gemm_fp16_tn -> gemm_tn<128,128,3> of the reference (yan/jit_kernels/cute_gemm.py:21-64,
+ * yan/include/gemm/cute_gemm.cuh:262-378), with the bf16 dtype and fp32 accumulation. */
+YAN_API int yan_gemm_bf16_tn(int m, int n, int k, const void* a, const void* b, void* c, void* stream);
+
+/* Same contraction for IEEE fp16 in / fp16 out, fp32 accumulate (the reference's dtype, cute_gemm.py:26). */
+YAN_API int yan_gemm_fp16_tn(int m, int n, int k, const void* a, const void* b, void* c, void* stream);
+
+/* out[i,j] = bf16( sum_kb lhs_scales(i,kb) * rhs_scales[j/128][kb] * sum_{t<128} lhs[i][128kb+t] * rhs[j][128kb+t] )
+ *   lhs        e4m3 (OCP, max 448) [m,k] row-major
+ *   lhs_scales fp32, element (i,kb) at lhs_scales[i*lhs_scales_stride_m + kb*lhs_scales_stride_k]
+ *              (row-major: strides (k/128, 1); token-contiguous as DeepGEMM callers pass it: (1, m))
+ *   rhs        e4m3 [n,k] row-major;  rhs_scales fp32 [ceil(n/128)][k/128] row-major
+ *   out        bf16 [m,n] row-major
+ * Requires k % 128 == 0, n % 4 == 0; m arbitrary. `num_sms` is the caller's compute-unit cap (the reference passes
+ * it to its persistent kernel, yan/jit_kernels/gemm.py:26-30); this build launches one workgroup per tile and
+ * accepts the argument for signature compatibility.
+ * Replaces the FP8 entry the reference only sketches: template yan/jit_kernels/gemm.py:9-31, kernel
+ * yan/include/gemm/fp8_gemm.cuh:40-196. */
+YAN_API int yan_gemm_fp8_fp8_bf16_nt(const void* lhs, const float* lhs_scales, long long lhs_scales_stride_m,
+                             long long lhs_scales_stride_k, const void* rhs, const float* rhs_scales, void* out,
+                             int m, int n, int k, void* stream, int num_sms);
+
+/* Macro tile the library uses for a problem: op 0 = dense 16-bit, 1 = FP8 block-scaled. Writes BLOCK_M / BLOCK_N.
+ * Host-only (no device call). Stands where the reference leaves tile choice to the caller's keys
+ * (yan/jit_kernels/cute_gemm.py:41, yan/jit_kernels/gemm.py:13-16). Returns 0, or 1 for an unknown op. */
+YAN_API int yan_gemm_select_tile(int op, int m, int n, int k, int num_cus, int* block_m, int* block_n);
+
+/* "yan-gemm gfx950 <n> dense + <n> fp8 tile variants". */
+YAN_API const char* yan_gemm_version(void);
+
+/* The JIT boundary, for reference: signatures of `launch` in the kernel.so of each op
+ * (argument lists of yan/jit_kernels/cute_gemm.py:55-59 and yan/jit_kernels/gemm.py:23-30; the last two ints of
+ * the FP8 form are this build's explicit activation-scale strides, in elements). */
+typedef void (*yan_jit_launch_dense_fn)(int m, int n, int k, void* A, void* B, void* C, void* stream, int* return_code);
+typedef void (*yan_jit_launch_fp8_fn)(void* lhs, void* lhs_scales, void* rhs, void* rhs_scales, void* out, int m,
+                                      void* stream, int num_sms, int smem_size, int lhs_scales_stride_m,
+                                      int lhs_scales_stride_k, int* return_code);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* YAN_GEMM_H */

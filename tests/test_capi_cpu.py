@@ -1,0 +1,65 @@
+"""The ahead-of-time C-ABI library without a GPU: it loads, exports exactly what include/yan_gemm.h declares, its
+host-only entry points work, and its compute entry points reject bad sizes before any device call."""
+import ctypes
+import os
+import re
+import subprocess
+
+import pytest
+
+from yan_amd import capi
+from yan_amd.jit_kernels import heuristics
+
+
+@pytest.fixture(scope='module')
+def lib():
+    return capi.load()
+
+
+def _declared(repo_root):
+    text = open(os.path.join(repo_root, 'include', 'yan_gemm.h')).read()
+    return sorted(re.findall(r'^YAN_API\s+[\w\s\*]+?\b(yan_\w+)\s*\(', text, flags=re.M))
+
+
+def test_library_exports_every_declared_symbol(lib, repo_root):
+    declared = _declared(repo_root)
+    assert declared == sorted(capi.SYMBOLS) and len(declared) == 5
+    for name in declared:
+        assert hasattr(lib, name), name
+    out = subprocess.check_output(['nm', '-D', '--defined-only', os.path.join(repo_root, 'yan_amd', 'csrc', 'libyan_gemm.so')], text=True)
+    exported = sorted(ln.split()[-1] for ln in out.splitlines() if ' T ' in ln)
+    assert exported == declared          # nothing else leaks out of the library
+
+
+def test_header_is_plain_c(repo_root, tmp_path):
+    src = tmp_path / 'use.c'
+    src.write_text('#include "yan_gemm.h"\nconst char* (*probe)(void) = yan_gemm_version;\nint main(void) { yan_jit_launch_dense_fn f = 0; yan_jit_launch_fp8_fn g = 0; (void)f; (void)g; return probe ? 0 : 1; }\n')
+    subprocess.check_call(['gcc', '-std=c99', '-Wall', '-Werror', '-pedantic', '-c', str(src), '-I', os.path.join(repo_root, 'include'),
+                           '-o', str(tmp_path / 'use.o')])
+
+
+def test_version_and_tile_selection_match_python(lib):
+    assert b'gfx950' in lib.yan_gemm_version()
+    shapes = [(4096, 7168, 7168), (64, 4096, 7168), (16384, 16384, 16384), (8192, 8192, 8192), (1024, 1024, 1024),
+              (1, 128, 128), (300, 96, 640), (257, 2112, 1024), (256, 24576, 1536), (4096, 2048, 7168), (129, 320, 128)]
+    for m, n, k in shapes:
+        for cus in (256, 128, 80):
+            assert capi.select_tile(0, m, n, k, cus) == heuristics.get_best_dense_config(m, n, k, cus), (m, n, k, cus)
+            assert capi.select_tile(1, m, n, k, cus) == heuristics.get_best_fp8_config(m, n, k, cus), (m, n, k, cus)
+    bm, bn = ctypes.c_int(), ctypes.c_int()
+    assert lib.yan_gemm_select_tile(7, 1, 1, 1, 256, ctypes.byref(bm), ctypes.byref(bn)) == 1
+    assert lib.yan_gemm_select_tile(0, 1, 1, 1, 0, ctypes.byref(bm), ctypes.byref(bn)) == 1
+
+
+def test_compute_entry_points_validate_before_touching_a_device(lib):
+    null = ctypes.c_void_p(0)
+    assert lib.yan_gemm_bf16_tn(0, 64, 64, null, null, null, null) == 0          # empty problem: no-op
+    assert lib.yan_gemm_fp16_tn(64, 0, 64, null, null, null, null) == 0
+    assert lib.yan_gemm_bf16_tn(-1, 64, 64, null, null, null, null) != 0
+    assert lib.yan_gemm_bf16_tn(64, 62, 64, null, null, null, null) != 0         # n % 4
+    assert lib.yan_gemm_bf16_tn(64, 64, 60, null, null, null, null) != 0         # k % 8
+    assert lib.yan_gemm_bf16_tn(64, 64, 64, null, null, null, null) != 0         # null operands
+    assert lib.yan_gemm_fp8_fp8_bf16_nt(null, null, 1, 1, null, null, null, 0, 128, 128, null, 256) == 0
+    assert lib.yan_gemm_fp8_fp8_bf16_nt(null, null, 1, 1, null, null, null, 4, 128, 64, null, 256) != 0    # k % 128
+    assert lib.yan_gemm_fp8_fp8_bf16_nt(null, null, 1, 1, null, null, null, 4, 126, 128, null, 256) != 0   # n % 4
+    assert lib.yan_gemm_fp8_fp8_bf16_nt(null, null, 1, 1, null, null, null, 4, 128, 128, null, 256) != 0   # null operands

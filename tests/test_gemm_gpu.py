@@ -1,0 +1,302 @@
+"""Parity of the HIP GEMMs against the CPU oracle, through the JIT boundary (`launch` in a cached kernel.so).
+
+bf16 / fp16: calc_diff < 1e-5 against the fp32 matmul of the same 16-bit inputs.
+FP8:         calc_diff < 1e-3 against the fp32 matmul of the dequantised operands; exactly representable cases
+             must match bit for bit.
+Sizes the oracle finishes in seconds are compared in full; the baseline sizes are checked on a seeded sample of
+rows against the oracle, in full against a chunked fp32 matmul on the device, and through size-independent
+properties (exact linearity in power-of-two scales, layout independence of the scale tensor).
+"""
+import os
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+import yan_amd as yan
+from yan_amd import jit, testing
+
+pytestmark = pytest.mark.gpu
+
+BF16_TOL, FP8_TOL = 1e-5, 1e-3
+
+
+def _announce(*what):
+    print('[case]', *what, flush=True)
+    sys.stdout.flush()
+
+
+def _np(t):
+    if t.dtype == torch.float8_e4m3fn:
+        return t.view(torch.uint8).cpu().numpy()
+    return t.float().cpu().numpy()
+
+
+@pytest.fixture(scope='module', autouse=True)
+def _device():
+    assert torch.cuda.is_available(), 'these tests need a GPU'
+    torch.cuda.set_device(0)
+    yield
+    torch.cuda.synchronize()
+
+
+# ----------------------------------------------------------------------------- the boundary itself
+def test_jit_boundary_known_answer(capfd):
+    """tests/test_jit.py:31-64 of the reference: the six arguments arrive in `launch` as passed."""
+    args = (('lhs', torch.float8_e4m3fn), ('rhs', torch.float8_e4m3fn), ('scale', torch.float), ('out', torch.bfloat16),
+            ('enable_double_streams', bool), ('stream', torch.cuda.Stream))
+    body = '\n' + ''.join(f'std::cout << reinterpret_cast<uint64_t>({n}) << std::endl;\n' for n in ('lhs', 'rhs', 'scale', 'out'))
+    body += 'std::cout << enable_double_streams << std::endl;\nstd::cout << reinterpret_cast<uint64_t>(stream) << std::endl;\n'
+    func = jit.build('test_func', args, jit.generate((), args, body))
+    fp8 = torch.empty((1,), dtype=torch.float8_e4m3fn, device='cuda')
+    fp32 = torch.empty((1,), dtype=torch.float, device='cuda')
+    bf16 = torch.empty((1,), dtype=torch.bfloat16, device='cuda')
+    stream = torch.cuda.current_stream()
+    capfd.readouterr()
+    assert func(fp8, fp8, fp32, bf16, True, stream) == 0
+    out = capfd.readouterr().out
+    assert out == f'{fp8.data_ptr()}\n{fp8.data_ptr()}\n{fp32.data_ptr()}\n{bf16.data_ptr()}\n1\n{stream.cuda_stream}\n'
+
+
+def test_launch_reports_bad_sizes_through_the_return_code():
+    from yan_amd.jit_kernels import bf16_gemm
+    name, keys, defs = bf16_gemm.dense_kernel_plan(64, 64, 64, torch.bfloat16, 256)
+    rt = jit.build(name, defs, jit.generate(bf16_gemm.includes, defs, jit.cpp_format(bf16_gemm.template, keys)))
+    a = torch.zeros(64, 64, dtype=torch.bfloat16, device='cuda')
+    assert rt(64, 64, 64, a, a, a, torch.cuda.current_stream()) == 0
+    assert rt(64, 62, 64, a, a, a, torch.cuda.current_stream()) != 0        # n % 4 != 0
+    assert rt(64, 64, 60, a, a, a, torch.cuda.current_stream()) != 0        # k % 8 != 0
+    assert rt(-1, 64, 64, a, a, a, torch.cuda.current_stream()) != 0
+    torch.cuda.synchronize()
+
+
+# ----------------------------------------------------------------------------- bf16 / fp16
+@pytest.mark.parametrize('m,n,k', [s for s in testing.DENSE_TEST_SHAPES if s[0] * s[1] * s[2] <= 7e10])
+@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.half])
+def test_dense_parity_vs_oracle(m, n, k, dtype):
+    _announce('dense', dtype, m, n, k)
+    a, b, c = testing.make_bf16_case(m, n, k, seed=42, dtype=dtype, device='cuda')
+    c.fill_(float('nan'))
+    (yan.gemm_bf16_tn if dtype == torch.bfloat16 else yan.gemm_fp16_tn)(a, b, c)
+    torch.cuda.synchronize()
+    got = _np(c)
+    assert np.isfinite(got).all()
+    ref = oracle.gemm_bf16_tn_ref(_np(a), _np(b))
+    assert oracle.calc_diff(got, ref) < BF16_TOL
+    # every element within one output rounding step of the fp32 result (plus fp32 accumulation slack)
+    ulp = 2.0 ** (-7 if dtype == torch.bfloat16 else -10)
+    assert bool(np.all(np.abs(got - ref) <= np.abs(ref) * ulp + 1e-4 * np.sqrt(k)))
+
+
+def test_dense_golden_fixture(repo_root):
+    z = np.load(os.path.join(repo_root, 'tests', 'golden', 'gemm_small.npz'))
+    a = torch.from_numpy(z['bf16_a_bits'].view(np.int16)).view(torch.bfloat16).cuda()
+    b = torch.from_numpy(z['bf16_b_bits'].view(np.int16)).view(torch.bfloat16).cuda()
+    c = torch.zeros(a.size(0), b.size(0), dtype=torch.bfloat16, device='cuda')
+    yan.gemm_bf16_tn(a, b, c)
+    assert oracle.calc_diff(_np(c), z['bf16_expected_f64']) < BF16_TOL
+    # the kernel's fp32 sum, rounded once to bf16, is within one bf16 step of the correctly rounded fp64 value
+    want = oracle.bf16_round(z['bf16_expected_f64'].astype(np.float32))
+    assert np.all(np.abs(_np(c) - want) <= np.abs(want) * 2.0 ** -7 + 1e-6)
+
+
+def test_dense_closed_forms_are_exact():
+    # ones pattern of the reference's smoke case (yan/jit_kernels/cute_gemm.py:74-79): c == ceil(k / 12) everywhere
+    m, n, k = 128, 256, 256
+    a = torch.zeros(m, k, dtype=torch.bfloat16, device='cuda')
+    b = torch.zeros(n, k, dtype=torch.bfloat16, device='cuda')
+    a[:, ::4] = 1.0
+    b[:, ::3] = 1.0
+    c = torch.zeros(m, n, dtype=torch.bfloat16, device='cuda')
+    yan.gemm_bf16_tn(a, b, c)
+    assert torch.equal(c, torch.full_like(c, -(-k // 12)))
+    # identity weights return the activations bit for bit; catches transposed or permuted operands
+    g = torch.Generator().manual_seed(3)
+    a = torch.randn(300, 256, generator=g).bfloat16().cuda()
+    eye = torch.eye(256, dtype=torch.bfloat16, device='cuda')
+    c = torch.zeros(300, 256, dtype=torch.bfloat16, device='cuda')
+    yan.gemm_bf16_tn(a, eye, c)
+    assert torch.equal(c, a)
+    # untouched memory around a ragged output stays untouched
+    big = torch.full((70, 136), 7.0, dtype=torch.bfloat16, device='cuda')
+    a, b, _ = testing.make_bf16_case(33, 132, 72, seed=5, device='cuda')
+    out = big[:33 * 132 // 136 + 1].view(-1)[:33 * 132].view(33, 132)
+    yan.gemm_bf16_tn(a, b, out)
+    assert torch.all(big.view(-1)[33 * 132:] == 7.0)
+    assert oracle.calc_diff(_np(out), oracle.gemm_bf16_tn_ref(_np(a), _np(b))) < BF16_TOL
+
+
+def test_dense_baseline_8192_cubed():
+    """cfg2: rows sampled against the oracle, the whole matrix against a chunked fp32 matmul on the device."""
+    m = n = k = 8192
+    _announce('dense cfg2', m, n, k)
+    a, b, c = testing.make_bf16_case(m, n, k, seed=42, scale=k ** -0.5, device='cuda', gen_device='cuda')
+    yan.gemm_bf16_tn(a, b, c)
+    rows = np.random.default_rng(0).choice(m, 64, replace=False)
+    ref = oracle.gemm_bf16_tn_ref(_np(a[rows]), _np(b))
+    assert oracle.calc_diff(_np(c[rows]), ref) < BF16_TOL
+    num = den = 0.0
+    for r0 in range(0, m, 1024):
+        ref = a[r0:r0 + 1024].float() @ b.float().t()
+        got = c[r0:r0 + 1024].float()
+        num += (got.double() * ref.double()).sum().item()
+        den += (got.double() ** 2 + ref.double() ** 2).sum().item()
+    assert 1 - 2 * num / den < BF16_TOL
+
+
+# ----------------------------------------------------------------------------- FP8 block-scaled
+def _fp8_ref(a8, sa, b8, sb):
+    return oracle.gemm_fp8_block_scaled_ref(_np(a8), sa.cpu().numpy(), _np(b8), sb.cpu().numpy())
+
+
+@pytest.mark.parametrize('m,n,k', [s for s in testing.FP8_TEST_SHAPES if s[0] * s[1] * s[2] <= 7e10])
+@pytest.mark.parametrize('col_major', [False, True])
+def test_fp8_parity_vs_oracle(m, n, k, col_major):
+    _announce('fp8', m, n, k, 'col-major scales' if col_major else 'row-major scales')
+    (a8, sa), (b8, sb), out = testing.make_fp8_case(m, n, k, seed=42, device='cuda', col_major_scales=col_major)
+    out.fill_(float('nan'))
+    yan.gemm_fp8_fp8_bf16_nt((a8, sa), (b8, sb), out)
+    torch.cuda.synchronize()
+    got = _np(out)
+    assert np.isfinite(got).all()
+    ref = _fp8_ref(a8, sa, b8, sb)
+    assert oracle.calc_diff(got, ref) < FP8_TOL
+    # far tighter than the contract: only the bf16 output rounding and fp32 summation order separate the two
+    assert oracle.calc_diff(got, ref) < 1e-5
+    # element-wise: within one bf16 step of the fp32 value, plus the matrix core's own summation error. The fp8
+    # MFMA does not carry full fp32 precision inside a 128-deep block: measured errors reach about 2^-15 of the
+    # largest product in the block, i.e. ~1e-5 of max|out| on N(0,1) data (this is why blocks are folded in fp32).
+    assert bool(np.all(np.abs(got - ref) <= np.abs(ref) * 2.0 ** -7 + 1e-4 * np.abs(ref).max()))
+
+
+def test_fp8_golden_fixtures(repo_root):
+    z = np.load(os.path.join(repo_root, 'tests', 'golden', 'gemm_small.npz'))
+
+    def dev(codes):
+        return torch.from_numpy(codes).cuda().view(torch.float8_e4m3fn)
+
+    out = torch.zeros(64, 256, dtype=torch.bfloat16, device='cuda')
+    yan.gemm_fp8_fp8_bf16_nt((dev(z['fp8_lhs']), torch.from_numpy(z['fp8_lhs_scales']).cuda()),
+                             (dev(z['fp8_rhs']), torch.from_numpy(z['fp8_rhs_scales']).cuda()), out)
+    assert oracle.calc_diff(_np(out), z['fp8_expected_f64']) < 1e-5
+    # integer-valued operands with power-of-two scales: every partial sum is exact, so the result is too
+    out = torch.zeros(40, 192, dtype=torch.bfloat16, device='cuda')
+    yan.gemm_fp8_fp8_bf16_nt((dev(z['int_lhs']), torch.from_numpy(z['int_lhs_scales']).cuda()),
+                             (dev(z['int_rhs']), torch.from_numpy(z['int_rhs_scales']).cuda()), out)
+    assert np.array_equal(_np(out), oracle.bf16_round(z['int_expected']))
+
+
+def test_fp8_exact_cases_and_scale_indexing():
+    rng = np.random.default_rng(12)
+    m, n, k = 130, 448, 640          # ragged m, n = 3.5 scale blocks, 5 K blocks
+    va = rng.integers(-2, 3, size=(m, k)).astype(np.float32)
+    vb = rng.integers(-2, 3, size=(n, k)).astype(np.float32)
+    a8 = torch.from_numpy(oracle.e4m3fn_encode(va)).cuda().view(torch.float8_e4m3fn)
+    b8 = torch.from_numpy(oracle.e4m3fn_encode(vb)).cuda().view(torch.float8_e4m3fn)
+    sa = (2.0 ** rng.integers(-3, 4, size=(m, 5))).astype(np.float32)
+    sb = (2.0 ** rng.integers(-3, 4, size=(4, 5))).astype(np.float32)
+    out = torch.zeros(m, n, dtype=torch.bfloat16, device='cuda')
+    yan.gemm_fp8_fp8_bf16_nt((a8, torch.from_numpy(sa).cuda()), (b8, torch.from_numpy(sb).cuda()), out)
+    want = oracle.gemm_fp8_block_scaled_ref(oracle.e4m3fn_encode(va), sa, oracle.e4m3fn_encode(vb), sb)
+    assert np.array_equal(_np(out), oracle.bf16_round(want))
+    # one non-zero K block with arbitrary scales isolates sA[m, kb] and sB[n // 128, kb]
+    kb = 3
+    a0 = np.zeros_like(va)
+    a0[:, kb * 128:(kb + 1) * 128] = va[:, kb * 128:(kb + 1) * 128]
+    sa_r = (rng.random((m, 5)) + 0.5).astype(np.float32)
+    sb_r = (rng.random((4, 5)) + 0.5).astype(np.float32)
+    a08 = torch.from_numpy(oracle.e4m3fn_encode(a0)).cuda().view(torch.float8_e4m3fn)
+    yan.gemm_fp8_fp8_bf16_nt((a08, torch.from_numpy(sa_r).cuda()), (b8, torch.from_numpy(sb_r).cuda()), out)
+    part = va[:, kb * 128:(kb + 1) * 128].astype(np.float64) @ vb[:, kb * 128:(kb + 1) * 128].astype(np.float64).T
+    want = part * sa_r[:, kb].astype(np.float64)[:, None] * np.repeat(sb_r[:, kb].astype(np.float64), 128)[:n][None, :]
+    assert bool(np.all(np.abs(_np(out) - want) <= np.abs(want) * 2.0 ** -7 + 1e-6))
+
+
+def test_fp8_linearity_and_layout_independence_at_headline_size():
+    """cfg3 (4096 x 7168 x 7168): doubling every activation scale doubles the output exactly; row-major and
+    token-contiguous scale tensors give identical bits; sampled rows match the oracle; the full matrix matches a
+    chunked fp32 matmul of the dequantised operands on the device."""
+    m, n, k = testing.BASELINE_FP8['cfg3']
+    _announce('fp8 cfg3', m, n, k)
+    (a8, sa), (b8, sb), out = testing.make_fp8_case(m, n, k, seed=42, device='cuda', gen_device='cuda')
+    yan.gemm_fp8_fp8_bf16_nt((a8, sa), (b8, sb), out)
+    out2 = torch.zeros_like(out)
+    yan.gemm_fp8_fp8_bf16_nt((a8, yan.get_col_major_tensor(sa * 2)), (b8, sb), out2)
+    assert torch.equal(out2.float(), out.float() * 2)
+    rows = np.random.default_rng(1).choice(m, 48, replace=False)
+    ref = _fp8_ref(a8[rows], sa[rows], b8, sb)
+    assert oracle.calc_diff(_np(out[rows]), ref) < 1e-5
+    wd = testing.dequant_rhs(b8, sb)
+    num = den = 0.0
+    for r0 in range(0, m, 1024):
+        ref = testing.dequant_lhs(a8[r0:r0 + 1024], sa[r0:r0 + 1024]) @ wd.t()
+        got = out[r0:r0 + 1024].float()
+        num += (got.double() * ref.double()).sum().item()
+        den += (got.double() ** 2 + ref.double() ** 2).sum().item()
+    assert 1 - 2 * num / den < FP8_TOL
+
+
+def test_fp8_decode_shape():
+    m, n, k = testing.BASELINE_FP8['cfg4']
+    _announce('fp8 cfg4', m, n, k)
+    (a8, sa), (b8, sb), out = testing.make_fp8_case(m, n, k, seed=42, device='cuda')
+    yan.gemm_fp8_fp8_bf16_nt((a8, sa), (b8, sb), out)
+    assert oracle.calc_diff(_np(out), _fp8_ref(a8, sa, b8, sb)) < 1e-5
+
+
+def test_fp8_outlier_16384_cubed():
+    """cfg5: uniform[-4,4] sources with 1% of entries x50. Sampled rows against the oracle, plus finiteness."""
+    m, n, k = testing.BASELINE_FP8['cfg5']
+    _announce('fp8 cfg5', m, n, k)
+    (a8, sa), (b8, sb), out = testing.make_fp8_case(m, n, k, seed=42, dist='outlier', device='cuda', gen_device='cuda')
+    assert not torch.isnan(a8.view(torch.uint8).float()).any()
+    assert int((a8.view(torch.uint8) & 0x7F).max()) <= 0x7E and int((b8.view(torch.uint8) & 0x7F).max()) <= 0x7E
+    yan.gemm_fp8_fp8_bf16_nt((a8, sa), (b8, sb), out)
+    torch.cuda.synchronize()
+    rows = np.random.default_rng(2).choice(m, 32, replace=False)
+    ref = _fp8_ref(a8[rows], sa[rows], b8, sb)
+    got = _np(out[rows])
+    assert np.isfinite(got).all()
+    assert oracle.calc_diff(got, ref) < FP8_TOL
+    assert oracle.calc_diff(got, ref) < 1e-5
+    assert bool(torch.isfinite(out[::97].float()).all())
+
+
+# ----------------------------------------------------------------------------- the ahead-of-time C-ABI library
+@pytest.mark.parametrize('m,n,k', [(1024, 1024, 1024), (255, 132, 72), (33, 4, 200), (257, 1028, 1096)])
+def test_capi_dense_matches_oracle_and_jit(m, n, k):
+    from yan_amd import capi
+    _announce('capi dense', m, n, k)
+    for dtype, fn, jit_fn in ((torch.bfloat16, capi.gemm_bf16_tn, yan.gemm_bf16_tn), (torch.half, capi.gemm_fp16_tn, yan.gemm_fp16_tn)):
+        a, b, c = testing.make_bf16_case(m, n, k, seed=9, dtype=dtype, device='cuda')
+        assert fn(a, b, c) == 0
+        assert oracle.calc_diff(_np(c), oracle.gemm_bf16_tn_ref(_np(a), _np(b))) < BF16_TOL
+        c2 = torch.zeros_like(c)
+        jit_fn(a, b, c2)
+        assert torch.equal(c, c2)            # same kernel source, same tile choice: same bits
+
+
+@pytest.mark.parametrize('m,n,k', [(64, 256, 384), (129, 320, 128), (300, 96, 640), (257, 2112, 1024), (64, 4096, 7168)])
+def test_capi_fp8_matches_oracle_and_jit(m, n, k):
+    from yan_amd import capi
+    _announce('capi fp8', m, n, k)
+    (a8, sa), (b8, sb), out = testing.make_fp8_case(m, n, k, seed=9, device='cuda')
+    assert capi.gemm_fp8_fp8_bf16_nt((a8, sa), (b8, sb), out) == 0
+    assert oracle.calc_diff(_np(out), _fp8_ref(a8, sa, b8, sb)) < 1e-5
+    out_cm = torch.zeros_like(out)
+    assert capi.gemm_fp8_fp8_bf16_nt((a8, yan.get_col_major_tensor(sa)), (b8, sb), out_cm) == 0
+    out_jit = torch.zeros_like(out)
+    yan.gemm_fp8_fp8_bf16_nt((a8, sa), (b8, sb), out_jit)
+    assert torch.equal(out, out_cm) and torch.equal(out, out_jit)
+
+
+def test_capi_rejects_bad_sizes_on_device():
+    from yan_amd import capi
+    a = torch.zeros(64, 64, dtype=torch.bfloat16, device='cuda')
+    lib = capi.load()
+    null = None
+    assert lib.yan_gemm_bf16_tn(64, 62, 64, a.data_ptr(), a.data_ptr(), a.data_ptr(), null) != 0
+    assert lib.yan_gemm_bf16_tn(64, 64, 64, a.data_ptr(), a.data_ptr(), a.data_ptr(), null) == 0
+    torch.cuda.synchronize()

@@ -1,0 +1,109 @@
+"""Host-side logic that needs no device: helpers, tile heuristics, tuner selection rules, entry-point argument
+checks (reference: yan/jit_kernels/utils.py:32-85, yan/jit_kernels/tuner.py:12-78, yan/jit_kernels/cute_gemm.py:21-30)."""
+import pytest
+import torch
+
+import yan_amd as yan
+from yan_amd.jit_kernels import heuristics, tuner as tuner_mod, bf16_gemm, gemm
+
+
+def test_ceil_div_and_alignment():
+    assert yan.ceil_div(7, 2) == 4 and yan.ceil_div(8, 2) == 4 and yan.ceil_div(0, 128) == 0 and yan.ceil_div(1, 128) == 1
+    assert yan.get_m_alignment_for_contiguous_layout() == 128
+
+
+def test_get_col_major_tensor():
+    x = torch.arange(12, dtype=torch.float32).view(3, 4)
+    y = yan.get_col_major_tensor(x)
+    assert y.shape == x.shape and torch.equal(x, y) and y.stride() == (1, 3)
+    assert yan.get_col_major_tensor(y).data_ptr() == y.data_ptr()          # already token-contiguous: untouched
+    b = torch.arange(24, dtype=torch.float32).view(2, 3, 4)
+    yb = yan.get_col_major_tensor(b)
+    assert torch.equal(b, yb) and yb.stride(1) == 1 and yb.stride(2) == 3
+    with pytest.raises(AssertionError):
+        yan.get_col_major_tensor(torch.zeros(3))
+
+
+def test_tile_heuristics_fill_256_cus():
+    # the headline FP8 shape: 256x256 tiles give 448 workgroups = 1.75 rounds
+    assert heuristics.get_best_fp8_config(4096, 7168, 7168, 256) in ((256, 256), (256, 128), (128, 256))
+    assert heuristics.get_best_dense_config(8192, 8192, 8192, 256) == (256, 256)
+    # a skinny problem must not pick a tile that leaves most CUs idle
+    bm, bn = heuristics.get_best_fp8_config(64, 4096, 7168, 256)
+    assert bm == 64 and yan.ceil_div(4096, bn) >= 64
+    # tiny problems get the smallest tile
+    assert heuristics.get_best_dense_config(64, 64, 64, 256) == (64, 64)
+    ranked = heuristics.rank_tiles(4096, 7168, 256, heuristics._FP8_TILES)
+    assert ranked == sorted(ranked) and len(ranked) == len(heuristics._FP8_TILES)
+
+
+def test_kernel_plans_keep_reference_keys_and_argument_order():
+    name, keys, defs = bf16_gemm.dense_kernel_plan(4096, 7168, 2048, torch.bfloat16, 256)
+    assert name == 'gemm_bf16_tn' and sorted(keys) == ['BLOCK_M', 'BLOCK_N', 'NUM_STAGES']
+    assert [d[0] for d in defs] == ['m', 'n', 'k', 'A', 'B', 'C', 'stream']
+    assert bf16_gemm.dense_kernel_plan(4096, 7168, 2048, torch.half, 256)[0] == 'gemm_fp16_tn'
+    name, keys, defs, smem = gemm.fp8_kernel_plan(4096, 7168, 7168, 256)
+    assert name == 'gemm_fp8_fp8_bf16_nt'
+    assert sorted(keys) == ['BLOCK_M', 'BLOCK_N', 'K', 'N', 'NUM_STAGES', 'NUM_TMA_MULTICAST']
+    assert [d[0] for d in defs][:9] == ['lhs', 'lhs_scales', 'rhs', 'rhs_scales', 'out', 'm', 'stream', 'num_sms', 'smem_size']
+    assert keys['N'] == 7168 and keys['K'] == 7168 and smem == 2 * (keys['BLOCK_M'] + keys['BLOCK_N']) * 128 <= 160 * 1024
+
+
+def test_entry_points_reject_bad_arguments_before_touching_a_device():
+    a, b = torch.zeros(8, 16, dtype=torch.bfloat16), torch.zeros(4, 16, dtype=torch.bfloat16)
+    with pytest.raises(AssertionError):
+        yan.gemm_bf16_tn(a, b, torch.zeros(8, 8, dtype=torch.bfloat16))          # n mismatch
+    with pytest.raises(AssertionError):
+        yan.gemm_bf16_tn(a.half(), b, torch.zeros(8, 4, dtype=torch.bfloat16))   # dtype mismatch
+    with pytest.raises(AssertionError):
+        yan.gemm_fp16_tn(a, b, torch.zeros(8, 4, dtype=torch.bfloat16))
+    # empty problems return before any device call
+    yan.gemm_bf16_tn(torch.zeros(0, 16, dtype=torch.bfloat16), b, torch.zeros(0, 4, dtype=torch.bfloat16))
+    yan.gemm_fp16_tn(torch.zeros(8, 16, dtype=torch.half), torch.zeros(0, 16, dtype=torch.half), torch.zeros(8, 0, dtype=torch.half))
+    q = torch.zeros(0, 128, dtype=torch.float8_e4m3fn)
+    w = torch.zeros(128, 128, dtype=torch.float8_e4m3fn)
+    yan.gemm_fp8_fp8_bf16_nt((q, torch.zeros(0, 1)), (w, torch.ones(1, 1)), torch.zeros(0, 128, dtype=torch.bfloat16))
+    with pytest.raises(AssertionError):     # k not a multiple of the 128-deep scale block
+        yan.gemm_fp8_fp8_bf16_nt((torch.zeros(4, 64, dtype=torch.float8_e4m3fn), torch.zeros(4, 1)),
+                                 (torch.zeros(128, 64, dtype=torch.float8_e4m3fn), torch.ones(1, 1)),
+                                 torch.zeros(4, 128, dtype=torch.bfloat16))
+    with pytest.raises(AssertionError):     # wrong scale-table shape
+        yan.gemm_fp8_fp8_bf16_nt((torch.zeros(4, 128, dtype=torch.float8_e4m3fn), torch.zeros(4, 2)),
+                                 (w, torch.ones(1, 1)), torch.zeros(4, 128, dtype=torch.bfloat16))
+
+
+class _FakeRuntime:
+    def __init__(self, tag, rc=0):
+        self.tag, self.rc, self.calls = tag, rc, 0
+
+    def __call__(self, *args):
+        self.calls += 1
+        return self.rc
+
+
+def test_tuner_memoises_skips_illegal_and_keeps_the_fastest(monkeypatch):
+    built = []
+    times = {'a': 3.0, 'b': 1.0, 'c': 2.0, 'bad': 0.1}
+
+    def fake_build(name, arg_defs, code):
+        tag = code.split('TAG=')[1].split(';')[0]
+        rt = _FakeRuntime(tag, rc=5 if tag == 'bad' else 0)
+        built.append(rt)
+        return rt
+
+    monkeypatch.setattr(tuner_mod, 'build', fake_build)
+    monkeypatch.setattr(tuner_mod, '_time_candidate', lambda rt, args: times[rt.tag])
+    t = tuner_mod.JITTuner()
+    kw = dict(includes=(), arg_defs=(('n', int),), template='\nint TAG={T}; int k={KEY};\n', args=(1,))
+    space = ({'T': 'a'}, {'T': 'bad'}, {'T': 'b'}, {'T': 'c'})
+    best = t.compile_and_tune(name='op', keys={'KEY': 1}, space=space, **kw)
+    assert best.tag == 'b' and len(built) == 4
+    assert [r.calls for r in built] == [1, 1, 1, 1]              # one validity run each; the illegal one is not timed
+    # memo hit: same name and keys (in any order) -> no new build
+    assert t.compile_and_tune(name='op', keys={'KEY': 1}, space=space, **kw) is best and len(built) == 4
+    # different keys -> new entry; empty space -> exactly one build, not run, time 0
+    one = t.compile_and_tune(name='op', keys={'KEY': 2, 'T': 'c'}, space=(), **kw)
+    assert one.tag == 'c' and one.calls == 0 and len(built) == 5
+    # every candidate illegal -> assertion
+    with pytest.raises(AssertionError, match='Failed to tune'):
+        t.compile_and_tune(name='op2', keys={'KEY': 3}, space=({'T': 'bad'}, {'T': 'bad'}), **kw)

@@ -1,0 +1,56 @@
+"""ctypes binding of the ahead-of-time C-ABI library (include/yan_gemm.h). There is no fallback: if
+libyan_gemm.so has not been built (`python yan_amd/csrc/build.py`), loading raises."""
+import ctypes
+import os
+
+import torch
+
+_LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), 'csrc', 'libyan_gemm.so')
+_lib = None
+
+SYMBOLS = ('yan_gemm_bf16_tn', 'yan_gemm_fp16_tn', 'yan_gemm_fp8_fp8_bf16_nt', 'yan_gemm_select_tile', 'yan_gemm_version')
+
+
+def load() -> ctypes.CDLL:
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            raise RuntimeError(f'{_LIB_PATH} is missing: build it with `python yan_amd/csrc/build.py`')
+        lib = ctypes.CDLL(_LIB_PATH)
+        vp, ci, ll = ctypes.c_void_p, ctypes.c_int, ctypes.c_longlong
+        lib.yan_gemm_bf16_tn.argtypes = lib.yan_gemm_fp16_tn.argtypes = [ci, ci, ci, vp, vp, vp, vp]
+        lib.yan_gemm_fp8_fp8_bf16_nt.argtypes = [vp, vp, ll, ll, vp, vp, vp, ci, ci, ci, vp, ci]
+        lib.yan_gemm_select_tile.argtypes = [ci, ci, ci, ci, ci, ctypes.POINTER(ci), ctypes.POINTER(ci)]
+        for name in SYMBOLS[:4]:
+            getattr(lib, name).restype = ci
+        lib.yan_gemm_version.restype = ctypes.c_char_p
+        _lib = lib
+    return _lib
+
+
+def _stream_handle():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def gemm_bf16_tn(a: torch.Tensor, b: torch.Tensor, c: torch.Tensor) -> int:
+    (m, k), n = a.shape, b.shape[0]
+    return load().yan_gemm_bf16_tn(m, n, k, a.data_ptr(), b.data_ptr(), c.data_ptr(), _stream_handle())
+
+
+def gemm_fp16_tn(a: torch.Tensor, b: torch.Tensor, c: torch.Tensor) -> int:
+    (m, k), n = a.shape, b.shape[0]
+    return load().yan_gemm_fp16_tn(m, n, k, a.data_ptr(), b.data_ptr(), c.data_ptr(), _stream_handle())
+
+
+def gemm_fp8_fp8_bf16_nt(lhs, rhs, out: torch.Tensor, num_sms: int = 0) -> int:
+    (a8, sa), (b8, sb) = lhs, rhs
+    (m, k), n = a8.shape, b8.shape[0]
+    return load().yan_gemm_fp8_fp8_bf16_nt(a8.data_ptr(), sa.data_ptr(), sa.stride(0), sa.stride(1), b8.data_ptr(),
+                                           sb.data_ptr(), out.data_ptr(), m, n, k, _stream_handle(), num_sms)
+
+
+def select_tile(op: int, m: int, n: int, k: int, num_cus: int):
+    bm, bn = ctypes.c_int(0), ctypes.c_int(0)
+    rc = load().yan_gemm_select_tile(op, m, n, k, num_cus, ctypes.byref(bm), ctypes.byref(bn))
+    assert rc == 0
+    return bm.value, bn.value

@@ -1,0 +1,97 @@
+// Ahead-of-time C-ABI library over the JIT's kernel headers: every tile variant instantiated once, sizes at run time.
+// Declarations and contracts: include/yan_gemm.h.
+#include "../../include/yan_gemm.h"
+
+#include "gemm/bf16_gemm.hpp"
+#include "gemm/fp8_gemm.hpp"
+
+namespace {
+
+struct TileCost { int bm, bn; double per_area; };
+
+// Same tables and cost model as yan_amd/jit_kernels/heuristics.py (a CPU test keeps the two in step).
+constexpr TileCost kDenseTiles[] = {{256, 256, 1.00}, {256, 128, 1.12}, {128, 256, 1.12}, {128, 128, 1.30}, {64, 128, 1.7}, {64, 64, 2.4}};
+constexpr TileCost kFp8Tiles[]   = {{256, 256, 1.00}, {256, 128, 1.12}, {128, 256, 1.12}, {128, 128, 1.30}, {64, 128, 1.7}, {64, 64, 2.2},
+                                    {64, 32, 3.0}, {64, 16, 4.5}};
+
+template <int COUNT>
+void pick(const TileCost (&tiles)[COUNT], int m, int n, int num_cus, int* bm, int* bn) {
+    double best = -1;
+    for (const TileCost& t : tiles) {
+        const long long count  = (long long)((m + t.bm - 1) / t.bm) * ((n + t.bn - 1) / t.bn);
+        const long long rounds = (count + num_cus - 1) / num_cus;
+        const double cost = double(rounds) * t.bm * t.bn * t.per_area;
+        // ties go to the earlier entry of the (cost, tile) ordering the Python side sorts by
+        if (best < 0 || cost < best || (cost == best && (t.bm < *bm || (t.bm == *bm && t.bn < *bn)))) { best = cost; *bm = t.bm; *bn = t.bn; }
+    }
+}
+
+int device_cus() {
+    static int cus = 0;
+    if (cus == 0) {
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+            cus = 256;
+    }
+    return cus;
+}
+
+template <typename Atom, typename Elem>
+int dense(int m, int n, int k, const void* a, const void* b, void* c, void* stream) {
+    if (m == 0 || n == 0) return 0;
+    if (m < 0 || n < 0) return int(hipErrorInvalidValue);
+    int bm = 0, bn = 0;
+    pick(kDenseTiles, m, n, device_cus(), &bm, &bn);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+#define YAN_DENSE_CASE(BM, BN) if (bm == BM && bn == BN) return int(yan::launch_dense<Atom, Elem, BM, BN>(m, n, k, a, b, c, s));
+    YAN_DENSE_CASE(256, 256) YAN_DENSE_CASE(256, 128) YAN_DENSE_CASE(128, 256) YAN_DENSE_CASE(128, 128) YAN_DENSE_CASE(64, 128) YAN_DENSE_CASE(64, 64)
+#undef YAN_DENSE_CASE
+    return int(hipErrorInvalidValue);
+}
+
+} // namespace
+
+extern "C" {
+
+int yan_gemm_bf16_tn(int m, int n, int k, const void* a, const void* b, void* c, void* stream) {
+    return dense<yan::MfmaBF16_32x32x16, __bf16>(m, n, k, a, b, c, stream);
+}
+
+int yan_gemm_fp16_tn(int m, int n, int k, const void* a, const void* b, void* c, void* stream) {
+    return dense<yan::MfmaF16_32x32x16, _Float16>(m, n, k, a, b, c, stream);
+}
+
+int yan_gemm_fp8_fp8_bf16_nt(const void* lhs, const float* lhs_scales, long long lhs_scales_stride_m,
+                             long long lhs_scales_stride_k, const void* rhs, const float* rhs_scales, void* out,
+                             int m, int n, int k, void* stream, int num_sms) {
+    if (m == 0 || n == 0) return 0;
+    if (m < 0 || n < 0 || k <= 0) return int(hipErrorInvalidValue);
+    // the kernel addresses the scale tensor with 32-bit byte offsets
+    const long long last = (long long)(m - 1) * lhs_scales_stride_m + (long long)(k / 128 - 1) * lhs_scales_stride_k;
+    if (lhs_scales_stride_m < 0 || lhs_scales_stride_k < 0 || last >= (1ll << 28)) return int(hipErrorInvalidValue);
+    int bm = 0, bn = 0;
+    pick(kFp8Tiles, m, n, num_sms > 0 ? num_sms : device_cus(), &bm, &bn);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    __hip_bfloat16* o = static_cast<__hip_bfloat16*>(out);
+#define YAN_FP8_CASE(BM, BN)                                                                                         \
+    if (bm == BM && bn == BN)                                                                                        \
+        return int(yan::Gemm<0, 0, BM, BN, 128, 1, 2, 1, yan::GemmType::Normal>::run_sized(                          \
+            o, lhs, lhs_scales, int(lhs_scales_stride_m), int(lhs_scales_stride_k), rhs, rhs_scales, m, n, k, s, num_sms, 0));
+    YAN_FP8_CASE(256, 256) YAN_FP8_CASE(256, 128) YAN_FP8_CASE(128, 256) YAN_FP8_CASE(128, 128) YAN_FP8_CASE(64, 128) YAN_FP8_CASE(64, 64)
+    YAN_FP8_CASE(64, 32) YAN_FP8_CASE(64, 16)
+#undef YAN_FP8_CASE
+    return int(hipErrorInvalidValue);
+}
+
+int yan_gemm_select_tile(int op, int m, int n, int k, int num_cus, int* block_m, int* block_n) {
+    (void)k;
+    if (!block_m || !block_n || num_cus <= 0) return 1;
+    if (op == 0) pick(kDenseTiles, m, n, num_cus, block_m, block_n);
+    else if (op == 1) pick(kFp8Tiles, m, n, num_cus, block_m, block_n);
+    else return 1;
+    return 0;
+}
+
+const char* yan_gemm_version(void) { return "yan-gemm gfx950 6 dense + 8 fp8 tile variants"; }
+
+} // extern "C"

@@ -93,11 +93,13 @@ BASELINE_FP8 = {'cfg3': (4096, 7168, 7168), 'cfg4': (64, 4096, 7168), 'cfg5': (1
 DENSE_TEST_SHAPES = [
     (1024, 1024, 1024), (8192, 8192, 8192),
     (128, 256, 256), (64, 64, 64), (1, 64, 64), (255, 132, 72), (300, 520, 8), (33, 4, 200), (257, 1028, 1096),
+    (300, 256, 256), (33, 132, 72), (96, 80, 136),
     (256, 5120, 5120), (4096, 2048, 7168), (4096, 7168, 2048), (256, 24576, 1536),
 ]
 FP8_TEST_SHAPES = [
     (4096, 7168, 7168), (64, 4096, 7168), (16384, 16384, 16384),
-    (64, 256, 384), (512, 1024, 1024), (1, 128, 128), (63, 192, 256), (129, 320, 128), (300, 96, 640), 
+    (64, 256, 384), (512, 1024, 1024), (1, 128, 128), (63, 192, 256), (129, 320, 128), (300, 96, 640),
+    (40, 192, 256), (130, 448, 640),
     (257, 2112, 1024), (128, 7168, 2048), (4096, 2048, 7168),
 ]
 
