@@ -72,10 +72,14 @@ dense_gemm_mfma(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, El
     const int num_k_tiles = ceil_div(k_bytes, kRowBytes);
     const int tail_tile = (k_bytes % kRowBytes) ? num_k_tiles - 1 : -1;
     const uint32_t tail_a = stage_a.tail_voff(k_bytes % kRowBytes), tail_b = stage_b.tail_voff(k_bytes % kRowBytes);
-    auto prefetch = [&](int kt, uint8_t* la, uint8_t* lb) {
+    using StA = TileStager<BLOCK_M, NW>;
+    using StB = TileStager<BLOCK_N, NW>;
+    constexpr int NUM_COPIES = StA::PASSES + StB::PASSES;
+    // Copy number `d` (A passes first, then B passes) of k-tile `kt` into the given stage.
+    auto copy_pass = [&](int d, int kt, uint8_t* la, uint8_t* lb) {
         const bool tail = kt == tail_tile;
-        stage_a.issue_from(rsrc_a, la, kt * kRowBytes, wave, tail ? tail_a : stage_a.voff);
-        stage_b.issue_from(rsrc_b, lb, kt * kRowBytes, wave, tail ? tail_b : stage_b.voff);
+        if (d < StA::PASSES) stage_a.issue_pass_from(rsrc_a, la, kt * kRowBytes, wave, d, tail ? tail_a : stage_a.voff);
+        else stage_b.issue_pass_from(rsrc_b, lb, kt * kRowBytes, wave, d - StA::PASSES, tail ? tail_b : stage_b.voff);
     };
 
     // Lane-constant LDS offsets of the four 16-deep K steps inside a 64-deep tile.
@@ -93,7 +97,14 @@ dense_gemm_mfma(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, El
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
     // One k-tile = four 16-deep steps; the fragments of step kk+1 are fetched before the MFMAs of step kk issue.
-    auto compute_tile = [&](const uint8_t* la, const uint8_t* lb) {
+    // `step_hook(kk)` runs once per step and is where the copies of the next k-tile are started.
+    constexpr int SPREAD_STEPS = 2;
+    auto copies_in_step = [](int kk) {
+        int c = 0;
+        for (int d = 0; d < NUM_COPIES; ++d) c += (d * SPREAD_STEPS / NUM_COPIES == kk);
+        return c;
+    };
+    auto compute_tile = [&](const uint8_t* la, const uint8_t* lb, auto&& step_hook) {
         using Frag = typename Atom::Frag;
         const uint8_t* pa = la + wm * Cfg::WTM * kRowBytes;
         const uint8_t* pb = lb + wn * Cfg::WTN * kRowBytes;
@@ -108,41 +119,50 @@ dense_gemm_mfma(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, El
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int kk = 0; kk < 4; ++kk) {
+            step_hook(kk);
             if (kk + 1 < 4) fetch(kk + 1);
 #pragma unroll
             for (int i = 0; i < TN; ++i)
 #pragma unroll
                 for (int j = 0; j < TM; ++j) acc[i][j] = Atom::mma(nf[kk & 1][i], mf[kk & 1][j], acc[i][j]);
-            // Issue order inside the step: one LDS read, one MFMA, ... so the reads ride under the MFMAs.
-            if (kk + 1 < 4) {
+            // Issue order inside the step: one LDS read, one copy instruction, one MFMA, ... so that reads and
+            // copies ride under the MFMAs instead of queueing in front of them.
+            {
+                constexpr int kDsRead = 0x100, kVmem = 0x020, kMfma = 0x008;
+                const int reads = kk + 1 < 4 ? TN + TM : 0, copies = copies_in_step(kk);
 #pragma unroll
-                for (int x = 0; x < TN + TM; ++x) {
-                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                for (int x = 0; x < TN * TM; ++x) {
+                    if (x < reads) __builtin_amdgcn_sched_group_barrier(kDsRead, 1, 0);
+                    if (x < copies) __builtin_amdgcn_sched_group_barrier(kVmem, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(kMfma, 1, 0);
                 }
-                __builtin_amdgcn_sched_group_barrier(0x008, TN * TM - (TN + TM), 0);
             }
             __builtin_amdgcn_sched_barrier(0);
         }
     };
 
     // Two LDS stages; the copy of tile kt+1 is in flight while tile kt is consumed. The barrier both publishes
-    // the tile that just landed and retires every wave's reads of the stage about to be overwritten. The
-    // steady-state body is branch-free: a copy started for a tile past the end is simply never consumed.
-    prefetch(0, lds_a0, lds_b0);
+    // the tile that just landed and retires every wave's reads of the stage about to be overwritten. The copies
+    // are started a few at a time during the first two of the four steps rather than in one burst after the
+    // barrier, so the memory pipeline's issue time hides under MFMAs and the copies still get half a k-tile to
+    // land. The steady-state body is branch-free: a copy started for a tile past the end is never consumed.
+    auto k_step = [&](int kt, const uint8_t* a_cur, const uint8_t* b_cur, uint8_t* a_nxt, uint8_t* b_nxt) {
+        wait_for_copies();
+        __syncthreads();
+        compute_tile(a_cur, b_cur, [&](int kk) {
+#pragma unroll
+            for (int d = 0; d < NUM_COPIES; ++d)
+                if (d * SPREAD_STEPS / NUM_COPIES == kk) copy_pass(d, kt + 1, a_nxt, b_nxt);
+        });
+    };
+#pragma unroll
+    for (int d = 0; d < NUM_COPIES; ++d) copy_pass(d, 0, lds_a0, lds_b0);
     int kt = 0;
     for (; kt + 1 < num_k_tiles; kt += 2) {
-        __syncthreads();
-        prefetch(kt + 1, lds_a1, lds_b1);
-        compute_tile(lds_a0, lds_b0);
-        __syncthreads();
-        prefetch(kt + 2, lds_a0, lds_b0);
-        compute_tile(lds_a1, lds_b1);
+        k_step(kt, lds_a0, lds_b0, lds_a1, lds_b1);
+        k_step(kt + 1, lds_a1, lds_b1, lds_a0, lds_b0);
     }
-    if (kt < num_k_tiles) {
-        __syncthreads();
-        compute_tile(lds_a0, lds_b0);
-    }
+    if (kt < num_k_tiles) k_step(kt, lds_a0, lds_b0, lds_a1, lds_b1);
 
     // Epilogue: registers 4*q .. 4*q+3 of an atom are n = 8*q + 4*g + {0,1,2,3} of column m = lane % 32.
     const int m_lane = m0 + wm * Cfg::WTM + lane % 32;

@@ -114,9 +114,11 @@ fp8_gemm_kernel(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_s
 
     // One k-tile: TN x TM atoms, software-pipelined by hand. Step t issues the MFMA of atom t (fresh zero
     // accumulator) and folds in the partial sums of atom t - DEPTH, whose MFMA has retired by then; the fragment of
-    // weight rows i+1 is fetched while rows i are being multiplied. sched_barrier keeps the compiler from
-    // regrouping the steps (it would otherwise hoist every MFMA and need a register per partial sum).
-    auto compute_tile = [&](const uint8_t* la, const uint8_t* lb, const float (&sa)[TM], const float (&sb)[NB]) {
+    // weight rows i+1 is fetched while rows i are being multiplied; `row_hook(i)` runs once per row of atoms and
+    // is where the copies of the next k-tile are started. sched_barrier keeps the compiler from regrouping the
+    // steps (it would otherwise hoist every MFMA and need a register per partial sum).
+    auto compute_tile = [&](const uint8_t* la, const uint8_t* lb, const float (&sa)[TM], const float (&sb)[NB],
+                            auto&& row_hook) {
         constexpr int T = TN * TM, DEPTH = 2, RING = 4;
         const uint8_t* pa = la + wm * Cfg::WTM * kRowBytes;
         const uint8_t* pb = lb + wn * Cfg::WTN * kRowBytes;
@@ -131,6 +133,7 @@ fp8_gemm_kernel(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_s
         for (int t = 0; t < T + DEPTH; ++t) {
             if (t < T) {
                 const int i = t / TM, j = t % TM;
+                if (j == 1 % TM) row_hook(i);
                 if (j == 0 && i + 1 < TN) nf[(i + 1) & 1] = read_frag(pb + (i + 1) * 16 * kRowBytes);
                 p[t % RING] = Atom::mma(nf[i & 1], mf[j], f32x4{0.f, 0.f, 0.f, 0.f});
             }
@@ -158,36 +161,41 @@ fp8_gemm_kernel(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_s
     };
 
     // Two LDS stages, one k-tile (= one scale block) of prefetch; the scales of the next block travel in
-    // registers alongside. The steady-state body is branch-free (a copy past the last k-tile is out of range
-    // for the descriptor and moves zeros), which keeps each MFMA/FMA step where it was written.
+    // registers alongside. The copies of the next k-tile are not issued in one burst after the barrier (the
+    // memory pipeline takes ~16 cycles per instruction and both waves of every SIMD would sit in its queue while
+    // the matrix core idles): they are handed out a few at a time over the first half of the rows of atoms, which
+    // still leaves them more than half a k-tile of MFMA time to land. The steady-state body is branch-free (a copy
+    // past the last k-tile reads bytes that are never consumed, or zeros past the end of the matrix), which keeps
+    // each MFMA/FMA step where it was written.
+    using StA = TileStager<BLOCK_M, NW>;
+    using StB = TileStager<BLOCK_N, NW>;
+    constexpr int NUM_COPIES = StA::PASSES + StB::PASSES, SPREAD_ROWS = TN >= 2 ? TN / 2 : 1;
     float sa_cur[TM], sb_cur[NB];
-    auto rotate_scales = [&]() {
+    auto k_step = [&](int kb, const uint8_t* a_cur, const uint8_t* b_cur, uint8_t* a_nxt, uint8_t* b_nxt) {
 #pragma unroll
         for (int j = 0; j < TM; ++j) sa_cur[j] = sa_next[j];
 #pragma unroll
         for (int b = 0; b < NB; ++b) sb_cur[b] = sb_next[b];
+        wait_for_copies();
+        __syncthreads();
+        load_scales(min(kb + 1, NUM_K_BLOCKS - 1));
+        compute_tile(a_cur, b_cur, sa_cur, sb_cur, [&](int row) {
+#pragma unroll
+            for (int d = 0; d < NUM_COPIES; ++d) {
+                if (d * SPREAD_ROWS / NUM_COPIES != row) continue;
+                if (d < StA::PASSES) stage_a.issue_pass(rsrc_a, a_nxt, (kb + 1) * kRowBytes, wave, d);
+                else stage_b.issue_pass(rsrc_b, b_nxt, (kb + 1) * kRowBytes, wave, d - StA::PASSES);
+            }
+        });
     };
-    auto prefetch = [&](int kb, uint8_t* la, uint8_t* lb) {
-        stage_a.issue(rsrc_a, la, kb * kRowBytes, wave);
-        stage_b.issue(rsrc_b, lb, kb * kRowBytes, wave);
-        load_scales(min(kb, NUM_K_BLOCKS - 1));
-    };
-    prefetch(0, lds_a0, lds_b0);
+    stage_a.issue(rsrc_a, lds_a0, 0, wave);
+    stage_b.issue(rsrc_b, lds_b0, 0, wave);
+    load_scales(0);
     for (int kb = 0; kb + 1 < NUM_K_BLOCKS; kb += 2) {
-        rotate_scales();
-        __syncthreads();
-        prefetch(kb + 1, lds_a1, lds_b1);
-        compute_tile(lds_a0, lds_b0, sa_cur, sb_cur);
-        rotate_scales();
-        __syncthreads();
-        prefetch(kb + 2, lds_a0, lds_b0);
-        compute_tile(lds_a1, lds_b1, sa_cur, sb_cur);
+        k_step(kb, lds_a0, lds_b0, lds_a1, lds_b1);
+        k_step(kb + 1, lds_a1, lds_b1, lds_a0, lds_b0);
     }
-    if (NUM_K_BLOCKS % 2 == 1) {
-        rotate_scales();
-        __syncthreads();
-        compute_tile(lds_a0, lds_b0, sa_cur, sb_cur);
-    }
+    if (NUM_K_BLOCKS % 2 == 1) k_step(NUM_K_BLOCKS - 1, lds_a0, lds_b0, lds_a1, lds_b1);
 
     // Epilogue: the 4 registers of atom (i, j) are n = n_slab + 16i + 4g + {0..3} of row m = m_slab + 16j + col.
 #pragma unroll

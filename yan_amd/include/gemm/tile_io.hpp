@@ -30,6 +30,14 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, ui
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, bytes, 0x00020000);
 }
 
+// Block until every copy this wave has started (and every other vector-memory load) has landed. A workgroup
+// barrier alone is not enough before reading a staged tile: the compiler's fence in __syncthreads() only waits
+// for as many outstanding vector-memory operations as its memory model needs, and it does not count copies into
+// LDS among them.
+__device__ __forceinline__ void wait_for_copies() {
+    __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, kNoWaitLgkm));
+}
+
 // One fp32 through a descriptor: per-lane byte offset + wave-uniform byte offset; out of range reads 0.0f.
 __device__ __forceinline__ float buffer_load_f32(__amdgpu_buffer_rsrc_t rsrc, uint32_t voffset, uint32_t soffset) {
     return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsrc, voffset, soffset, 0));
@@ -65,6 +73,19 @@ struct TileStager {
     // whose chunk lies beyond the row end are sent out of range and move zeros.
     __device__ __forceinline__ uint32_t tail_voff(int valid_bytes) const {
         return logical * kChunk < valid_bytes ? voff : kOutOfRange;
+    }
+
+    // One pass (8 rows per wave) of the copy, for callers that interleave the passes with other work.
+    __device__ __forceinline__ void issue_pass(__amdgpu_buffer_rsrc_t rsrc, uint8_t* lds_tile, int k_byte0, int wave, int j) const {
+        issue_pass_from(rsrc, lds_tile, k_byte0, wave, j, voff);
+    }
+
+    __device__ __forceinline__ void issue_pass_from(__amdgpu_buffer_rsrc_t rsrc, uint8_t* lds_tile, int k_byte0, int wave, int j,
+                                                    uint32_t lane_voff) const {
+        const int q = j * NUM_WAVES + wave;
+        if (GROUPS % NUM_WAVES == 0 || q < GROUPS)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, YAN_LDS_PTR(lds_tile + q * 8 * kRowBytes), kChunk, lane_voff,
+                                                     k_byte0 + j * pass_pitch, 0, 0);
     }
 
     __device__ __forceinline__ void issue_from(__amdgpu_buffer_rsrc_t rsrc, uint8_t* lds_tile, int k_byte0, int wave,
