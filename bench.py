@@ -75,6 +75,19 @@ def _cpu_baseline_fp8(a8, sa, b8, sb, budget_s=12.0):
                                       f'best of 2, {t:.2f} s, os.cpu_count()={os.cpu_count()}'}
 
 
+def _measured_traffic():
+    """HBM bytes per launch of the GEMM kernel as measured with rocprofv3 hardware counters (FETCH_SIZE + WRITE_SIZE,
+    scaled by a copy of known size); the figure is kept with the profile summary it comes from. None if absent."""
+    path = os.path.join(ROOT, 'profiles', 'fp8_gemm_4096x7168x7168_hbm_traffic.md')
+    try:
+        for line in open(path):
+            if line.startswith('traffic_bytes_per_launch:'):
+                return float(line.split(':', 1)[1].split()[0])
+    except OSError:
+        pass
+    return None
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument('--gpus', type=int, default=1)
@@ -82,6 +95,9 @@ def main():
     ap.add_argument('--warmup', type=int, default=20)
     ap.add_argument('--also', action='store_true', help='also time bf16 8192^3, the decode shape and 16384^3 (extra fields)')
     ap.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline leg')
+    ap.add_argument('--calibrate-copy', action='store_true',
+                    help='also run a 1 GiB device-to-device copy three times, as the known-size kernel that hardware '
+                         'byte counters (FETCH_SIZE / WRITE_SIZE) are scaled by when profiling')
     args = ap.parse_args()
     if args.gpus != 1:
         print(f'bench.py: this build runs on one GPU; --gpus {args.gpus} is not supported (every figure is a 1-GPU figure)',
@@ -108,6 +124,14 @@ def main():
     assert diff < 1e-3, f'parity lost: calc_diff={diff}'
     del ref
 
+    if args.calibrate_copy:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device='cuda').fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+
     kernel_ms, wall_ms = _event_time_ms(step, args.steps, args.warmup)
     flops = 2.0 * m * n * k
     tflops_job = flops / (wall_ms * 1e-3) / 1e12
@@ -124,7 +148,7 @@ def main():
                    'tile': f"{keys['BLOCK_M']}x{keys['BLOCK_N']}x128", 'cache_state': 'warm (same operands every step)',
                    'calc_diff_sampled_rows': diff},
         'roofline': {'bound': 'mfma', 'achieved': round(tflops_kernel, 1), 'peak': PEAK_FP8_TFLOPS, 'unit': 'TFLOP/s',
-                     'frac': round(tflops_kernel / PEAK_FP8_TFLOPS, 4), 'traffic': None,
+                     'frac': round(tflops_kernel / PEAK_FP8_TFLOPS, 4), 'traffic': _measured_traffic(),
                      'kernel': 'fp8_gemm_kernel', 'kernel_us': round(kernel_ms * 1e3, 2),
                      'algorithmic_flop_per_launch': flops, 'algorithmic_bytes_per_launch': bytes_alg},
     }
