@@ -137,7 +137,7 @@ def main():
     tflops_job = flops / (wall_ms * 1e-3) / 1e12
     tflops_kernel = flops / (kernel_ms * 1e-3) / 1e12
     bytes_alg = m * k + n * k + 4 * m * (k // 128) + 4 * ((n + 127) // 128) * (k // 128) + 2 * m * n
-    _, keys, _, _ = fp8_kernel_plan(m, n, k, yan.get_num_sms())
+    _, keys, _, _, _ = fp8_kernel_plan(m, n, k, yan.get_num_sms())
 
     line = {
         'metric': METRIC, 'value': round(tflops_job, 1), 'unit': 'TFLOPS', 'n_gpus': 1,

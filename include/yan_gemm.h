@@ -57,11 +57,12 @@ YAN_API int yan_gemm_fp8_fp8_bf16_nt(const void* lhs, const float* lhs_scales, l
                              int m, int n, int k, void* stream, int num_sms);
 
 /* Macro tile the library uses for a problem: op 0 = dense 16-bit, 1 = FP8 block-scaled. Writes BLOCK_M / BLOCK_N.
+ * For op 1 with few activation rows the answer is (16 * atoms, 16): the weight-streaming kernel.
  * Host-only (no device call). Stands where the reference leaves tile choice to the caller's keys
  * (yan/jit_kernels/cute_gemm.py:41, yan/jit_kernels/gemm.py:13-16). Returns 0, or 1 for an unknown op. */
 YAN_API int yan_gemm_select_tile(int op, int m, int n, int k, int num_cus, int* block_m, int* block_n);
 
-/* "yan-gemm gfx950 <n> dense + <n> fp8 tile variants". */
+/* "yan-gemm gfx950 <n> dense + <n> fp8 tile variants + <n> weight-streaming fp8 variants". */
 YAN_API const char* yan_gemm_version(void);
 
 /* The JIT boundary, for reference: signatures of `launch` in the kernel.so of each op

@@ -41,11 +41,11 @@ def test_header_is_plain_c(repo_root, tmp_path):
 def test_version_and_tile_selection_match_python(lib):
     assert b'gfx950' in lib.yan_gemm_version()
     shapes = [(4096, 7168, 7168), (64, 4096, 7168), (16384, 16384, 16384), (8192, 8192, 8192), (1024, 1024, 1024),
-              (1, 128, 128), (300, 96, 640), (257, 2112, 1024), (256, 24576, 1536), (4096, 2048, 7168), (129, 320, 128)]
+              (1, 128, 128), (300, 96, 640), (1, 4096, 7168), (17, 4096, 1024), (33, 2112, 640), (64, 7168, 2048), (65, 7168, 2048), (257, 2112, 1024), (256, 24576, 1536), (4096, 2048, 7168), (129, 320, 128)]
     for m, n, k in shapes:
         for cus in (256, 128, 80):
             assert capi.select_tile(0, m, n, k, cus) == heuristics.get_best_dense_config(m, n, k, cus), (m, n, k, cus)
-            assert capi.select_tile(1, m, n, k, cus) == heuristics.get_best_fp8_config(m, n, k, cus), (m, n, k, cus)
+            assert capi.select_tile(1, m, n, k, cus) == heuristics.get_fp8_tile(m, n, k, cus), (m, n, k, cus)
     bm, bn = ctypes.c_int(), ctypes.c_int()
     assert lib.yan_gemm_select_tile(7, 1, 1, 1, 256, ctypes.byref(bm), ctypes.byref(bn)) == 1
     assert lib.yan_gemm_select_tile(0, 1, 1, 1, 0, ctypes.byref(bm), ctypes.byref(bn)) == 1

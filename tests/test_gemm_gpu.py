@@ -278,7 +278,8 @@ def test_capi_dense_matches_oracle_and_jit(m, n, k):
         assert torch.equal(c, c2)            # same kernel source, same tile choice: same bits
 
 
-@pytest.mark.parametrize('m,n,k', [(64, 256, 384), (129, 320, 128), (300, 96, 640), (257, 2112, 1024), (64, 4096, 7168)])
+@pytest.mark.parametrize('m,n,k', [(64, 256, 384), (129, 320, 128), (300, 96, 640), (257, 2112, 1024), (64, 4096, 7168), (1, 4096, 7168),
+                                   (17, 4096, 1024), (33, 2112, 640)])
 def test_capi_fp8_matches_oracle_and_jit(m, n, k):
     from yan_amd import capi
     _announce('capi fp8', m, n, k)

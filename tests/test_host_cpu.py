@@ -31,6 +31,9 @@ def test_tile_heuristics_fill_256_cus():
     # a skinny problem must not pick a tile that leaves most CUs idle
     bm, bn = heuristics.get_best_fp8_config(64, 4096, 7168, 256)
     assert bm == 64 and yan.ceil_div(4096, bn) >= 64
+    # ... and the decode shape goes to the weight-streaming kernel: one workgroup per 16 weight rows
+    assert heuristics.get_fp8_tile(64, 4096, 7168, 256) == (64, 16) and heuristics.get_fp8_tile(1, 4096, 7168, 256) == (16, 16)
+    assert heuristics.get_skinny_fp8_config(65, 4096, 7168, 256) == 0 and heuristics.get_skinny_fp8_config(64, 1024, 7168, 256) == 0
     # tiny problems get the smallest tile
     assert heuristics.get_best_dense_config(64, 64, 64, 256) == (64, 64)
     ranked = heuristics.rank_tiles(4096, 7168, 256, heuristics._FP8_TILES)
@@ -42,7 +45,7 @@ def test_kernel_plans_keep_reference_keys_and_argument_order():
     assert name == 'gemm_bf16_tn' and sorted(keys) == ['BLOCK_M', 'BLOCK_N', 'NUM_STAGES']
     assert [d[0] for d in defs] == ['m', 'n', 'k', 'A', 'B', 'C', 'stream']
     assert bf16_gemm.dense_kernel_plan(4096, 7168, 2048, torch.half, 256)[0] == 'gemm_fp16_tn'
-    name, keys, defs, smem = gemm.fp8_kernel_plan(4096, 7168, 7168, 256)
+    name, keys, defs, smem, _ = gemm.fp8_kernel_plan(4096, 7168, 7168, 256)
     assert name == 'gemm_fp8_fp8_bf16_nt'
     assert sorted(keys) == ['BLOCK_M', 'BLOCK_N', 'K', 'N', 'NUM_STAGES', 'NUM_TMA_MULTICAST']
     assert [d[0] for d in defs][:9] == ['lhs', 'lhs_scales', 'rhs', 'rhs_scales', 'out', 'm', 'stream', 'num_sms', 'smem_size']

@@ -146,6 +146,6 @@ def test_gemm_kernels_compile_for_gfx950(cache_dir):
     name, keys, defs = bf16_gemm.dense_kernel_plan(64, 64, 64, torch.bfloat16, 256)
     rt = jit.build(name, defs, jit.generate(bf16_gemm.includes, defs, jit.cpp_format(bf16_gemm.template, keys)))
     assert runtime.Runtime.is_path_valid(rt.path)
-    name, keys, defs, _ = gemm.fp8_kernel_plan(1, 128, 128, 256)
-    rt = jit.build(name, defs, jit.generate(gemm.includes, defs, jit.cpp_format(gemm.template, keys)))
+    name, keys, defs, _, tmpl = gemm.fp8_kernel_plan(1, 128, 128, 256)
+    rt = jit.build(name, defs, jit.generate(gemm.includes, defs, jit.cpp_format(tmpl, keys)))
     assert runtime.Runtime.is_path_valid(rt.path)

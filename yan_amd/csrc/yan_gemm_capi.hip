@@ -4,6 +4,7 @@
 
 #include "gemm/bf16_gemm.hpp"
 #include "gemm/fp8_gemm.hpp"
+#include "gemm/fp8_gemm_skinny.hpp"
 
 namespace {
 
@@ -24,6 +25,12 @@ void pick(const TileCost (&tiles)[COUNT], int m, int n, int num_cus, int* bm, in
         // ties go to the earlier entry of the (cost, tile) ordering the Python side sorts by
         if (best < 0 || cost < best || (cost == best && (t.bm < *bm || (t.bm == *bm && t.bn < *bn)))) { best = cost; *bm = t.bm; *bn = t.bn; }
     }
+}
+
+// Activation atoms of the weight-streaming kernel, or 0 for the tiled kernel (get_skinny_fp8_config in heuristics.py).
+int skinny_atoms(int m, int n, int num_cus) {
+    if (m > 0 && m <= 64 && n >= 8 * num_cus) return m <= 16 ? 1 : (m <= 32 ? 2 : 4);
+    return 0;
 }
 
 int device_cus() {
@@ -69,10 +76,17 @@ int yan_gemm_fp8_fp8_bf16_nt(const void* lhs, const float* lhs_scales, long long
     // the kernel addresses the scale tensor with 32-bit byte offsets
     const long long last = (long long)(m - 1) * lhs_scales_stride_m + (long long)(k / 128 - 1) * lhs_scales_stride_k;
     if (lhs_scales_stride_m < 0 || lhs_scales_stride_k < 0 || last >= (1ll << 28)) return int(hipErrorInvalidValue);
-    int bm = 0, bn = 0;
-    pick(kFp8Tiles, m, n, num_sms > 0 ? num_sms : device_cus(), &bm, &bn);
+    const int cus = num_sms > 0 ? num_sms : device_cus();
     hipStream_t s = static_cast<hipStream_t>(stream);
     __hip_bfloat16* o = static_cast<__hip_bfloat16*>(out);
+    if (const int atoms = skinny_atoms(m, n, cus)) {
+        const int sm = int(lhs_scales_stride_m), sk = int(lhs_scales_stride_k);
+        if (atoms == 1) return int(yan::launch_fp8_skinny<0, 0, 1, 8>(o, lhs, lhs_scales, sm, sk, rhs, rhs_scales, m, n, k, s));
+        if (atoms == 2) return int(yan::launch_fp8_skinny<0, 0, 2, 8>(o, lhs, lhs_scales, sm, sk, rhs, rhs_scales, m, n, k, s));
+        return int(yan::launch_fp8_skinny<0, 0, 4, 8>(o, lhs, lhs_scales, sm, sk, rhs, rhs_scales, m, n, k, s));
+    }
+    int bm = 0, bn = 0;
+    pick(kFp8Tiles, m, n, cus, &bm, &bn);
 #define YAN_FP8_CASE(BM, BN)                                                                                         \
     if (bm == BM && bn == BN)                                                                                        \
         return int(yan::Gemm<0, 0, BM, BN, 128, 1, 2, 1, yan::GemmType::Normal>::run_sized(                          \
@@ -87,11 +101,14 @@ int yan_gemm_select_tile(int op, int m, int n, int k, int num_cus, int* block_m,
     (void)k;
     if (!block_m || !block_n || num_cus <= 0) return 1;
     if (op == 0) pick(kDenseTiles, m, n, num_cus, block_m, block_n);
-    else if (op == 1) pick(kFp8Tiles, m, n, num_cus, block_m, block_n);
+    else if (op == 1) {
+        if (const int atoms = skinny_atoms(m, n, num_cus)) { *block_m = 16 * atoms; *block_n = 16; }
+        else pick(kFp8Tiles, m, n, num_cus, block_m, block_n);
+    }
     else return 1;
     return 0;
 }
 
-const char* yan_gemm_version(void) { return "yan-gemm gfx950 6 dense + 8 fp8 tile variants"; }
+const char* yan_gemm_version(void) { return "yan-gemm gfx950 6 dense + 8 fp8 tile variants + 3 weight-streaming fp8 variants"; }
 
 } // extern "C"

@@ -5,9 +5,11 @@
 // contiguous, C [m,n] row-major written in place, work enqueued on `stream`), but none of its structure:
 // the reference kernel (cute_gemm.cuh:14-260) is a 128x128x32 cp.async/ldmatrix/mma.sync pipeline with fp16
 // accumulation and no bounds handling. Here:
-//   * macro tile BLOCK_M x BLOCK_N x 64 (128-byte rows), 8 waves (2 per SIMD) for big tiles, 4 otherwise;
+//   * macro tile BLOCK_M x BLOCK_N x 64 (128-byte rows), 4 waves, one per SIMD;
 //   * HBM -> LDS with buffer_load ... lds into two static LDS stages (tile_io.hpp);
-//   * each wave owns a (BLOCK_N/WAVES_N) x (BLOCK_M/WAVES_M) slab computed with 32x32x16 MFMAs. B rows feed the
+//   * each wave owns a (BLOCK_N/WAVES_N) x (BLOCK_M/WAVES_M) slab, up to 128 x 128 (256 accumulator registers, which
+//     the compiler keeps in AGPRs), computed with 32x32x16 MFMAs: the larger the slab, the fewer LDS bytes are read
+//     per flop, and on a part whose clock is set by power that is what buys throughput. B rows feed the
 //     MFMA row operand and A rows the column operand, so a lane's four consecutive accumulator registers are
 //     four consecutive n of one m: contiguous in C;
 //   * fp32 accumulators, round-to-nearest-even on the way out;
@@ -27,9 +29,9 @@ namespace yan {
 
 template <int BLOCK_M, int BLOCK_N>
 struct DenseTileConfig {
-    static constexpr int NUM_WAVES = get_num_waves(BLOCK_M, BLOCK_N);
-    // A slab of at most 128 x 64 outputs: 128 accumulator registers per lane.
-    static constexpr int WAVES_N   = pick_waves_n(BLOCK_M, BLOCK_N, NUM_WAVES, 32, 128 * 64);
+    static constexpr int NUM_WAVES = 4;
+    // A slab of at most 128 x 128 outputs: 256 accumulator registers per lane, out of the 512 a lone wave may hold.
+    static constexpr int WAVES_N   = pick_waves_n(BLOCK_M, BLOCK_N, NUM_WAVES, 32, 128 * 128);
     static_assert(WAVES_N > 0, "no wave layout fits this tile");
     static constexpr int WAVES_M   = NUM_WAVES / WAVES_N;
     static constexpr int WTN = BLOCK_N / WAVES_N, WTM = BLOCK_M / WAVES_M;
@@ -39,7 +41,7 @@ struct DenseTileConfig {
 };
 
 template <typename Atom, typename Elem, int BLOCK_M, int BLOCK_N>
-__global__ void __launch_bounds__((get_num_waves(BLOCK_M, BLOCK_N) * kWaveSize))
+__global__ void __launch_bounds__(4 * kWaveSize)
 dense_gemm_mfma(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, Elem* __restrict__ C,
                 int m, int n, int k) {
     using Cfg = DenseTileConfig<BLOCK_M, BLOCK_N>;

@@ -13,12 +13,12 @@ from typing import Tuple
 
 import torch
 
-from .heuristics import get_best_fp8_config
+from .heuristics import get_best_fp8_config, get_skinny_fp8_config
 from .tuner import jit_tuner
 from .utils import get_num_sms, ceil_div, get_col_major_tensor
 
 # C++ code templates
-includes = ('"gemm/fp8_gemm.hpp"', )
+includes = ('"gemm/fp8_gemm.hpp"', '"gemm/fp8_gemm_skinny.hpp"')
 template = """
 using namespace yan;
 
@@ -37,6 +37,24 @@ __return_code = static_cast<int>(GemmType::run(out, lhs, lhs_scales, lhs_scales_
                                                rhs, rhs_scales, m, stream, num_sms, smem_size));
 """
 
+# Few activation rows (decode): BLOCK_M / 16 activation atoms per workgroup, 16 weight rows per workgroup, the K blocks
+# of a workgroup shared out over NUM_WAVES waves; no LDS staging, so NUM_STAGES is the per-wave load depth's name only.
+skinny_template = """
+using namespace yan;
+
+// Templated args from Python JIT call
+constexpr auto N = {N}, K = {K};
+constexpr auto BLOCK_M = {BLOCK_M};
+constexpr auto BLOCK_N = {BLOCK_N};
+constexpr auto kNumStages = {NUM_STAGES};
+constexpr auto kNumTMAMulticast = {NUM_TMA_MULTICAST};
+static_assert(BLOCK_N == 16 && BLOCK_M % 16 == 0);
+
+// Launch kernel
+__return_code = static_cast<int>(launch_fp8_skinny<N, K, BLOCK_M / 16, {NUM_WAVES}>(
+    out, lhs, lhs_scales, lhs_scales_stride_m, lhs_scales_stride_k, rhs, rhs_scales, m, N, K, stream));
+"""
+
 arg_defs = (('lhs', torch.float8_e4m3fn), ('lhs_scales', torch.float),
             ('rhs', torch.float8_e4m3fn), ('rhs_scales', torch.float),
             ('out', torch.bfloat16), ('m', int),
@@ -45,11 +63,16 @@ arg_defs = (('lhs', torch.float8_e4m3fn), ('lhs_scales', torch.float),
 
 
 def fp8_kernel_plan(m: int, n: int, k: int, num_cus: int):
-    """(name, keys, arg_defs, smem_size) of the JIT kernel a call with these sizes uses; needs no GPU."""
+    """(name, keys, arg_defs, smem_size, template) of the JIT kernel a call with these sizes uses; needs no GPU."""
+    skinny_atoms = get_skinny_fp8_config(m, n, k, num_cus)
+    if skinny_atoms:
+        keys = {'N': n, 'K': k, 'BLOCK_M': 16 * skinny_atoms, 'BLOCK_N': 16, 'NUM_STAGES': 4, 'NUM_TMA_MULTICAST': 1,
+                'NUM_WAVES': 8}
+        return 'gemm_fp8_fp8_bf16_nt', keys, arg_defs, 8 * skinny_atoms * 64 * 16, skinny_template
     block_m, block_n = get_best_fp8_config(m, n, k, num_cus)
     keys = {'N': n, 'K': k, 'BLOCK_M': block_m, 'BLOCK_N': block_n, 'NUM_STAGES': 2, 'NUM_TMA_MULTICAST': 1}
     smem_size = 2 * (block_m + block_n) * 128
-    return 'gemm_fp8_fp8_bf16_nt', keys, arg_defs, smem_size
+    return 'gemm_fp8_fp8_bf16_nt', keys, arg_defs, smem_size, template
 
 
 def gemm_fp8_fp8_bf16_nt(lhs: Tuple[torch.Tensor, torch.Tensor],
@@ -81,10 +104,10 @@ def gemm_fp8_fp8_bf16_nt(lhs: Tuple[torch.Tensor, torch.Tensor],
         return
 
     num_sms = get_num_sms()
-    name, keys, defs, smem_size = fp8_kernel_plan(m, n, k, num_sms)
+    name, keys, defs, smem_size, code_template = fp8_kernel_plan(m, n, k, num_sms)
     args = (lhs, lhs_scales, rhs, rhs_scales, out, m, torch.cuda.current_stream(), num_sms, smem_size,
             lhs_scales.stride(0), lhs_scales.stride(1))
     runtime = jit_tuner.compile_and_tune(name=name, keys=keys, space=(), includes=includes,
-                                         arg_defs=defs, template=template, args=args)
+                                         arg_defs=defs, template=code_template, args=args)
     rc = runtime(*args)
     assert rc == 0, f'{name} failed with HIP error {rc}'

@@ -32,3 +32,17 @@ def get_best_dense_config(m: int, n: int, k: int, num_cus: int) -> Tuple[int, in
 
 def get_best_fp8_config(m: int, n: int, k: int, num_cus: int) -> Tuple[int, int]:
     return rank_tiles(m, n, num_cus, _FP8_TILES)[0][1]
+
+
+def get_skinny_fp8_config(m: int, n: int, k: int, num_cus: int) -> int:
+    """Number of 16-row activation atoms (1, 2 or 4) when the weight-streaming kernel should run instead of the tiled
+    one, else 0: up to 64 activation rows, and enough weight rows that N/16 workgroups fill at least half the CUs."""
+    if 0 < m <= 64 and n >= 8 * num_cus:
+        return 1 if m <= 16 else (2 if m <= 32 else 4)
+    return 0
+
+
+def get_fp8_tile(m: int, n: int, k: int, num_cus: int) -> Tuple[int, int]:
+    """(BLOCK_M, BLOCK_N) of the FP8 kernel that runs: (16 * atoms, 16) for the weight-streaming kernel."""
+    atoms = get_skinny_fp8_config(m, n, k, num_cus)
+    return (16 * atoms, 16) if atoms else get_best_fp8_config(m, n, k, num_cus)

@@ -101,6 +101,7 @@ FP8_TEST_SHAPES = [
     (64, 256, 384), (512, 1024, 1024), (1, 128, 128), (63, 192, 256), (129, 320, 128), (300, 96, 640),
     (40, 192, 256), (130, 448, 640),
     (257, 2112, 1024), (128, 7168, 2048), (4096, 2048, 7168),
+    (1, 4096, 7168), (17, 4096, 1024), (33, 2112, 640), (64, 7168, 2048), (48, 4100, 384),
 ]
 
 
@@ -124,8 +125,8 @@ def prebuild_jit_kernels(num_cus: int = 256, verbose: bool = False) -> int:
     for m, n, k in FP8_TEST_SHAPES:
         if m == 0:
             continue
-        name, keys, arg_defs, _ = gemm.fp8_kernel_plan(m, n, k, num_cus)
-        code = generate(gemm.includes, arg_defs, cpp_format(gemm.template, keys))
+        name, keys, arg_defs, _, code_template = gemm.fp8_kernel_plan(m, n, k, num_cus)
+        code = generate(gemm.includes, arg_defs, cpp_format(code_template, keys))
         if (name, code) not in seen:
             seen.add((name, code))
             rt = build(name, arg_defs, code)
