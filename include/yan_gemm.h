@@ -49,7 +49,11 @@ YAN_API int yan_gemm_fp16_tn(int m, int n, int k, const void* a, const void* b, 
  *   out        bf16 [m,n] row-major
  * Requires k % 128 == 0, n % 4 == 0; m arbitrary. `num_sms` is the caller's compute-unit cap (the reference passes
  * it to its persistent kernel, yan/jit_kernels/gemm.py:26-30); this build launches one workgroup per tile and
- * accepts the argument for signature compatibility.
+ * accepts the argument for signature compatibility (the split-K decode kernel uses it to size its grid).
+ * For 33..64 activation rows and n >= 8 * CUs the split-K kernel runs: it keeps a library-owned scratch buffer
+ * (allocated with hipMalloc on first use, at most ceil(n/64) * splits * 16 KB) and a self-resetting counter per 64
+ * output columns, shared by all calls on a device: such calls must not overlap in time on one device, and the
+ * first of them cannot be captured into a HIP graph.
  * Replaces the FP8 entry the reference only sketches: template yan/jit_kernels/gemm.py:9-31, kernel
  * yan/include/gemm/fp8_gemm.cuh:40-196. */
 YAN_API int yan_gemm_fp8_fp8_bf16_nt(const void* lhs, const float* lhs_scales, long long lhs_scales_stride_m,
@@ -62,7 +66,7 @@ YAN_API int yan_gemm_fp8_fp8_bf16_nt(const void* lhs, const float* lhs_scales, l
  * (yan/jit_kernels/cute_gemm.py:41, yan/jit_kernels/gemm.py:13-16). Returns 0, or 1 for an unknown op. */
 YAN_API int yan_gemm_select_tile(int op, int m, int n, int k, int num_cus, int* block_m, int* block_n);
 
-/* "yan-gemm gfx950 <n> dense + <n> fp8 tile variants + <n> weight-streaming fp8 variants". */
+/* "yan-gemm gfx950 <n> dense + <n> fp8 tile variants + <n> weight-streaming + <n> split-K fp8 variants". */
 YAN_API const char* yan_gemm_version(void);
 
 /* The JIT boundary, for reference: signatures of `launch` in the kernel.so of each op

@@ -83,7 +83,7 @@ int yan_gemm_fp8_fp8_bf16_nt(const void* lhs, const float* lhs_scales, long long
         const int sm = int(lhs_scales_stride_m), sk = int(lhs_scales_stride_k);
         if (atoms == 1) return int(yan::launch_fp8_skinny<0, 0, 1, 8>(o, lhs, lhs_scales, sm, sk, rhs, rhs_scales, m, n, k, s));
         if (atoms == 2) return int(yan::launch_fp8_skinny<0, 0, 2, 8>(o, lhs, lhs_scales, sm, sk, rhs, rhs_scales, m, n, k, s));
-        return int(yan::launch_fp8_skinny<0, 0, 4, 8>(o, lhs, lhs_scales, sm, sk, rhs, rhs_scales, m, n, k, s));
+        return int(yan::launch_fp8_splitk<0, 0, 4, 16>(o, lhs, lhs_scales, sm, sk, rhs, rhs_scales, m, n, k, s, cus));
     }
     int bm = 0, bn = 0;
     pick(kFp8Tiles, m, n, cus, &bm, &bn);
@@ -109,6 +109,6 @@ int yan_gemm_select_tile(int op, int m, int n, int k, int num_cus, int* block_m,
     return 0;
 }
 
-const char* yan_gemm_version(void) { return "yan-gemm gfx950 6 dense + 8 fp8 tile variants + 3 weight-streaming fp8 variants"; }
+const char* yan_gemm_version(void) { return "yan-gemm gfx950 6 dense + 8 fp8 tile variants + 2 weight-streaming + 1 split-K fp8 variants"; }
 
 } // extern "C"

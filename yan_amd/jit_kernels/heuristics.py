@@ -35,8 +35,11 @@ def get_best_fp8_config(m: int, n: int, k: int, num_cus: int) -> Tuple[int, int]
 
 
 def get_skinny_fp8_config(m: int, n: int, k: int, num_cus: int) -> int:
-    """Number of 16-row activation atoms (1, 2 or 4) when the weight-streaming kernel should run instead of the tiled
-    one, else 0: up to 64 activation rows, and enough weight rows that N/16 workgroups fill at least half the CUs."""
+    """Number of 16-row activation atoms (1, 2 or 4) when one of the two decode kernels should run instead of the tiled
+    one, else 0: up to 64 activation rows, and enough weight rows that N/16 workgroups fill at least half the CUs.
+    Up to 32 rows (1 or 2 atoms) the weight-streaming kernel runs; 33..64 rows (4 atoms) go to the split-K kernel,
+    whose activations are read N/64 instead of N/16 times (measured: 15 vs 19 us warm, 25 vs 25 us cold at m = 64;
+    6.5-12 vs 8.5-12.7 us warm at m <= 32)."""
     if 0 < m <= 64 and n >= 8 * num_cus:
         return 1 if m <= 16 else (2 if m <= 32 else 4)
     return 0
