@@ -151,6 +151,32 @@ def _fp8_ref(a8, sa, b8, sb):
     return oracle.gemm_fp8_block_scaled_ref(_np(a8), sa.cpu().numpy(), _np(b8), sb.cpu().numpy())
 
 
+@pytest.mark.parametrize('m,n,k', testing.REFERENCE_DENSE_TEST_SHAPES)
+def test_fp16_entry_on_the_reference_test_shapes(m, n, k):
+    """The flow of the reference's dense test (tests/test_cute.py:9-27): fp16 randn operands, zeroed output,
+    `gemm_fp16_tn`, calc_diff < 1e-3 against torch's own fp16 `x @ y.t()`; and the bar of this build, < 1e-5 against
+    the fp32 product of the same operands."""
+    g = torch.Generator(device='cuda').manual_seed(42 + m + n + k)
+    x = torch.randn(m, k, device='cuda', dtype=torch.half, generator=g)
+    y = torch.randn(n, k, device='cuda', dtype=torch.half, generator=g)
+    out = torch.zeros(m, n, device='cuda', dtype=torch.half)
+    assert yan.gemm_fp16_tn(x, y, out) is None
+    assert float(yan.calc_diff(out, x @ y.t())) < 1e-3
+    assert float(yan.calc_diff(out.float(), x.float() @ y.float().t())) < 1e-5
+
+
+def test_fp16_kernel_answers_to_the_reference_kernel_name():
+    """tests/test_cute.py:35 times the kernel whose name contains 'fp16_gemm_cute'; the reference's package-level
+    smoke check is reachable under its name as well (yan/jit_kernels/__init__.py:2)."""
+    m, n, k = 256, 5120, 5120
+    x = torch.randn(m, k, device='cuda', dtype=torch.half)
+    y = torch.randn(n, k, device='cuda', dtype=torch.half)
+    out = torch.zeros(m, n, device='cuda', dtype=torch.half)
+    t = yan.bench_kineto(lambda: yan.gemm_fp16_tn(x, y, out), 'fp16_gemm_cute', suppress_kineto_output=True)
+    assert 0 < t < 1e-3
+    assert yan.jit_kernels.cute_gemm_accuracy_test is yan.jit_kernels.bf16_gemm_accuracy_test
+
+
 @pytest.mark.parametrize('m,n,k', [s for s in testing.FP8_TEST_SHAPES if s[0] * s[1] * s[2] <= 7e10])
 @pytest.mark.parametrize('col_major', [False, True])
 def test_fp8_parity_vs_oracle(m, n, k, col_major):

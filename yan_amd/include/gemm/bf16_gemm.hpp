@@ -41,8 +41,8 @@ struct DenseTileConfig {
 };
 
 template <typename Atom, typename Elem, int BLOCK_M, int BLOCK_N>
-__global__ void __launch_bounds__(4 * kWaveSize)
-dense_gemm_mfma(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, Elem* __restrict__ C,
+__device__ __forceinline__ void
+dense_gemm_body(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, Elem* __restrict__ C,
                 int m, int n, int k) {
     using Cfg = DenseTileConfig<BLOCK_M, BLOCK_N>;
     constexpr int NW = Cfg::NUM_WAVES, TN = Cfg::WTN / 32, TM = Cfg::WTM / 32;
@@ -187,6 +187,20 @@ dense_gemm_mfma(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, El
     }
 }
 
+template <typename Atom, typename Elem, int BLOCK_M, int BLOCK_N>
+__global__ void __launch_bounds__(4 * kWaveSize)
+dense_gemm_mfma(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, Elem* __restrict__ C, int m, int n, int k) {
+    dense_gemm_body<Atom, Elem, BLOCK_M, BLOCK_N>(A, B, C, m, n, k);
+}
+
+// The fp16 flavour under the name of the reference's kernel (yan/include/gemm/cute_gemm.cuh:20), so that profiler
+// filters written for it (tests/test_cute.py:35 looks for 'fp16_gemm_cute') keep finding it.
+template <int BLOCK_M, int BLOCK_N>
+__global__ void __launch_bounds__(4 * kWaveSize)
+fp16_gemm_cute(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, _Float16* __restrict__ C, int m, int n, int k) {
+    dense_gemm_body<MfmaF16_32x32x16, _Float16, BLOCK_M, BLOCK_N>(A, B, C, m, n, k);
+}
+
 // Arguments every dense launcher checks before touching the GPU. Returns hipSuccess or hipErrorInvalidValue.
 inline hipError_t check_dense_args(int m, int n, int k, const void* a, const void* b, const void* c,
                                    int block_m, int block_n) {
@@ -204,9 +218,14 @@ inline hipError_t launch_dense(int m, int n, int k, const void* a, const void* b
     if (hipError_t e = check_dense_args(m, n, k, a, b, c, BLOCK_M, BLOCK_N); e != hipSuccess) return e;
     using Cfg = DenseTileConfig<BLOCK_M, BLOCK_N>;
     const XcdTileScheduler<> sched(m, n, BLOCK_M, BLOCK_N);
-    hipLaunchKernelGGL((dense_gemm_mfma<Atom, Elem, BLOCK_M, BLOCK_N>), dim3(sched.grid_size()),
-                       dim3(Cfg::NUM_WAVES * kWaveSize), 0, stream, static_cast<const uint8_t*>(a),
-                       static_cast<const uint8_t*>(b), static_cast<Elem*>(c), m, n, k);
+    if constexpr (__is_same(Elem, _Float16))
+        hipLaunchKernelGGL((fp16_gemm_cute<BLOCK_M, BLOCK_N>), dim3(sched.grid_size()),
+                           dim3(Cfg::NUM_WAVES * kWaveSize), 0, stream, static_cast<const uint8_t*>(a),
+                           static_cast<const uint8_t*>(b), static_cast<Elem*>(c), m, n, k);
+    else
+        hipLaunchKernelGGL((dense_gemm_mfma<Atom, Elem, BLOCK_M, BLOCK_N>), dim3(sched.grid_size()),
+                           dim3(Cfg::NUM_WAVES * kWaveSize), 0, stream, static_cast<const uint8_t*>(a),
+                           static_cast<const uint8_t*>(b), static_cast<Elem*>(c), m, n, k);
     return hipGetLastError();
 }
 

@@ -96,6 +96,9 @@ DENSE_TEST_SHAPES = [
     (300, 256, 256), (33, 132, 72), (96, 80, 136),
     (256, 5120, 5120), (4096, 2048, 7168), (4096, 7168, 2048), (256, 24576, 1536),
 ]
+# (m, n, k) of the reference's own dense test (tests/test_cute.py:21-22: m in (256, 4096) x six (k, n) pairs)
+REFERENCE_DENSE_TEST_SHAPES = [(m, n, k) for m in (256, 4096)
+                               for k, n in ((5120, 5120), (1536, 24576), (512, 32768), (16384, 7168), (7168, 2048), (2048, 7168))]
 FP8_TEST_SHAPES = [
     (4096, 7168, 7168), (64, 4096, 7168), (16384, 16384, 16384),
     (64, 256, 384), (512, 1024, 1024), (1, 128, 128), (63, 192, 256), (129, 320, 128), (300, 96, 640),
@@ -111,7 +114,7 @@ def prebuild_jit_kernels(num_cus: int = 256, verbose: bool = False) -> int:
     from .jit import build, cpp_format, generate
     from .jit_kernels import bf16_gemm, gemm
     seen = set()
-    for m, n, k in DENSE_TEST_SHAPES:
+    for m, n, k in DENSE_TEST_SHAPES + REFERENCE_DENSE_TEST_SHAPES:
         for dtype in (torch.bfloat16, torch.half):
             if m == 0 or n == 0:
                 continue
