@@ -60,7 +60,30 @@ YAN_API int yan_gemm_fp8_fp8_bf16_nt(const void* lhs, const float* lhs_scales, l
                              long long lhs_scales_stride_k, const void* rhs, const float* rhs_scales, void* out,
                              int m, int n, int k, void* stream, int num_sms);
 
-/* Macro tile the library uses for a problem: op 0 = dense 16-bit, 1 = FP8 block-scaled. Writes BLOCK_M / BLOCK_N.
+/* Grouped (mixture-of-experts) forms of the FP8 GEMM: group g has its own weights rhs[g] ([n,k] e4m3) and scale table
+ * rhs_scales[g] ([ceil(n/128)][k/128]); both arrays are contiguous over g. Arithmetic per row as above.
+ * They fill in the reference's GemmType::GroupedContiguous / GroupedMasked and `int* grouped_layout` hooks
+ * (yan/include/gemm/scheduler.cuh:7-11,31-48, yan/include/gemm/fp8_gemm.cuh:41), for which it has no entry point.
+ *
+ * contiguous: lhs [m,k] holds the rows of all groups one after the other, every group padded to a multiple of 128 rows
+ *   (get_m_alignment_for_contiguous_layout, yan/jit_kernels/utils.py:46-55), so m % 128 == 0; m_indices[i] (device,
+ *   int32 [m]) is the group of row i, constant over each aligned block of 128 rows; a negative value marks a block of
+ *   padding rows, whose rows of `out` are not written. */
+YAN_API int yan_m_grouped_gemm_fp8_fp8_bf16_nt_contiguous(const void* lhs, const float* lhs_scales, long long lhs_scales_stride_m,
+                                                  long long lhs_scales_stride_k, const void* rhs, const float* rhs_scales,
+                                                  void* out, const int* m_indices, int num_groups, int m, int n, int k,
+                                                  void* stream, int num_sms);
+
+/* masked: lhs [num_groups][m_max][k], out [num_groups][m_max][n], both contiguous; scale (g,i,kb) of lhs at
+ *   lhs_scales[g*stride_g + i*stride_m + kb*stride_k]; masked_m (device, int32 [num_groups]) says how many leading rows
+ *   of each group are valid; the other rows of `out` are not written. expected_m > 0 is a hint for the tile choice. */
+YAN_API int yan_m_grouped_gemm_fp8_fp8_bf16_nt_masked(const void* lhs, const float* lhs_scales, long long lhs_scales_stride_g,
+                                              long long lhs_scales_stride_m, long long lhs_scales_stride_k, const void* rhs,
+                                              const float* rhs_scales, void* out, const int* masked_m, int num_groups,
+                                              int m_max, int expected_m, int n, int k, void* stream, int num_sms);
+
+/* Macro tile the library uses for a problem: op 0 = dense 16-bit, 1 = FP8 block-scaled, 2 = FP8 grouped contiguous
+ * (m = total rows). Writes BLOCK_M / BLOCK_N.
  * For op 1 with few activation rows the answer is (16 * atoms, 16): the weight-streaming kernel.
  * Host-only (no device call). Stands where the reference leaves tile choice to the caller's keys
  * (yan/jit_kernels/cute_gemm.py:41, yan/jit_kernels/gemm.py:13-16). Returns 0, or 1 for an unknown op. */

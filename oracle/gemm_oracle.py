@@ -8,6 +8,11 @@ What each function restates (paths relative to the reference tree):
                              yan/include/gemm/fp8_gemm.cuh:48-61        one A scale per row per 128-K, one B scale per
                                                                        128x128 block; the reference has no executable FP8
                                                                        path, so the closed form is the oracle
+  m_grouped_gemm_contiguous_ref,
+  m_grouped_gemm_masked_ref  yan/include/gemm/scheduler.cuh:7-11,31-48, yan/include/gemm/fp8_gemm.cuh:41 (the GemmType
+                             enumerators and grouped_layout hook; the reference has no grouped entry point and no test):
+                             gemm_fp8_block_scaled_ref applied per group, row by row -- the row's group picks the weight
+                             matrix; rows with a negative index / beyond masked_m keep the caller's values
   e4m3fn_decode / encode     OCP FP8 E4M3 (the dtype named in yan/jit/template.py:18): 1-4-3, bias 7, no inf, S.1111.111 NaN
   per_token_cast_to_fp8,
   per_block_cast_to_fp8      harness-side quantisers of the benchmark configs (amax over 1x128 / 128x128 groups,
@@ -16,13 +21,16 @@ What each function restates (paths relative to the reference tree):
 Pinned by tests/test_oracle.py: closed forms (identity, ones pattern of cute_gemm.py:74-79, unit and power-of-two
 scales giving exact integer results, single-K-block scale isolation), the independent C triple loop in
 gemm_oracle.c, brute force on tiny inputs, the 256-entry e4m3 table against torch's CPU cast, and the committed
-fixtures under tests/golden/. The reference holds no golden vectors for this path.
+fixtures under tests/golden/. The reference holds no golden vectors for this path. The grouped forms are pinned
+against a row-by-row brute force (every row multiplied with the weight matrix its index names, one row at a time),
+against the plain form for a single group, and by permuting the groups.
 """
 import numpy as np
 
 __all__ = ['calc_diff', 'e4m3fn_decode_table', 'e4m3fn_decode', 'e4m3fn_encode', 'bf16_bits_to_f32', 'f32_to_bf16_bits',
            'bf16_round', 'per_token_cast_to_fp8', 'per_block_cast_to_fp8', 'dequant_lhs', 'dequant_rhs',
-           'gemm_bf16_tn_ref', 'gemm_fp8_block_scaled_ref', 'gemm_fp8_blockwise_f32']
+           'gemm_bf16_tn_ref', 'gemm_fp8_block_scaled_ref', 'gemm_fp8_blockwise_f32',
+           'm_grouped_gemm_contiguous_ref', 'm_grouped_gemm_masked_ref']
 
 FP8_MAX = 448.0
 
@@ -150,3 +158,30 @@ def gemm_fp8_blockwise_f32(lhs, lhs_scales, rhs, rhs_scales) -> np.ndarray:
         part = a[:, kb * 128:(kb + 1) * 128] @ b[:, kb * 128:(kb + 1) * 128].T
         acc += part * (sa[:, kb][:, None] * sb[:, kb][None, :])
     return acc
+
+
+def m_grouped_gemm_contiguous_ref(lhs, lhs_scales, rhs, rhs_scales, m_indices, out_init=None, dtype=np.float32) -> np.ndarray:
+    """lhs [m, k] codes, lhs_scales [m, k/128]; rhs [G, n, k] codes, rhs_scales [G, ceil(n/128), k/128];
+    m_indices [m] ints: out[i] = row i of the block-scaled product with group m_indices[i]'s weights; rows with a
+    negative index keep `out_init` (zeros if not given)."""
+    lhs, rhs, m_indices = np.asarray(lhs), np.asarray(rhs), np.asarray(m_indices)
+    m, n = lhs.shape[0], rhs.shape[1]
+    out = np.zeros((m, n), dtype=dtype) if out_init is None else np.array(out_init, dtype=dtype)
+    for g in range(rhs.shape[0]):
+        rows = np.nonzero(m_indices == g)[0]
+        if rows.size:
+            out[rows] = gemm_fp8_block_scaled_ref(lhs[rows], np.asarray(lhs_scales)[rows], rhs[g], np.asarray(rhs_scales)[g], dtype)
+    return out
+
+
+def m_grouped_gemm_masked_ref(lhs, lhs_scales, rhs, rhs_scales, masked_m, out_init=None, dtype=np.float32) -> np.ndarray:
+    """lhs [G, m_max, k], lhs_scales [G, m_max, k/128], rhs [G, n, k], rhs_scales [G, ceil(n/128), k/128], masked_m [G]:
+    out[g, :masked_m[g]] = block-scaled product of group g's first masked_m[g] rows; other rows keep `out_init`."""
+    lhs, rhs = np.asarray(lhs), np.asarray(rhs)
+    G, m_max, n = lhs.shape[0], lhs.shape[1], rhs.shape[1]
+    out = np.zeros((G, m_max, n), dtype=dtype) if out_init is None else np.array(out_init, dtype=dtype)
+    for g in range(G):
+        r = int(min(max(int(np.asarray(masked_m)[g]), 0), m_max))
+        if r:
+            out[g, :r] = gemm_fp8_block_scaled_ref(lhs[g, :r], np.asarray(lhs_scales)[g, :r], rhs[g], np.asarray(rhs_scales)[g], dtype)
+    return out

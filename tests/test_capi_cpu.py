@@ -23,7 +23,7 @@ def _declared(repo_root):
 
 def test_library_exports_every_declared_symbol(lib, repo_root):
     declared = _declared(repo_root)
-    assert declared == sorted(capi.SYMBOLS) and len(declared) == 5
+    assert declared == sorted(capi.SYMBOLS) and len(declared) == 7
     for name in declared:
         assert hasattr(lib, name), name
     out = subprocess.check_output(['nm', '-D', '--defined-only', os.path.join(repo_root, 'yan_amd', 'csrc', 'libyan_gemm.so')], text=True)
@@ -46,6 +46,9 @@ def test_version_and_tile_selection_match_python(lib):
         for cus in (256, 128, 80):
             assert capi.select_tile(0, m, n, k, cus) == heuristics.get_best_dense_config(m, n, k, cus), (m, n, k, cus)
             assert capi.select_tile(1, m, n, k, cus) == heuristics.get_fp8_tile(m, n, k, cus), (m, n, k, cus)
+    for m, n in [(4096, 4096), (32768, 4096), (128, 7168), (256, 200), (1024, 24576)]:
+        for cus in (256, 80):
+            assert capi.select_tile(2, m, n, 1024, cus) == heuristics.get_best_grouped_fp8_config(m, n, 1024, cus, 1, 128)
     bm, bn = ctypes.c_int(), ctypes.c_int()
     assert lib.yan_gemm_select_tile(7, 1, 1, 1, 256, ctypes.byref(bm), ctypes.byref(bn)) == 1
     assert lib.yan_gemm_select_tile(0, 1, 1, 1, 0, ctypes.byref(bm), ctypes.byref(bn)) == 1
@@ -63,3 +66,13 @@ def test_compute_entry_points_validate_before_touching_a_device(lib):
     assert lib.yan_gemm_fp8_fp8_bf16_nt(null, null, 1, 1, null, null, null, 4, 128, 64, null, 256) != 0    # k % 128
     assert lib.yan_gemm_fp8_fp8_bf16_nt(null, null, 1, 1, null, null, null, 4, 126, 128, null, 256) != 0   # n % 4
     assert lib.yan_gemm_fp8_fp8_bf16_nt(null, null, 1, 1, null, null, null, 4, 128, 128, null, 256) != 0   # null operands
+    grouped_c, grouped_m = lib.yan_m_grouped_gemm_fp8_fp8_bf16_nt_contiguous, lib.yan_m_grouped_gemm_fp8_fp8_bf16_nt_masked
+    assert grouped_c(null, null, 1, 1, null, null, null, null, 2, 0, 128, 128, null, 256) == 0             # no rows
+    assert grouped_c(null, null, 1, 1, null, null, null, null, 2, 100, 128, 128, null, 256) != 0           # m % 128
+    assert grouped_c(null, null, 1, 1, null, null, null, null, 2, 128, 128, 64, null, 256) != 0            # k % 128
+    assert grouped_c(null, null, 1, 1, null, null, null, null, 0, 128, 128, 128, null, 256) != 0           # no groups
+    assert grouped_c(null, null, 1, 1, null, null, null, null, 2, 128, 128, 128, null, 256) != 0           # null operands
+    assert grouped_m(null, null, 1, 1, 1, null, null, null, null, 0, 64, 64, 128, 128, null, 256) == 0     # no groups
+    assert grouped_m(null, null, 1, 1, 1, null, null, null, null, 2, 64, 0, 128, 128, null, 256) != 0      # expected_m
+    assert grouped_m(null, null, 1, 1, 1, null, null, null, null, 2, 64, 64, 126, 128, null, 256) != 0     # n % 4
+    assert grouped_m(null, null, 1, 1, 1, null, null, null, null, 2, 64, 64, 128, 128, null, 256) != 0     # null operands

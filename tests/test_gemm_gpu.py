@@ -16,7 +16,7 @@ import torch
 
 import oracle
 import yan_amd as yan
-from yan_amd import jit, testing
+from yan_amd import capi, jit, testing
 
 pytestmark = pytest.mark.gpu
 
@@ -309,6 +309,82 @@ def test_fp8_outlier_16384_cubed():
 
 
 # ----------------------------------------------------------------------------- the ahead-of-time C-ABI library
+# ----------------------------------------------------------------------------- grouped FP8 GEMMs
+def _np_codes(t):
+    return t.view(torch.uint8).cpu().numpy()
+
+
+@pytest.mark.parametrize('rows,n,k,pad_blocks', testing.GROUPED_CONTIGUOUS_TEST_CASES)
+def test_grouped_contiguous_parity(rows, n, k, pad_blocks):
+    """Contiguous layout against the oracle (per-group block-scaled product, same seeded inputs generated on the
+    CPU); rows of padding blocks (index -1) keep the caller's values; the C-ABI library gives the same bits as the
+    JIT kernel; a single group gives the bits of the plain GEMM."""
+    (a8, sa), (b8, sb), out, idx = testing.make_grouped_contiguous_case(rows, n, k, seed=5, padding_blocks=pad_blocks)
+    m = a8.size(0)
+    a8d, sad, b8d, sbd, idxd = a8.cuda(), sa.cuda(), b8.cuda(), sb.cuda(), idx.cuda()
+    got = out.cuda()
+    assert yan.m_grouped_gemm_fp8_fp8_bf16_nt_contiguous((a8d, sad), (b8d, sbd), got, idxd) is None
+    if m * n * k <= 2e10:
+        ref = oracle.m_grouped_gemm_contiguous_ref(_np_codes(a8), sa.numpy(), _np_codes(b8), sb.numpy(), idx.numpy(),
+                                                   out_init=out.float().numpy())
+        ref = torch.from_numpy(ref)
+    else:       # the per-group product on the device in fp32, rows of the oracle sampled below
+        ref = out.float()
+        for g in range(len(rows)):
+            sel = (idx == g).nonzero().flatten()
+            ref[sel] = (testing.dequant_lhs(a8d[sel.cuda()], sad[sel.cuda()]) @ testing.dequant_rhs(b8d[g], sbd[g]).t()).cpu()
+        pick = torch.arange(0, m, 97)
+        want = oracle.m_grouped_gemm_contiguous_ref(_np_codes(a8[pick]), sa[pick].numpy(), _np_codes(b8), sb.numpy(), idx[pick].numpy())
+        assert oracle.calc_diff(got[pick.cuda()].float().cpu().numpy(), want) < 1e-3
+    assert float(yan.calc_diff(got.float().cpu(), ref)) < 1e-3
+    real = idx >= 0
+    assert torch.equal(got.cpu()[~real], out[~real])                      # padding blocks untouched
+    bound = ref.abs() * 2.0 ** -7 + 1e-4 * ref.abs().max()
+    assert bool(((got.float().cpu() - ref).abs() <= bound)[real].all())
+    via_lib = out.cuda()
+    assert capi.m_grouped_gemm_fp8_fp8_bf16_nt_contiguous((a8d, sad), (b8d, sbd), via_lib, idxd) == 0
+    assert torch.equal(via_lib, got)
+    # scales handed over token-contiguous give the same bits
+    again = out.cuda()
+    yan.m_grouped_gemm_fp8_fp8_bf16_nt_contiguous((a8d, yan.get_col_major_tensor(sad)), (b8d, sbd), again, idxd)
+    assert torch.equal(again, got)
+    # the first group's rows through the plain entry point
+    r0 = (rows[0] + 127) // 128 * 128
+    plain = torch.zeros(r0, n, dtype=torch.bfloat16, device='cuda')
+    yan.gemm_fp8_fp8_bf16_nt((a8d[:r0], sad[:r0].contiguous()), (b8d[0], sbd[0]), plain)
+    assert float(yan.calc_diff(plain.float(), got[:r0].float())) < 1e-9
+
+
+@pytest.mark.parametrize('groups,m_max,n,k,masked,expected_m', testing.GROUPED_MASKED_TEST_CASES)
+def test_grouped_masked_parity(groups, m_max, n, k, masked, expected_m):
+    """Masked layout against the oracle; rows at and beyond masked_m keep the caller's values; library == JIT."""
+    (a8, sa), (b8, sb), out, mm = testing.make_grouped_masked_case(groups, m_max, n, k, masked, seed=6)
+    a8d, sad, b8d, sbd, mmd = a8.cuda(), sa.cuda(), b8.cuda(), sb.cuda(), mm.cuda()
+    got = out.cuda()
+    assert yan.m_grouped_gemm_fp8_fp8_bf16_nt_masked((a8d, sad), (b8d, sbd), got, mmd, expected_m) is None
+    if groups * m_max * n * k <= 2e10:
+        ref = torch.from_numpy(oracle.m_grouped_gemm_masked_ref(_np_codes(a8), sa.numpy(), _np_codes(b8), sb.numpy(), mm.numpy(),
+                                                                out_init=out.float().numpy()))
+    else:
+        ref = out.float()
+        for g in range(groups):
+            r = masked[g]
+            ref[g, :r] = (testing.dequant_lhs(a8d[g, :r], sad[g, :r]) @ testing.dequant_rhs(b8d[g], sbd[g]).t()).cpu()
+        g, r = 1, min(masked[1], 16)
+        want = oracle.gemm_fp8_block_scaled_ref(_np_codes(a8[g, :r]), sa[g, :r].numpy(), _np_codes(b8[g]), sb[g].numpy())
+        assert oracle.calc_diff(got[g, :r].float().cpu().numpy(), want) < 1e-3
+    assert float(yan.calc_diff(got.float().cpu(), ref)) < 1e-3
+    for g in range(groups):
+        assert torch.equal(got[g, masked[g]:].cpu(), out[g, masked[g]:])  # masked-out rows untouched
+        r = masked[g]
+        if r:
+            refg = ref[g, :r]
+            assert bool(((got[g, :r].float().cpu() - refg).abs() <= refg.abs() * 2.0 ** -7 + 1e-4 * refg.abs().max()).all())
+    via_lib = out.cuda()
+    assert capi.m_grouped_gemm_fp8_fp8_bf16_nt_masked((a8d, sad), (b8d, sbd), via_lib, mmd, expected_m) == 0
+    assert torch.equal(via_lib, got)
+
+
 @pytest.mark.parametrize('m,n,k', [(1024, 1024, 1024), (255, 132, 72), (33, 4, 200), (257, 1028, 1096)])
 def test_capi_dense_matches_oracle_and_jit(m, n, k):
     from yan_amd import capi

@@ -236,6 +236,51 @@ def test_fp8_three_evaluations_agree_on_random_data_and_track_the_unquantised_pr
 
 
 # ----------------------------------------------------------------------------- committed fixtures
+def test_grouped_forms_against_row_by_row_brute_force():
+    """The grouped oracles are the plain one applied per group. Pinned by: the C triple loop on every row taken alone
+    with the weight matrix its index names (small-integer data and power-of-two scales, so everything is exact);
+    one group == the plain form; relabelling the groups together with their weights changes nothing; rows that are
+    padding (negative index) or beyond masked_m keep what the caller had there."""
+    rng = np.random.default_rng(21)
+    G, n, k = 3, 136, 256
+    qb = np.stack([_small_int_codes(rng, (n, k))[0] for _ in range(G)])
+    sb = 2.0 ** rng.integers(-2, 3, size=(G, 2, k // 128)).astype(np.float32)
+    m = 24
+    qa, _ = _small_int_codes(rng, (m, k))
+    sa = 2.0 ** rng.integers(-2, 3, size=(m, k // 128)).astype(np.float32)
+    idx = np.array([0] * 8 + [2] * 8 + [-1] * 4 + [1] * 4, dtype=np.int32)
+    init = rng.standard_normal((m, n)).astype(np.float32)
+    got = oracle.m_grouped_gemm_contiguous_ref(qa, sa, qb, sb, idx, out_init=init)
+    for i in range(m):
+        if idx[i] < 0:
+            assert np.array_equal(got[i], init[i])
+        else:
+            want = c_oracle.gemm_fp8_nt(qa[i:i + 1], sa[i:i + 1], qb[idx[i]], sb[idx[i]])
+            assert np.array_equal(got[i:i + 1], want)
+    # one group: the plain form
+    one = oracle.m_grouped_gemm_contiguous_ref(qa, sa, qb[1:2], sb[1:2], np.zeros(m, np.int32))
+    assert np.array_equal(one, oracle.gemm_fp8_block_scaled_ref(qa, sa, qb[1], sb[1]))
+    # relabel groups 0 <-> 2 and swap their weights: same answer; swap only the labels: different answer
+    perm = np.array([2, 1, 0])
+    relabeled = np.where(idx >= 0, perm[np.maximum(idx, 0)], idx).astype(np.int32)
+    assert np.array_equal(oracle.m_grouped_gemm_contiguous_ref(qa, sa, qb[perm], sb[perm], relabeled, out_init=init), got)
+    assert not np.array_equal(oracle.m_grouped_gemm_contiguous_ref(qa, sa, qb, sb, relabeled, out_init=init), got)
+
+    # masked layout
+    m_max = 10
+    qa3 = np.stack([_small_int_codes(rng, (m_max, k))[0] for _ in range(G)])
+    sa3 = 2.0 ** rng.integers(-2, 3, size=(G, m_max, k // 128)).astype(np.float32)
+    masked = np.array([10, 0, 3], dtype=np.int32)
+    init3 = rng.standard_normal((G, m_max, n)).astype(np.float32)
+    got3 = oracle.m_grouped_gemm_masked_ref(qa3, sa3, qb, sb, masked, out_init=init3)
+    for g in range(G):
+        for i in range(m_max):
+            if i >= masked[g]:
+                assert np.array_equal(got3[g, i], init3[g, i])
+            else:
+                assert np.array_equal(got3[g, i:i + 1], c_oracle.gemm_fp8_nt(qa3[g, i:i + 1], sa3[g, i:i + 1], qb[g], sb[g]))
+
+
 def test_golden_fixtures_reproduce(repo_root):
     import os
     path = os.path.join(repo_root, 'tests', 'golden', 'gemm_small.npz')

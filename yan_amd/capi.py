@@ -8,7 +8,8 @@ import torch
 _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), 'csrc', 'libyan_gemm.so')
 _lib = None
 
-SYMBOLS = ('yan_gemm_bf16_tn', 'yan_gemm_fp16_tn', 'yan_gemm_fp8_fp8_bf16_nt', 'yan_gemm_select_tile', 'yan_gemm_version')
+SYMBOLS = ('yan_gemm_bf16_tn', 'yan_gemm_fp16_tn', 'yan_gemm_fp8_fp8_bf16_nt', 'yan_m_grouped_gemm_fp8_fp8_bf16_nt_contiguous',
+           'yan_m_grouped_gemm_fp8_fp8_bf16_nt_masked', 'yan_gemm_select_tile', 'yan_gemm_version')
 
 
 def load() -> ctypes.CDLL:
@@ -21,7 +22,9 @@ def load() -> ctypes.CDLL:
         lib.yan_gemm_bf16_tn.argtypes = lib.yan_gemm_fp16_tn.argtypes = [ci, ci, ci, vp, vp, vp, vp]
         lib.yan_gemm_fp8_fp8_bf16_nt.argtypes = [vp, vp, ll, ll, vp, vp, vp, ci, ci, ci, vp, ci]
         lib.yan_gemm_select_tile.argtypes = [ci, ci, ci, ci, ci, ctypes.POINTER(ci), ctypes.POINTER(ci)]
-        for name in SYMBOLS[:4]:
+        lib.yan_m_grouped_gemm_fp8_fp8_bf16_nt_contiguous.argtypes = [vp, vp, ll, ll, vp, vp, vp, vp, ci, ci, ci, ci, vp, ci]
+        lib.yan_m_grouped_gemm_fp8_fp8_bf16_nt_masked.argtypes = [vp, vp, ll, ll, ll, vp, vp, vp, vp, ci, ci, ci, ci, ci, vp, ci]
+        for name in SYMBOLS[:-1]:
             getattr(lib, name).restype = ci
         lib.yan_gemm_version.restype = ctypes.c_char_p
         _lib = lib
@@ -47,6 +50,23 @@ def gemm_fp8_fp8_bf16_nt(lhs, rhs, out: torch.Tensor, num_sms: int = 0) -> int:
     (m, k), n = a8.shape, b8.shape[0]
     return load().yan_gemm_fp8_fp8_bf16_nt(a8.data_ptr(), sa.data_ptr(), sa.stride(0), sa.stride(1), b8.data_ptr(),
                                            sb.data_ptr(), out.data_ptr(), m, n, k, _stream_handle(), num_sms)
+
+
+def m_grouped_gemm_fp8_fp8_bf16_nt_contiguous(lhs, rhs, out: torch.Tensor, m_indices: torch.Tensor, num_sms: int = 0) -> int:
+    (a8, sa), (b8, sb) = lhs, rhs
+    (m, k), (groups, n, _) = a8.shape, b8.shape
+    return load().yan_m_grouped_gemm_fp8_fp8_bf16_nt_contiguous(
+        a8.data_ptr(), sa.data_ptr(), sa.stride(0), sa.stride(1), b8.data_ptr(), sb.data_ptr(), out.data_ptr(),
+        m_indices.data_ptr(), groups, m, n, k, _stream_handle(), num_sms)
+
+
+def m_grouped_gemm_fp8_fp8_bf16_nt_masked(lhs, rhs, out: torch.Tensor, masked_m: torch.Tensor, expected_m: int,
+                                          num_sms: int = 0) -> int:
+    (a8, sa), (b8, sb) = lhs, rhs
+    (groups, m_max, k), n = a8.shape, b8.shape[1]
+    return load().yan_m_grouped_gemm_fp8_fp8_bf16_nt_masked(
+        a8.data_ptr(), sa.data_ptr(), sa.stride(0), sa.stride(1), sa.stride(2), b8.data_ptr(), sb.data_ptr(),
+        out.data_ptr(), masked_m.data_ptr(), groups, m_max, expected_m, n, k, _stream_handle(), num_sms)
 
 
 def select_tile(op: int, m: int, n: int, k: int, num_cus: int):

@@ -27,6 +27,20 @@ void pick(const TileCost (&tiles)[COUNT], int m, int n, int num_cus, int* bm, in
     }
 }
 
+// Tile of a grouped FP8 GEMM (get_best_grouped_fp8_config in heuristics.py): tiles at least 64 wide, BLOCK_M dividing
+// `m_alignment` when that is non-zero, tile count multiplied by `groups`.
+void pick_grouped(int m, int n, int num_cus, int groups, int m_alignment, int* bm, int* bn) {
+    double best = -1;
+    if (m < 1) m = 1;
+    for (const TileCost& t : kFp8Tiles) {
+        if (t.bn < 64 || (m_alignment && m_alignment % t.bm != 0)) continue;
+        const long long count  = (long long)((m + t.bm - 1) / t.bm) * ((n + t.bn - 1) / t.bn) * groups;
+        const long long rounds = (count + num_cus - 1) / num_cus;
+        const double cost = double(rounds) * t.bm * t.bn * t.per_area;
+        if (best < 0 || cost < best || (cost == best && (t.bm < *bm || (t.bm == *bm && t.bn < *bn)))) { best = cost; *bm = t.bm; *bn = t.bn; }
+    }
+}
+
 // Activation atoms of the weight-streaming kernel, or 0 for the tiled kernel (get_skinny_fp8_config in heuristics.py).
 int skinny_atoms(int m, int n, int num_cus) {
     if (m > 0 && m <= 64 && n >= 8 * num_cus) return m <= 16 ? 1 : (m <= 32 ? 2 : 4);
@@ -97,6 +111,50 @@ int yan_gemm_fp8_fp8_bf16_nt(const void* lhs, const float* lhs_scales, long long
     return int(hipErrorInvalidValue);
 }
 
+int yan_m_grouped_gemm_fp8_fp8_bf16_nt_contiguous(const void* lhs, const float* lhs_scales, long long lhs_scales_stride_m,
+                                                  long long lhs_scales_stride_k, const void* rhs, const float* rhs_scales,
+                                                  void* out, const int* m_indices, int num_groups, int m, int n, int k,
+                                                  void* stream, int num_sms) {
+    if (m == 0 || n == 0) return 0;
+    if (m < 0 || n < 0 || k <= 0 || num_groups <= 0 || (m % 128) != 0) return int(hipErrorInvalidValue);
+    const long long last = (long long)(m - 1) * lhs_scales_stride_m + (long long)(k / 128 - 1) * lhs_scales_stride_k;
+    if (lhs_scales_stride_m < 0 || lhs_scales_stride_k < 0 || last >= (1ll << 28)) return int(hipErrorInvalidValue);
+    const int cus = num_sms > 0 ? num_sms : device_cus();
+    int bm = 0, bn = 0;
+    pick_grouped(m, n, cus, 1, 128, &bm, &bn);
+#define YAN_GROUPED_CASE(BM, BN)                                                                                     \
+    if (bm == BM && bn == BN)                                                                                        \
+        return int(yan::Gemm<0, 0, BM, BN, 128, 1, 2, 1, yan::GemmType::GroupedContiguous>::run_grouped(             \
+            static_cast<__hip_bfloat16*>(out), lhs, lhs_scales, int(lhs_scales_stride_m), int(lhs_scales_stride_k), 0, rhs, \
+            rhs_scales, m_indices, num_groups, m, n, k, static_cast<hipStream_t>(stream)));
+    YAN_GROUPED_CASE(128, 256) YAN_GROUPED_CASE(128, 128) YAN_GROUPED_CASE(64, 128) YAN_GROUPED_CASE(64, 64)
+#undef YAN_GROUPED_CASE
+    return int(hipErrorInvalidValue);
+}
+
+int yan_m_grouped_gemm_fp8_fp8_bf16_nt_masked(const void* lhs, const float* lhs_scales, long long lhs_scales_stride_g,
+                                              long long lhs_scales_stride_m, long long lhs_scales_stride_k, const void* rhs,
+                                              const float* rhs_scales, void* out, const int* masked_m, int num_groups,
+                                              int m_max, int expected_m, int n, int k, void* stream, int num_sms) {
+    if (m_max == 0 || n == 0 || num_groups == 0) return 0;
+    if (m_max < 0 || n < 0 || k <= 0 || num_groups < 0 || expected_m <= 0) return int(hipErrorInvalidValue);
+    const long long last = (long long)(m_max - 1) * lhs_scales_stride_m + (long long)(k / 128 - 1) * lhs_scales_stride_k;
+    if (lhs_scales_stride_m < 0 || lhs_scales_stride_k < 0 || lhs_scales_stride_g < 0 || last >= (1ll << 28) ||
+        lhs_scales_stride_g >= (1ll << 31)) return int(hipErrorInvalidValue);
+    const int cus = num_sms > 0 ? num_sms : device_cus();
+    int bm = 0, bn = 0;
+    pick_grouped(expected_m < m_max ? expected_m : m_max, n, cus, num_groups, 0, &bm, &bn);
+#define YAN_GROUPED_CASE(BM, BN)                                                                                     \
+    if (bm == BM && bn == BN)                                                                                        \
+        return int(yan::Gemm<0, 0, BM, BN, 128, 1, 2, 1, yan::GemmType::GroupedMasked>::run_grouped(                 \
+            static_cast<__hip_bfloat16*>(out), lhs, lhs_scales, int(lhs_scales_stride_m), int(lhs_scales_stride_k),  \
+            int(lhs_scales_stride_g), rhs, rhs_scales, masked_m, num_groups, m_max, n, k, static_cast<hipStream_t>(stream)));
+    YAN_GROUPED_CASE(256, 256) YAN_GROUPED_CASE(256, 128) YAN_GROUPED_CASE(128, 256) YAN_GROUPED_CASE(128, 128)
+    YAN_GROUPED_CASE(64, 128) YAN_GROUPED_CASE(64, 64)
+#undef YAN_GROUPED_CASE
+    return int(hipErrorInvalidValue);
+}
+
 int yan_gemm_select_tile(int op, int m, int n, int k, int num_cus, int* block_m, int* block_n) {
     (void)k;
     if (!block_m || !block_n || num_cus <= 0) return 1;
@@ -105,10 +163,11 @@ int yan_gemm_select_tile(int op, int m, int n, int k, int num_cus, int* block_m,
         if (const int atoms = skinny_atoms(m, n, num_cus)) { *block_m = 16 * atoms; *block_n = 16; }
         else pick(kFp8Tiles, m, n, num_cus, block_m, block_n);
     }
+    else if (op == 2) pick_grouped(m, n, num_cus, 1, 128, block_m, block_n);
     else return 1;
     return 0;
 }
 
-const char* yan_gemm_version(void) { return "yan-gemm gfx950 6 dense + 8 fp8 tile variants + 2 weight-streaming + 1 split-K fp8 variants"; }
+const char* yan_gemm_version(void) { return "yan-gemm gfx950 6 dense + 8 fp8 tile variants + 2 weight-streaming + 1 split-K fp8 variants + 10 grouped fp8 variants"; }
 
 } // extern "C"

@@ -12,7 +12,11 @@
 //     s = sA * sB. Weights feed the MFMA row operand and activations the column operand, so a lane only ever
 //     meets one activation row per atom: one sA per lane per atom per K block, and sB is wave-uniform;
 //   * the running sums stay in architectural VGPRs (the VALU cannot address AGPRs): 128 per wave;
-//   * m is a run-time argument with tails predicated; N and K are compile-time.
+//   * m is a run-time argument with tails predicated; N and K are compile-time;
+//   * grouped (mixture-of-experts) layouts, the reference's GemmType::GroupedContiguous / GroupedMasked hooks
+//     (yan/include/gemm/scheduler.cuh:7-11,31-48, `int* grouped_layout` of fp8_gemm.cuh:41): every output tile
+//     belongs to one group, which picks the [N, K] weight matrix and its scale table; the rest of the kernel
+//     does not know about groups.
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -43,11 +47,19 @@ struct Fp8TileConfig {
     static_assert(LDS_BYTES <= 160 * 1024, "two stages must fit the 160 KB LDS");
 };
 
-template <int SHAPE_N, int SHAPE_K, int BLOCK_M, int BLOCK_N>
+// Normal:            lhs [m, K], rhs [N, K], out [m, N]; grouped_layout unused.
+// GroupedContiguous: lhs [m, K] is the concatenation of the groups' rows, every group padded to a multiple of 128
+//                    rows (BLOCK_M divides 128); grouped_layout[i] is the group of row i, negative for padding rows,
+//                    whose tiles are skipped; rhs [G, N, K], rhs_scales [G, ceil(N/128), K/128].
+// GroupedMasked:     lhs [G, m, K], out [G, m, N], rhs as above; only the first grouped_layout[g] rows of group g
+//                    are computed; lhs_scales of group g start at g * sa_stride_g floats. The grid is G times the
+//                    grid of one [m, N] problem.
+template <int SHAPE_N, int SHAPE_K, int BLOCK_M, int BLOCK_N, GemmType kGemmType = GemmType::Normal>
 __global__ void __launch_bounds__((get_num_waves(BLOCK_M, BLOCK_N) * kWaveSize))
 fp8_gemm_kernel(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_scales,
                 const uint8_t* __restrict__ rhs, const float* __restrict__ rhs_scales,
-                __bf16* __restrict__ out, int m, int n_rt, int k_rt, int sa_stride_m, int sa_stride_k) {
+                __bf16* __restrict__ out, int m, int n_rt, int k_rt, int sa_stride_m, int sa_stride_k,
+                const int* __restrict__ grouped_layout = nullptr, int sa_stride_g = 0) {
     using Cfg  = Fp8TileConfig<BLOCK_M, BLOCK_N>;
     using Atom = MfmaFP8_16x16x128;
     constexpr int NW = Cfg::NUM_WAVES, TN = Cfg::WTN / 16, TM = Cfg::WTM / 16;
@@ -63,9 +75,28 @@ fp8_gemm_kernel(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_s
     __shared__ __attribute__((aligned(1024))) uint8_t lds_b1[BLOCK_N * kRowBytes];
 
     const XcdTileScheduler<> sched(m, N, BLOCK_M, BLOCK_N);
-    const TileCoord tile = sched.tile_of(blockIdx.x);
+    int bid = blockIdx.x;
+    if constexpr (kGemmType == GemmType::GroupedMasked) {
+        const int group = bid / sched.grid_size();
+        bid -= group * sched.grid_size();
+        lhs        += size_t(group) * m * K;
+        lhs_scales += size_t(group) * sa_stride_g;
+        out        += size_t(group) * m * N;
+        rhs        += size_t(group) * N * K;
+        rhs_scales += size_t(group) * NUM_N_BLOCKS * NUM_K_BLOCKS;
+        m = min(m, grouped_layout[group]);        // rows of this group that exist; tiles past them leave at once
+    }
+    const TileCoord tile = sched.tile_of(bid);
     if (!tile.valid) return;
     const int m0 = tile.m_idx * BLOCK_M, n0 = tile.n_idx * BLOCK_N;
+    if (m0 >= m) return;
+    if constexpr (kGemmType == GemmType::GroupedContiguous) {
+        static_assert(128 % BLOCK_M == 0, "a tile must not straddle two groups (groups are padded to 128 rows)");
+        const int group = grouped_layout[m0];
+        if (group < 0) return;
+        rhs        += size_t(group) * N * K;
+        rhs_scales += size_t(group) * NUM_N_BLOCKS * NUM_K_BLOCKS;
+    }
 
     const int lane = get_lane_id();
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWaveSize);
@@ -220,7 +251,8 @@ template <uint32_t SHAPE_N, uint32_t SHAPE_K, uint32_t BLOCK_M, uint32_t BLOCK_N
           uint32_t kNumGroups, uint32_t kNumStages, uint32_t kNumTMAMulticast, GemmType kGemmType>
 class Gemm {
     static_assert(BLOCK_K == 128, "one k-tile is one 128-deep scale block");
-    static_assert(kGemmType == GemmType::Normal && kNumGroups == 1, "grouped layouts are not implemented");
+    static_assert(kGemmType != GemmType::Normal || kNumGroups == 1, "a plain GEMM has one group");
+    static_assert(kGemmType != GemmType::GroupedContiguous || 128 % BLOCK_M == 0, "contiguous groups are padded to 128 rows");
 
 public:
     // lhs [m, K] e4m3 row-major; lhs_scales fp32, element (i, kb) at i * stride_m + kb * stride_k;
@@ -228,8 +260,34 @@ public:
     static hipError_t run(__hip_bfloat16* out, const void* lhs, const float* lhs_scales, int lhs_scales_stride_m,
                           int lhs_scales_stride_k, const void* rhs, const float* rhs_scales, int m,
                           hipStream_t stream, int num_sms, uint32_t smem_size) {
+        static_assert(kGemmType == GemmType::Normal, "grouped layouts go through run_grouped");
         return run_sized(out, lhs, lhs_scales, lhs_scales_stride_m, lhs_scales_stride_k, rhs, rhs_scales, m,
                          int(SHAPE_N), int(SHAPE_K), stream, num_sms, smem_size);
+    }
+
+    // Grouped layouts (see the kernel's comment). `m` is the total number of rows (contiguous) or the rows
+    // allotted to each group (masked); `grouped_layout` is a device array of m (contiguous) or num_groups (masked)
+    // ints; `lhs_scales_stride_g` is used by the masked layout only. n and k as in run_sized.
+    static hipError_t run_grouped(__hip_bfloat16* out, const void* lhs, const float* lhs_scales, int lhs_scales_stride_m,
+                                  int lhs_scales_stride_k, int lhs_scales_stride_g, const void* rhs, const float* rhs_scales,
+                                  const int* grouped_layout, int num_groups, int m, int n, int k, hipStream_t stream) {
+        static_assert(kGemmType != GemmType::Normal);
+        if (m == 0 || n == 0 || num_groups == 0) return hipSuccess;
+        if (m < 0 || n < 0 || k <= 0 || num_groups < 0 || (n % 4) != 0 || (k % 128) != 0) return hipErrorInvalidValue;
+        if ((SHAPE_N && n != int(SHAPE_N)) || (SHAPE_K && k != int(SHAPE_K))) return hipErrorInvalidValue;
+        if (kNumGroups > 1 && num_groups != int(kNumGroups)) return hipErrorInvalidValue;
+        if (!out || !lhs || !lhs_scales || !rhs || !rhs_scales || !grouped_layout) return hipErrorInvalidValue;
+        const uint64_t m_pad = uint64_t(ceil_div<uint32_t>(m, BLOCK_M)) * BLOCK_M, n_pad = uint64_t(ceil_div<uint32_t>(n, BLOCK_N)) * BLOCK_N;
+        if (m_pad * k >= kOutOfRange || n_pad * k >= kOutOfRange) return hipErrorInvalidValue;
+        using Cfg = Fp8TileConfig<BLOCK_M, BLOCK_N>;
+        const XcdTileScheduler<> sched(m, n, BLOCK_M, BLOCK_N);
+        const uint64_t grid = uint64_t(sched.grid_size()) * (kGemmType == GemmType::GroupedMasked ? num_groups : 1);
+        if (grid >= kOutOfRange) return hipErrorInvalidValue;
+        hipLaunchKernelGGL((fp8_gemm_kernel<SHAPE_N, SHAPE_K, BLOCK_M, BLOCK_N, kGemmType>), dim3(uint32_t(grid)),
+                           dim3(Cfg::NUM_WAVES * kWaveSize), 0, stream, static_cast<const uint8_t*>(lhs), lhs_scales,
+                           static_cast<const uint8_t*>(rhs), rhs_scales, reinterpret_cast<__bf16*>(out), m, n, k,
+                           lhs_scales_stride_m, lhs_scales_stride_k, grouped_layout, lhs_scales_stride_g);
+        return hipGetLastError();
     }
 
     // Same with explicit n and k, which must equal SHAPE_N / SHAPE_K unless those are 0 (sizes known at run time).

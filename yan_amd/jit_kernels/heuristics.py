@@ -17,10 +17,10 @@ _FP8_TILES = {(256, 256): 1.00, (256, 128): 1.12, (128, 256): 1.12, (128, 128): 
               (64, 32): 3.0, (64, 16): 4.5}
 
 
-def rank_tiles(m: int, n: int, num_cus: int, table) -> List[Tuple[float, Tuple[int, int]]]:
+def rank_tiles(m: int, n: int, num_cus: int, table, groups: int = 1) -> List[Tuple[float, Tuple[int, int]]]:
     ranked = []
     for (bm, bn), per_area in table.items():
-        tiles = ceil_div(m, bm) * ceil_div(n, bn)
+        tiles = ceil_div(m, bm) * ceil_div(n, bn) * groups
         rounds = ceil_div(tiles, num_cus)
         ranked.append((rounds * bm * bn * per_area, (bm, bn)))
     return sorted(ranked)
@@ -32,6 +32,14 @@ def get_best_dense_config(m: int, n: int, k: int, num_cus: int) -> Tuple[int, in
 
 def get_best_fp8_config(m: int, n: int, k: int, num_cus: int) -> Tuple[int, int]:
     return rank_tiles(m, n, num_cus, _FP8_TILES)[0][1]
+
+
+def get_best_grouped_fp8_config(m: int, n: int, k: int, num_cus: int, groups: int = 1, m_alignment: int = 0) -> Tuple[int, int]:
+    """Tile of a grouped FP8 GEMM. Contiguous layout: `m` is the total row count and `m_alignment` the padding of
+    every group (a tile must not straddle two groups, so BLOCK_M has to divide it). Masked layout: `m` is the
+    expected row count of one group and `groups` multiplies the tile count."""
+    table = {t: c for t, c in _FP8_TILES.items() if t[1] >= 64 and (m_alignment == 0 or m_alignment % t[0] == 0)}
+    return rank_tiles(max(m, 1), n, num_cus, table, groups)[0][1]
 
 
 def get_skinny_fp8_config(m: int, n: int, k: int, num_cus: int) -> int:

@@ -85,6 +85,44 @@ def make_fp8_case(m: int, n: int, k: int, seed: int = 42, dist: str = 'normal', 
     return (a8, sa), (b8, sb), torch.zeros(m, n, dtype=torch.bfloat16, device=device)
 
 
+def make_grouped_contiguous_case(group_rows, n: int, k: int, seed: int = 42, device='cpu', gen_device='cpu',
+                                 padding_blocks: int = 0, alignment: int = 128):
+    """((A8, sA), (B8 [G,n,k], sB [G,ceil(n/128),k/128]), out, m_indices) for the contiguous grouped layout:
+    group g contributes `group_rows[g]` real rows, padded with zero rows up to the alignment (padding rows carry
+    the group's index, as a caller that pads with zeros would do); `padding_blocks` whole blocks with index -1 follow.
+    `out` is pre-filled with a sentinel so that rows the kernel must not write can be checked."""
+    groups = len(group_rows)
+    gen = torch.Generator(device=gen_device).manual_seed(seed)
+    qs, ss, idx = [], [], []
+    for g, rows in enumerate(group_rows):
+        padded = (rows + alignment - 1) // alignment * alignment
+        x = torch.zeros(padded, k, device=gen_device)
+        x[:rows] = torch.randn(rows, k, generator=gen, device=gen_device)
+        q, sc = per_token_cast_to_fp8(x.to(device))
+        qs.append(q), ss.append(sc), idx.append(torch.full((padded,), g, dtype=torch.int32))
+    if padding_blocks:
+        rows = padding_blocks * alignment
+        q, sc = per_token_cast_to_fp8(torch.randn(rows, k, generator=gen, device=gen_device).to(device))
+        qs.append(q), ss.append(sc), idx.append(torch.full((rows,), -1, dtype=torch.int32))
+    a8, sa = torch.cat(qs), torch.cat(ss)
+    ws = [per_block_cast_to_fp8(torch.randn(n, k, generator=gen, device=gen_device).to(device)) for _ in range(groups)]
+    b8, sb = torch.stack([w[0] for w in ws]), torch.stack([w[1] for w in ws])
+    out = torch.full((a8.size(0), n), -7.0, dtype=torch.bfloat16, device=device)
+    return (a8, sa), (b8, sb), out, torch.cat(idx).to(device)
+
+
+def make_grouped_masked_case(groups: int, m_max: int, n: int, k: int, masked, seed: int = 42, device='cpu', gen_device='cpu'):
+    """((A8 [G,m_max,k], sA [G,m_max,k/128]), (B8 [G,n,k], sB), out [G,m_max,n], masked_m) for the masked layout;
+    `out` is pre-filled with a sentinel."""
+    gen = torch.Generator(device=gen_device).manual_seed(seed)
+    xs = [per_token_cast_to_fp8(torch.randn(m_max, k, generator=gen, device=gen_device).to(device)) for _ in range(groups)]
+    ws = [per_block_cast_to_fp8(torch.randn(n, k, generator=gen, device=gen_device).to(device)) for _ in range(groups)]
+    a8, sa = torch.stack([x[0] for x in xs]), torch.stack([x[1] for x in xs])
+    b8, sb = torch.stack([w[0] for w in ws]), torch.stack([w[1] for w in ws])
+    out = torch.full((groups, m_max, n), -7.0, dtype=torch.bfloat16, device=device)
+    return (a8, sa), (b8, sb), out, torch.tensor(list(masked), dtype=torch.int32, device=device)
+
+
 # ----------------------------------------------------------------------------- shapes exercised on the GPU
 # (m, n, k). Listed here so that every JIT kernel they need can be compiled ahead of time, without a GPU.
 BASELINE_BF16 = {'cfg1': (1024, 1024, 1024), 'cfg2': (8192, 8192, 8192)}
@@ -105,6 +143,15 @@ FP8_TEST_SHAPES = [
     (40, 192, 256), (130, 448, 640),
     (257, 2112, 1024), (128, 7168, 2048), (4096, 2048, 7168),
     (1, 4096, 7168), (17, 4096, 1024), (33, 2112, 640), (64, 7168, 2048), (48, 4100, 384), (40, 2112, 640),
+]
+# Grouped FP8 GEMMs: (rows per group, n, k, blocks of padding rows) and (groups, m_max, n, k, masked_m, expected_m).
+GROUPED_CONTIGUOUS_TEST_CASES = [
+    ((100, 128, 1, 300), 320, 384, 1), ((128, 128), 4096, 1024, 0), ((129,), 200, 128, 2),
+    ((1024, 1024, 1024, 1024), 4096, 7168, 0),
+]
+GROUPED_MASKED_TEST_CASES = [
+    (3, 200, 320, 384, (200, 0, 77), 128), (4, 256, 4096, 1024, (1, 256, 130, 64), 64), (2, 64, 200, 128, (64, 3), 32),
+    (4, 1024, 4096, 7168, (1024, 900, 512, 1), 1024),
 ]
 
 
@@ -130,6 +177,25 @@ def prebuild_jit_kernels(num_cus: int = 256, verbose: bool = False) -> int:
             continue
         name, keys, arg_defs, _, code_template = gemm.fp8_kernel_plan(m, n, k, num_cus)
         code = generate(gemm.includes, arg_defs, cpp_format(code_template, keys))
+        if (name, code) not in seen:
+            seen.add((name, code))
+            rt = build(name, arg_defs, code)
+            if verbose:
+                print(f'built {name} {keys} -> {rt.path}')
+    from .jit_kernels import m_grouped_gemm
+    for rows, n, k, pad_blocks in GROUPED_CONTIGUOUS_TEST_CASES:
+        m = sum((r + 127) // 128 * 128 for r in rows) + 128 * pad_blocks
+        plans = [m_grouped_gemm.grouped_kernel_plan('GroupedContiguous', len(rows), m, n, k, num_cus)]
+        for name, keys, arg_defs, _ in plans:
+            code = generate(m_grouped_gemm.includes, arg_defs, cpp_format(m_grouped_gemm.template, keys))
+            if (name, code) not in seen:
+                seen.add((name, code))
+                rt = build(name, arg_defs, code)
+                if verbose:
+                    print(f'built {name} {keys} -> {rt.path}')
+    for groups, m_max, n, k, _, expected_m in GROUPED_MASKED_TEST_CASES:
+        name, keys, arg_defs, _ = m_grouped_gemm.grouped_kernel_plan('GroupedMasked', groups, min(expected_m, m_max), n, k, num_cus)
+        code = generate(m_grouped_gemm.includes, arg_defs, cpp_format(m_grouped_gemm.template, keys))
         if (name, code) not in seen:
             seen.add((name, code))
             rt = build(name, arg_defs, code)
