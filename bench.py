@@ -91,8 +91,8 @@ def _measured_traffic():
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument('--gpus', type=int, default=1)
-    ap.add_argument('--steps', type=int, default=200)
-    ap.add_argument('--warmup', type=int, default=20)
+    ap.add_argument('--steps', type=int, default=1000)
+    ap.add_argument('--warmup', type=int, default=100)
     ap.add_argument('--also', action='store_true', help='also time bf16 8192^3, the decode shape and 16384^3 (extra fields)')
     ap.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline leg')
     ap.add_argument('--calibrate-copy', action='store_true',
@@ -182,6 +182,20 @@ def main():
         ms, _ = _event_time_ms(lambda: yan.gemm_fp8_fp8_bf16_nt((x8, sx), (w8, sw), o), 10, 2)
         extra['fp8_16384_outliers'] = {'us': round(ms * 1e3, 1), 'tflops': round(2.0 * mm * nn * kk / ms / 1e9, 1),
                                        'frac_of_fp8_peak': round(2.0 * mm * nn * kk / ms / 1e9 / PEAK_FP8_TFLOPS, 4)}
+        del x8, sx, w8, sw, o
+        # grouped (mixture-of-experts) layouts: 4 groups x 8192 rows contiguous; 4 groups x 1024 of 1024 rows masked
+        rows, nn, kk = (8192,) * 4, 4096, 7168
+        (x8, sx), (w8, sw), o, idx = testing.make_grouped_contiguous_case(rows, nn, kk, seed=42, device='cuda', gen_device='cuda')
+        sx = yan.get_col_major_tensor(sx)
+        ms, _ = _event_time_ms(lambda: yan.m_grouped_gemm_fp8_fp8_bf16_nt_contiguous((x8, sx), (w8, sw), o, idx), 20, 3)
+        fl = 2.0 * sum(rows) * nn * kk
+        extra['fp8_grouped_contiguous_4x8192x4096x7168'] = {'us': round(ms * 1e3, 1), 'tflops': round(fl / ms / 1e9, 1),
+                                                            'frac_of_fp8_peak': round(fl / ms / 1e9 / PEAK_FP8_TFLOPS, 4)}
+        (x8, sx), (w8, sw), o, mm_ = testing.make_grouped_masked_case(4, 1024, nn, kk, (1024,) * 4, seed=42, device='cuda', gen_device='cuda')
+        ms, _ = _event_time_ms(lambda: yan.m_grouped_gemm_fp8_fp8_bf16_nt_masked((x8, sx), (w8, sw), o, mm_, 1024), 50, 5)
+        fl = 2.0 * 4 * 1024 * nn * kk
+        extra['fp8_grouped_masked_4x1024x4096x7168'] = {'us': round(ms * 1e3, 1), 'tflops': round(fl / ms / 1e9, 1),
+                                                        'frac_of_fp8_peak': round(fl / ms / 1e9 / PEAK_FP8_TFLOPS, 4)}
         del x8, sx, w8, sw, o
         line['extra'] = extra
 

@@ -83,7 +83,7 @@ YAN_API int yan_m_grouped_gemm_fp8_fp8_bf16_nt_masked(const void* lhs, const flo
                                               int m_max, int expected_m, int n, int k, void* stream, int num_sms);
 
 /* Macro tile the library uses for a problem: op 0 = dense 16-bit, 1 = FP8 block-scaled, 2 = FP8 grouped contiguous
- * (m = total rows). Writes BLOCK_M / BLOCK_N.
+ * (m = total rows, and `k` carries the number of groups instead of the depth). Writes BLOCK_M / BLOCK_N.
  * For op 1 with few activation rows the answer is (16 * atoms, 16): the weight-streaming kernel.
  * Host-only (no device call). Stands where the reference leaves tile choice to the caller's keys
  * (yan/jit_kernels/cute_gemm.py:41, yan/jit_kernels/gemm.py:13-16). Returns 0, or 1 for an unknown op. */

@@ -48,7 +48,8 @@ def test_version_and_tile_selection_match_python(lib):
             assert capi.select_tile(1, m, n, k, cus) == heuristics.get_fp8_tile(m, n, k, cus), (m, n, k, cus)
     for m, n in [(4096, 4096), (32768, 4096), (128, 7168), (256, 200), (1024, 24576)]:
         for cus in (256, 80):
-            assert capi.select_tile(2, m, n, 1024, cus) == heuristics.get_best_grouped_fp8_config(m, n, 1024, cus, 1, 128)
+            for groups in (1, 4, 64):
+                assert capi.select_tile(2, m, n, groups, cus) == heuristics.get_best_grouped_fp8_config(m, n, 1024, cus, 1, 128, groups)
     bm, bn = ctypes.c_int(), ctypes.c_int()
     assert lib.yan_gemm_select_tile(7, 1, 1, 1, 256, ctypes.byref(bm), ctypes.byref(bn)) == 1
     assert lib.yan_gemm_select_tile(0, 1, 1, 1, 0, ctypes.byref(bm), ctypes.byref(bn)) == 1

@@ -348,6 +348,13 @@ def test_grouped_contiguous_parity(rows, n, k, pad_blocks):
     again = out.cuda()
     yan.m_grouped_gemm_fp8_fp8_bf16_nt_contiguous((a8d, yan.get_col_major_tensor(sad)), (b8d, sbd), again, idxd)
     assert torch.equal(again, got)
+    if pad_blocks:
+        # the same rows rotated by one 128-row block: the padding block now leads, and every group boundary moves
+        rolled = [torch.roll(a8d.view(torch.uint8), 128, 0).view(torch.float8_e4m3fn), torch.roll(sad, 128, 0).contiguous(),
+                  torch.roll(idxd, 128, 0).contiguous()]
+        got2 = out.cuda()
+        yan.m_grouped_gemm_fp8_fp8_bf16_nt_contiguous((rolled[0], rolled[1]), (b8d, sbd), got2, rolled[2])
+        assert torch.equal(torch.roll(got2, -128, 0), got)
     # the first group's rows through the plain entry point
     r0 = (rows[0] + 127) // 128 * 128
     plain = torch.zeros(r0, n, dtype=torch.bfloat16, device='cuda')

@@ -27,13 +27,16 @@ void pick(const TileCost (&tiles)[COUNT], int m, int n, int num_cus, int* bm, in
     }
 }
 
-// Tile of a grouped FP8 GEMM (get_best_grouped_fp8_config in heuristics.py): tiles at least 64 wide, BLOCK_M dividing
-// `m_alignment` when that is non-zero, tile count multiplied by `groups`.
-void pick_grouped(int m, int n, int num_cus, int groups, int m_alignment, int* bm, int* bn) {
+// Tile of a grouped FP8 GEMM (get_best_grouped_fp8_config in heuristics.py): tiles at least 64 wide; with a non-zero
+// `m_alignment` BLOCK_M divides it, or is twice it when the `groups_in_m` groups average 1024 rows or more; the tile
+// count is multiplied by `groups`.
+void pick_grouped(int m, int n, int num_cus, int groups, int m_alignment, int groups_in_m, int* bm, int* bn) {
     double best = -1;
     if (m < 1) m = 1;
     for (const TileCost& t : kFp8Tiles) {
-        if (t.bn < 64 || (m_alignment && m_alignment % t.bm != 0)) continue;
+        const bool fits = m_alignment == 0 || m_alignment % t.bm == 0 ||
+                          (t.bm == 2 * m_alignment && (long long)m >= 1024ll * groups_in_m);
+        if (t.bn < 64 || !fits) continue;
         const long long count  = (long long)((m + t.bm - 1) / t.bm) * ((n + t.bn - 1) / t.bn) * groups;
         const long long rounds = (count + num_cus - 1) / num_cus;
         const double cost = double(rounds) * t.bm * t.bn * t.per_area;
@@ -121,13 +124,14 @@ int yan_m_grouped_gemm_fp8_fp8_bf16_nt_contiguous(const void* lhs, const float* 
     if (lhs_scales_stride_m < 0 || lhs_scales_stride_k < 0 || last >= (1ll << 28)) return int(hipErrorInvalidValue);
     const int cus = num_sms > 0 ? num_sms : device_cus();
     int bm = 0, bn = 0;
-    pick_grouped(m, n, cus, 1, 128, &bm, &bn);
+    pick_grouped(m, n, cus, 1, 128, num_groups, &bm, &bn);
 #define YAN_GROUPED_CASE(BM, BN)                                                                                     \
     if (bm == BM && bn == BN)                                                                                        \
         return int(yan::Gemm<0, 0, BM, BN, 128, 1, 2, 1, yan::GemmType::GroupedContiguous>::run_grouped(             \
             static_cast<__hip_bfloat16*>(out), lhs, lhs_scales, int(lhs_scales_stride_m), int(lhs_scales_stride_k), 0, rhs, \
             rhs_scales, m_indices, num_groups, m, n, k, static_cast<hipStream_t>(stream)));
-    YAN_GROUPED_CASE(128, 256) YAN_GROUPED_CASE(128, 128) YAN_GROUPED_CASE(64, 128) YAN_GROUPED_CASE(64, 64)
+    YAN_GROUPED_CASE(256, 256) YAN_GROUPED_CASE(256, 128) YAN_GROUPED_CASE(128, 256) YAN_GROUPED_CASE(128, 128)
+    YAN_GROUPED_CASE(64, 128) YAN_GROUPED_CASE(64, 64)
 #undef YAN_GROUPED_CASE
     return int(hipErrorInvalidValue);
 }
@@ -143,7 +147,7 @@ int yan_m_grouped_gemm_fp8_fp8_bf16_nt_masked(const void* lhs, const float* lhs_
         lhs_scales_stride_g >= (1ll << 31)) return int(hipErrorInvalidValue);
     const int cus = num_sms > 0 ? num_sms : device_cus();
     int bm = 0, bn = 0;
-    pick_grouped(expected_m < m_max ? expected_m : m_max, n, cus, num_groups, 0, &bm, &bn);
+    pick_grouped(expected_m < m_max ? expected_m : m_max, n, cus, num_groups, 0, 1, &bm, &bn);
 #define YAN_GROUPED_CASE(BM, BN)                                                                                     \
     if (bm == BM && bn == BN)                                                                                        \
         return int(yan::Gemm<0, 0, BM, BN, 128, 1, 2, 1, yan::GemmType::GroupedMasked>::run_grouped(                 \
@@ -163,11 +167,11 @@ int yan_gemm_select_tile(int op, int m, int n, int k, int num_cus, int* block_m,
         if (const int atoms = skinny_atoms(m, n, num_cus)) { *block_m = 16 * atoms; *block_n = 16; }
         else pick(kFp8Tiles, m, n, num_cus, block_m, block_n);
     }
-    else if (op == 2) pick_grouped(m, n, num_cus, 1, 128, block_m, block_n);
+    else if (op == 2) pick_grouped(m, n, num_cus, 1, 128, k, block_m, block_n);
     else return 1;
     return 0;
 }
 
-const char* yan_gemm_version(void) { return "yan-gemm gfx950 6 dense + 8 fp8 tile variants + 2 weight-streaming + 1 split-K fp8 variants + 10 grouped fp8 variants"; }
+const char* yan_gemm_version(void) { return "yan-gemm gfx950 6 dense + 8 fp8 tile variants + 2 weight-streaming + 1 split-K fp8 variants + 12 grouped fp8 variants"; }
 
 } // extern "C"

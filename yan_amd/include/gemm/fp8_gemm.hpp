@@ -90,13 +90,27 @@ fp8_gemm_kernel(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_s
     if (!tile.valid) return;
     const int m0 = tile.m_idx * BLOCK_M, n0 = tile.n_idx * BLOCK_N;
     if (m0 >= m) return;
+    // Contiguous groups are padded to 128 rows. A tile of up to 128 rows lies in one group. A 256-row tile may
+    // hold two: it then makes two passes over K, one per 128-row half, each with its own group's weights and
+    // storing only its half (rare when groups are long, and long groups are when 256-row tiles pay off).
+    constexpr bool kTwoHalves = kGemmType == GemmType::GroupedContiguous && BLOCK_M == 256;
+    int num_passes = 1, pass_group[2] = {0, 0}, pass_lo[2] = {m0, m0}, pass_hi[2] = {m, m};
     if constexpr (kGemmType == GemmType::GroupedContiguous) {
-        static_assert(128 % BLOCK_M == 0, "a tile must not straddle two groups (groups are padded to 128 rows)");
-        const int group = grouped_layout[m0];
-        if (group < 0) return;
-        rhs        += size_t(group) * N * K;
-        rhs_scales += size_t(group) * NUM_N_BLOCKS * NUM_K_BLOCKS;
+        static_assert(128 % BLOCK_M == 0 || BLOCK_M == 256, "tiles are 128-row blocks, parts of one, or two of them");
+        const int g0 = grouped_layout[m0];
+        const int g1 = (kTwoHalves && m0 + 128 < m) ? grouped_layout[m0 + 128] : g0;
+        if (g0 == g1) {
+            if (g0 < 0) return;
+            pass_group[0] = g0;
+        } else {
+            num_passes = 0;
+            if (g0 >= 0) { pass_group[0] = g0; pass_hi[0] = m0 + 128; num_passes = 1; }
+            if (g1 >= 0) { pass_group[num_passes] = g1; pass_lo[num_passes] = m0 + 128; ++num_passes; }
+            if (num_passes == 0) return;
+        }
     }
+    const uint8_t* const rhs_all = rhs;
+    const float* const rhs_scales_all = rhs_scales;
 
     const int lane = get_lane_id();
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWaveSize);
@@ -105,7 +119,7 @@ fp8_gemm_kernel(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_s
     const int m_slab = m0 + wm * Cfg::WTM, n_slab = n0 + wn * Cfg::WTN;
 
     const __amdgpu_buffer_rsrc_t rsrc_a = make_rsrc(lhs, uint32_t(m) * K);
-    const __amdgpu_buffer_rsrc_t rsrc_b = make_rsrc(rhs, uint32_t(N) * K);
+    __amdgpu_buffer_rsrc_t rsrc_b = make_rsrc(rhs, uint32_t(N) * K);
     TileStager<BLOCK_M, NW> stage_a;
     TileStager<BLOCK_N, NW> stage_b;
     stage_a.init(m0, K, wave, lane);
@@ -128,10 +142,6 @@ fp8_gemm_kernel(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_s
     };
 
     f32x4 acc[TN][TM];
-#pragma unroll
-    for (int i = 0; i < TN; ++i)
-#pragma unroll
-        for (int j = 0; j < TM; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
 
     float sa_next[TM];     // activation scales of the k-tile in flight
     float sb_next[NB];     // weight scales of the k-tile in flight (wave-uniform)
@@ -219,6 +229,17 @@ fp8_gemm_kernel(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_s
             }
         });
     };
+    for (int pass = 0; pass < (kGemmType == GemmType::GroupedContiguous ? num_passes : 1); ++pass) {
+    if constexpr (kGemmType == GemmType::GroupedContiguous) {
+        rhs        = rhs_all + size_t(pass_group[pass]) * N * K;
+        rhs_scales = rhs_scales_all + size_t(pass_group[pass]) * NUM_N_BLOCKS * NUM_K_BLOCKS;
+        rsrc_b     = make_rsrc(rhs, uint32_t(N) * K);
+        if (pass) __syncthreads();        // every wave has read the last k-tile of the previous pass
+    }
+#pragma unroll
+    for (int i = 0; i < TN; ++i)
+#pragma unroll
+        for (int j = 0; j < TM; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
     stage_a.issue(rsrc_a, lds_a0, 0, wave);
     stage_b.issue(rsrc_b, lds_b0, 0, wave);
     load_scales(0);
@@ -233,6 +254,7 @@ fp8_gemm_kernel(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_s
     for (int j = 0; j < TM; ++j) {
         const int mm = m_slab + j * 16 + col;
         if (mm >= m) continue;
+        if constexpr (kTwoHalves) { if (mm < pass_lo[pass] || mm >= pass_hi[pass]) continue; }
         __bf16* row = out + size_t(mm) * N;
 #pragma unroll
         for (int i = 0; i < TN; ++i) {
@@ -240,6 +262,7 @@ fp8_gemm_kernel(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_s
             if (nn < N) *reinterpret_cast<bf16x4*>(row + nn) = pack4(acc[i][j], __bf16{});
         }
     }
+    }   // pass
 }
 
 // Host side of the kernel, shaped after the class the reference's JIT template instantiates
@@ -252,7 +275,7 @@ template <uint32_t SHAPE_N, uint32_t SHAPE_K, uint32_t BLOCK_M, uint32_t BLOCK_N
 class Gemm {
     static_assert(BLOCK_K == 128, "one k-tile is one 128-deep scale block");
     static_assert(kGemmType != GemmType::Normal || kNumGroups == 1, "a plain GEMM has one group");
-    static_assert(kGemmType != GemmType::GroupedContiguous || 128 % BLOCK_M == 0, "contiguous groups are padded to 128 rows");
+    static_assert(kGemmType != GemmType::GroupedContiguous || 128 % BLOCK_M == 0 || BLOCK_M == 256, "contiguous groups are padded to 128 rows");
 
 public:
     // lhs [m, K] e4m3 row-major; lhs_scales fp32, element (i, kb) at i * stride_m + kb * stride_k;

@@ -1,7 +1,7 @@
 // Workgroup -> output-tile mapping for a 256-CU, 8-XCD part.
 // Replaces the reference's persistent tile Scheduler (yan/include/gemm/scheduler.cuh:15-58: block count
-// ceil(m/BLOCK_M)*ceil(N/BLOCK_N), grouped swizzle of 16 blocks for L2 reuse). Only GemmType::Normal is
-// implemented; the other two enumerators are kept so the template surface reads the same.
+// ceil(m/BLOCK_M)*ceil(N/BLOCK_N), grouped swizzle of 16 blocks for L2 reuse). The mapping is the same for all
+// three GemmTypes; what a group changes (operand bases, valid rows) is applied by the kernel on top of the tile.
 #pragma once
 
 #include "utils.hpp"

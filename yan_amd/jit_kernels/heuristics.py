@@ -34,11 +34,18 @@ def get_best_fp8_config(m: int, n: int, k: int, num_cus: int) -> Tuple[int, int]
     return rank_tiles(m, n, num_cus, _FP8_TILES)[0][1]
 
 
-def get_best_grouped_fp8_config(m: int, n: int, k: int, num_cus: int, groups: int = 1, m_alignment: int = 0) -> Tuple[int, int]:
-    """Tile of a grouped FP8 GEMM. Contiguous layout: `m` is the total row count and `m_alignment` the padding of
-    every group (a tile must not straddle two groups, so BLOCK_M has to divide it). Masked layout: `m` is the
-    expected row count of one group and `groups` multiplies the tile count."""
-    table = {t: c for t, c in _FP8_TILES.items() if t[1] >= 64 and (m_alignment == 0 or m_alignment % t[0] == 0)}
+def get_best_grouped_fp8_config(m: int, n: int, k: int, num_cus: int, groups: int = 1, m_alignment: int = 0,
+                                groups_in_m: int = 1) -> Tuple[int, int]:
+    """Tile of a grouped FP8 GEMM. Contiguous layout: `m` is the total row count, `m_alignment` the padding of every
+    group and `groups_in_m` the number of groups sharing the rows: a tile of up to `m_alignment` rows must divide it;
+    the 256-row tile, which handles a group boundary in its middle with a second pass over K, is offered when groups
+    average at least 1024 rows. Masked layout: `m` is the expected row count of one group and `groups` multiplies
+    the tile count."""
+    def allowed(bm):
+        if m_alignment == 0 or m_alignment % bm == 0:
+            return True
+        return bm == 2 * m_alignment and m >= 1024 * groups_in_m
+    table = {t: c for t, c in _FP8_TILES.items() if t[1] >= 64 and allowed(t[0])}
     return rank_tiles(max(m, 1), n, num_cus, table, groups)[0][1]
 
 

@@ -48,7 +48,7 @@ def grouped_kernel_plan(gemm_type: str, num_groups: int, m: int, n: int, k: int,
     for 'GroupedContiguous' and the expected rows per group for 'GroupedMasked'."""
     assert gemm_type in ('GroupedContiguous', 'GroupedMasked')
     if gemm_type == 'GroupedContiguous':
-        block_m, block_n = get_best_grouped_fp8_config(m, n, k, num_cus, 1, get_m_alignment_for_contiguous_layout())
+        block_m, block_n = get_best_grouped_fp8_config(m, n, k, num_cus, 1, get_m_alignment_for_contiguous_layout(), num_groups)
         name = 'm_grouped_gemm_fp8_fp8_bf16_nt'
     else:
         block_m, block_n = get_best_grouped_fp8_config(m, n, k, num_cus, num_groups)

@@ -147,7 +147,9 @@ FP8_TEST_SHAPES = [
 # Grouped FP8 GEMMs: (rows per group, n, k, blocks of padding rows) and (groups, m_max, n, k, masked_m, expected_m).
 GROUPED_CONTIGUOUS_TEST_CASES = [
     ((100, 128, 1, 300), 320, 384, 1), ((128, 128), 4096, 1024, 0), ((129,), 200, 128, 2),
-    ((1024, 1024, 1024, 1024), 4096, 7168, 0),
+    ((1024, 1024, 1024, 1024), 4096, 7168, 0), ((8192, 8192, 8192, 8192), 4096, 7168, 0),
+    # long groups whose boundaries fall in the middle of 256-row tiles (two-pass tiles), with a trailing padding block
+    ((1150, 900, 1300, 1100), 512, 512, 1),
 ]
 GROUPED_MASKED_TEST_CASES = [
     (3, 200, 320, 384, (200, 0, 77), 128), (4, 256, 4096, 1024, (1, 256, 130, 64), 64), (2, 64, 200, 128, (64, 3), 32),
