@@ -197,6 +197,20 @@ def main():
         extra['fp8_grouped_masked_4x1024x4096x7168'] = {'us': round(ms * 1e3, 1), 'tflops': round(fl / ms / 1e9, 1),
                                                         'frac_of_fp8_peak': round(fl / ms / 1e9 / PEAK_FP8_TFLOPS, 4)}
         del x8, sx, w8, sw, o
+        # quantisers in front of the GEMM (HBM-bound): cfg3's activations per token, its weights per block, from bf16
+        mm, nn, kk = testing.BASELINE_FP8['cfg3']
+        xs = torch.randn(mm, kk, device='cuda').bfloat16()
+        ws = torch.randn(nn, kk, device='cuda').bfloat16()
+        for name, fn, kern, elems, groups in (
+                ('per_token_cast_4096x7168_bf16', lambda: yan.per_token_cast_to_fp8(xs, col_major_scales=True), 'per_token_cast_kernel', mm * kk, mm * kk // 128),
+                ('per_block_cast_7168x7168_bf16', lambda: yan.per_block_cast_to_fp8(ws), 'per_block_cast_kernel', nn * kk, (nn // 128) * (kk // 128))):
+            t_warm = yan.bench_kineto(fn, kern, suppress_kineto_output=True)
+            t_cold = yan.bench_kineto(fn, kern, suppress_kineto_output=True, flush_l2=True)
+            byt = 3 * elems + 4 * groups
+            extra[name] = {'kernel_us_warm': round(t_warm * 1e6, 2), 'kernel_us_cold': round(t_cold * 1e6, 2),
+                           'algorithmic_bytes': byt, 'gb_per_s_cold': round(byt / t_cold / 1e9, 1),
+                           'frac_of_hbm_peak_cold': round(byt / t_cold / 1e9 / PEAK_HBM_GBPS, 4)}
+        del xs, ws
         line['extra'] = extra
 
     if not args.no_cpu:

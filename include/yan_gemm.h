@@ -82,6 +82,18 @@ YAN_API int yan_m_grouped_gemm_fp8_fp8_bf16_nt_masked(const void* lhs, const flo
                                               const float* rhs_scales, void* out, const int* masked_m, int num_groups,
                                               int m_max, int expected_m, int n, int k, void* stream, int num_sms);
 
+/* Quantisers producing the GEMM's operands in one pass over HBM: amax over the group clamped at 1e-4,
+ * q = e4m3(x * (448 / amax)) with round to nearest even, scale = amax / 448; bit-identical to the torch op chain
+ * callers of this convention use. Sources are bf16 (x_is_fp32 == 0) or fp32, row-major, k % 128 == 0.
+ * per-token: groups of 1 x 128; scale (i, kb) is written to scales[i*scales_stride_m + kb*scales_stride_k]
+ *            ((k/128, 1) for row-major, (1, m) for the token-contiguous layout the GEMM reads fastest).
+ * per-block: groups of 128 x 128 (a ragged last block of rows uses the rows that exist); scales [ceil(n/128)][k/128].
+ * They produce what the reference's operand names lhs/lhs_scales and rhs/rhs_scales stand for
+ * (yan/jit_kernels/gemm.py:23-30); the reference has no quantiser of its own. */
+YAN_API int yan_per_token_cast_to_fp8(const void* x, int x_is_fp32, void* q, float* scales, long long scales_stride_m,
+                              long long scales_stride_k, int m, int k, void* stream);
+YAN_API int yan_per_block_cast_to_fp8(const void* w, int w_is_fp32, void* q, float* scales, int n, int k, void* stream);
+
 /* Macro tile the library uses for a problem: op 0 = dense 16-bit, 1 = FP8 block-scaled, 2 = FP8 grouped contiguous
  * (m = total rows, and `k` carries the number of groups instead of the depth). Writes BLOCK_M / BLOCK_N.
  * For op 1 with few activation rows the answer is (16 * atoms, 16): the weight-streaming kernel.

@@ -23,7 +23,7 @@ def _declared(repo_root):
 
 def test_library_exports_every_declared_symbol(lib, repo_root):
     declared = _declared(repo_root)
-    assert declared == sorted(capi.SYMBOLS) and len(declared) == 7
+    assert declared == sorted(capi.SYMBOLS) and len(declared) == 9
     for name in declared:
         assert hasattr(lib, name), name
     out = subprocess.check_output(['nm', '-D', '--defined-only', os.path.join(repo_root, 'yan_amd', 'csrc', 'libyan_gemm.so')], text=True)
@@ -67,6 +67,12 @@ def test_compute_entry_points_validate_before_touching_a_device(lib):
     assert lib.yan_gemm_fp8_fp8_bf16_nt(null, null, 1, 1, null, null, null, 4, 128, 64, null, 256) != 0    # k % 128
     assert lib.yan_gemm_fp8_fp8_bf16_nt(null, null, 1, 1, null, null, null, 4, 126, 128, null, 256) != 0   # n % 4
     assert lib.yan_gemm_fp8_fp8_bf16_nt(null, null, 1, 1, null, null, null, 4, 128, 128, null, 256) != 0   # null operands
+    assert lib.yan_per_token_cast_to_fp8(null, 0, null, null, 1, 1, 0, 128, null) == 0                     # no rows
+    assert lib.yan_per_token_cast_to_fp8(null, 0, null, null, 1, 1, 4, 100, null) != 0                     # k % 128
+    assert lib.yan_per_token_cast_to_fp8(null, 1, null, null, 1, 1, 4, 128, null) != 0                     # null operands
+    assert lib.yan_per_block_cast_to_fp8(null, 0, null, null, 0, 128, null) == 0
+    assert lib.yan_per_block_cast_to_fp8(null, 1, null, null, 4, 130, null) != 0
+    assert lib.yan_per_block_cast_to_fp8(null, 0, null, null, 4, 128, null) != 0
     grouped_c, grouped_m = lib.yan_m_grouped_gemm_fp8_fp8_bf16_nt_contiguous, lib.yan_m_grouped_gemm_fp8_fp8_bf16_nt_masked
     assert grouped_c(null, null, 1, 1, null, null, null, null, 2, 0, 128, 128, null, 256) == 0             # no rows
     assert grouped_c(null, null, 1, 1, null, null, null, null, 2, 100, 128, 128, null, 256) != 0           # m % 128

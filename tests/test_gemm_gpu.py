@@ -309,6 +309,104 @@ def test_fp8_outlier_16384_cubed():
 
 
 # ----------------------------------------------------------------------------- the ahead-of-time C-ABI library
+# ----------------------------------------------------------------------------- quantisers in front of the FP8 GEMM
+def _oracle_per_token(x):
+    q, s_ = oracle.per_token_cast_to_fp8(x.float().numpy())
+    return torch.from_numpy(q), torch.from_numpy(s_)
+
+
+def _oracle_per_block(w):
+    q, s_ = oracle.per_block_cast_to_fp8(w.float().numpy())
+    return torch.from_numpy(q), torch.from_numpy(s_)
+
+
+def _tie_rows():
+    """Rows of 128 values with |max| = 448 exactly (so the quantiser's factor is 1.0) holding every positive e4m3
+    value, every midpoint between neighbours and the fp32 numbers just below and above each midpoint, both signs:
+    any deviation from round-to-nearest-even, or from exact handling of subnormals, changes a code."""
+    vals = np.sort(np.unique(np.abs(oracle.e4m3fn_decode_table()[np.isfinite(oracle.e4m3fn_decode_table())])))
+    mids = (vals[:-1] + vals[1:]) / 2
+    cand = np.concatenate([vals, mids, np.nextafter(mids, np.float32(0)), np.nextafter(mids, np.float32(1e9))]).astype(np.float32)
+    cand = np.concatenate([cand, -cand])
+    rows = -(-cand.size // 127)
+    buf = np.zeros((rows, 128), dtype=np.float32)
+    buf[:, 0] = 448.0
+    flat = np.zeros(rows * 127, dtype=np.float32)
+    flat[:cand.size] = cand
+    buf[:, 1:] = flat.reshape(rows, 127)
+    return torch.from_numpy(buf)
+
+
+@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize('m,k', [(1, 128), (63, 256), (300, 640), (4096, 7168)])
+def test_per_token_cast_is_bit_identical_to_the_oracle(m, k, dtype):
+    g = torch.Generator().manual_seed(m + k)
+    x = (torch.randn(m, k, generator=g) * 3).to(dtype)
+    x[m // 2, :128] = 0                                     # an all-zero group: amax clamps at 1e-4
+    want_q, want_s = _oracle_per_token(x)
+    q, sc = yan.per_token_cast_to_fp8(x.cuda())
+    assert q.dtype == torch.float8_e4m3fn and q.shape == (m, k) and sc.shape == (m, k // 128)
+    assert torch.equal(q.view(torch.uint8).cpu(), want_q) and torch.equal(sc.cpu(), want_s)
+    # token-contiguous scales: same values, the layout get_col_major_tensor gives
+    q2, sc2 = yan.per_token_cast_to_fp8(x.cuda(), col_major_scales=True)
+    assert sc2.stride(0) == 1 and torch.equal(sc2.cpu(), want_s) and torch.equal(q2.view(torch.uint8), q.view(torch.uint8))
+    assert yan.get_col_major_tensor(sc2).data_ptr() == sc2.data_ptr()
+    # torch's own op chain run on the device: its division kernel is not correctly rounded, so it may sit one ulp
+    # away in a scale and one code away in the few elements that land next to a rounding boundary
+    tq, ts = testing.per_token_cast_to_fp8(x.cuda())
+    assert torch.allclose(ts, sc, rtol=2.5e-7, atol=0)
+    assert float((tq.view(torch.uint8) != q.view(torch.uint8)).float().mean()) < 2e-3
+    # the C-ABI library gives the JIT kernel's bits
+    lq, ls = torch.empty_like(q), torch.empty_like(sc)
+    assert capi.per_token_cast_to_fp8(x.cuda(), lq, ls) == 0
+    assert torch.equal(lq.view(torch.uint8), q.view(torch.uint8)) and torch.equal(ls, sc)
+
+
+@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize('n,k', [(128, 128), (129, 128), (300, 640), (7168, 7168)])
+def test_per_block_cast_is_bit_identical_to_the_oracle(n, k, dtype):
+    g = torch.Generator().manual_seed(n * 3 + k)
+    w = torch.randn(n, k, generator=g).to(dtype)
+    w[:128, :128] = 0                                       # an all-zero block
+    want_q, want_s = _oracle_per_block(w)
+    q, sc = yan.per_block_cast_to_fp8(w.cuda())
+    assert q.shape == (n, k) and sc.shape == ((n + 127) // 128, k // 128)
+    assert torch.equal(q.view(torch.uint8).cpu(), want_q) and torch.equal(sc.cpu(), want_s)
+    lq, ls = torch.empty_like(q), torch.empty_like(sc)
+    assert capi.per_block_cast_to_fp8(w.cuda(), lq, ls) == 0
+    assert torch.equal(lq.view(torch.uint8), q.view(torch.uint8)) and torch.equal(ls, sc)
+
+
+def test_casts_round_to_nearest_even_on_every_tie():
+    x = _tie_rows()
+    want = torch.from_numpy(oracle.e4m3fn_encode(x.numpy()))
+    q, sc = yan.per_token_cast_to_fp8(x.cuda())
+    assert torch.equal(sc.cpu(), torch.ones(x.size(0), 1))
+    assert torch.equal(q.view(torch.uint8).cpu(), want)
+    assert torch.equal(x.to(torch.float8_e4m3fn).view(torch.uint8), want)       # torch's CPU cast says the same
+    # the per-block kernel shares the conversion; one 128 x 128 block, padded with copies of the first row
+    w = x[:128] if x.size(0) >= 128 else torch.cat([x, x[:1].expand(128 - x.size(0), 128)])
+    qb, sb = yan.per_block_cast_to_fp8(w.contiguous().cuda())
+    assert float(sb) == 1.0 and torch.equal(qb.view(torch.uint8).cpu(), torch.from_numpy(oracle.e4m3fn_encode(w.numpy())))
+
+
+def test_quantise_then_gemm_matches_the_oracle_end_to_end():
+    """bf16 sources -> device quantisers -> FP8 GEMM, against the oracle's quantisers and product from the same sources."""
+    m, n, k = 200, 384, 512
+    g = torch.Generator().manual_seed(77)
+    x, w = torch.randn(m, k, generator=g).bfloat16(), torch.randn(n, k, generator=g).bfloat16()
+    lhs = yan.per_token_cast_to_fp8(x.cuda(), col_major_scales=True)
+    rhs = yan.per_block_cast_to_fp8(w.cuda())
+    out = torch.zeros(m, n, dtype=torch.bfloat16, device='cuda')
+    yan.gemm_fp8_fp8_bf16_nt(lhs, rhs, out)
+    qa, sa = oracle.per_token_cast_to_fp8(x.float().numpy())
+    qb, sb = oracle.per_block_cast_to_fp8(w.float().numpy())
+    ref = oracle.gemm_fp8_block_scaled_ref(qa, sa, qb, sb)
+    assert oracle.calc_diff(out.float().cpu().numpy(), ref) < 1e-5
+    # and the quantised product stays within the FP8 tolerance of the unquantised one
+    assert oracle.calc_diff(out.float().cpu().numpy(), x.float().numpy() @ w.float().numpy().T) < 1e-3
+
+
 # ----------------------------------------------------------------------------- grouped FP8 GEMMs
 def _np_codes(t):
     return t.view(torch.uint8).cpu().numpy()

@@ -9,7 +9,8 @@ _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), 'csrc', 'li
 _lib = None
 
 SYMBOLS = ('yan_gemm_bf16_tn', 'yan_gemm_fp16_tn', 'yan_gemm_fp8_fp8_bf16_nt', 'yan_m_grouped_gemm_fp8_fp8_bf16_nt_contiguous',
-           'yan_m_grouped_gemm_fp8_fp8_bf16_nt_masked', 'yan_gemm_select_tile', 'yan_gemm_version')
+           'yan_m_grouped_gemm_fp8_fp8_bf16_nt_masked', 'yan_per_token_cast_to_fp8', 'yan_per_block_cast_to_fp8',
+           'yan_gemm_select_tile', 'yan_gemm_version')
 
 
 def load() -> ctypes.CDLL:
@@ -24,6 +25,8 @@ def load() -> ctypes.CDLL:
         lib.yan_gemm_select_tile.argtypes = [ci, ci, ci, ci, ci, ctypes.POINTER(ci), ctypes.POINTER(ci)]
         lib.yan_m_grouped_gemm_fp8_fp8_bf16_nt_contiguous.argtypes = [vp, vp, ll, ll, vp, vp, vp, vp, ci, ci, ci, ci, vp, ci]
         lib.yan_m_grouped_gemm_fp8_fp8_bf16_nt_masked.argtypes = [vp, vp, ll, ll, ll, vp, vp, vp, vp, ci, ci, ci, ci, ci, vp, ci]
+        lib.yan_per_token_cast_to_fp8.argtypes = [vp, ci, vp, vp, ll, ll, ci, ci, vp]
+        lib.yan_per_block_cast_to_fp8.argtypes = [vp, ci, vp, vp, ci, ci, vp]
         for name in SYMBOLS[:-1]:
             getattr(lib, name).restype = ci
         lib.yan_gemm_version.restype = ctypes.c_char_p
@@ -67,6 +70,18 @@ def m_grouped_gemm_fp8_fp8_bf16_nt_masked(lhs, rhs, out: torch.Tensor, masked_m:
     return load().yan_m_grouped_gemm_fp8_fp8_bf16_nt_masked(
         a8.data_ptr(), sa.data_ptr(), sa.stride(0), sa.stride(1), sa.stride(2), b8.data_ptr(), sb.data_ptr(),
         out.data_ptr(), masked_m.data_ptr(), groups, m_max, expected_m, n, k, _stream_handle(), num_sms)
+
+
+def per_token_cast_to_fp8(x: torch.Tensor, q: torch.Tensor, scales: torch.Tensor) -> int:
+    m, k = x.shape
+    return load().yan_per_token_cast_to_fp8(x.data_ptr(), int(x.dtype == torch.float32), q.data_ptr(), scales.data_ptr(),
+                                            scales.stride(0), scales.stride(1), m, k, _stream_handle())
+
+
+def per_block_cast_to_fp8(w: torch.Tensor, q: torch.Tensor, scales: torch.Tensor) -> int:
+    n, k = w.shape
+    return load().yan_per_block_cast_to_fp8(w.data_ptr(), int(w.dtype == torch.float32), q.data_ptr(), scales.data_ptr(),
+                                            n, k, _stream_handle())
 
 
 def select_tile(op: int, m: int, n: int, k: int, num_cus: int):

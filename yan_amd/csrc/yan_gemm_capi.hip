@@ -5,6 +5,7 @@
 #include "gemm/bf16_gemm.hpp"
 #include "gemm/fp8_gemm.hpp"
 #include "gemm/fp8_gemm_skinny.hpp"
+#include "gemm/fp8_cast.hpp"
 
 namespace {
 
@@ -159,6 +160,19 @@ int yan_m_grouped_gemm_fp8_fp8_bf16_nt_masked(const void* lhs, const float* lhs_
     return int(hipErrorInvalidValue);
 }
 
+int yan_per_token_cast_to_fp8(const void* x, int x_is_fp32, void* q, float* scales, long long scales_stride_m,
+                              long long scales_stride_k, int m, int k, void* stream) {
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (x_is_fp32) return int(yan::launch_per_token_cast(static_cast<const float*>(x), q, scales, scales_stride_m, scales_stride_k, m, k, s));
+    return int(yan::launch_per_token_cast(static_cast<const __bf16*>(x), q, scales, scales_stride_m, scales_stride_k, m, k, s));
+}
+
+int yan_per_block_cast_to_fp8(const void* w, int w_is_fp32, void* q, float* scales, int n, int k, void* stream) {
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (w_is_fp32) return int(yan::launch_per_block_cast(static_cast<const float*>(w), q, scales, n, k, s));
+    return int(yan::launch_per_block_cast(static_cast<const __bf16*>(w), q, scales, n, k, s));
+}
+
 int yan_gemm_select_tile(int op, int m, int n, int k, int num_cus, int* block_m, int* block_n) {
     (void)k;
     if (!block_m || !block_n || num_cus <= 0) return 1;
@@ -172,6 +186,6 @@ int yan_gemm_select_tile(int op, int m, int n, int k, int num_cus, int* block_m,
     return 0;
 }
 
-const char* yan_gemm_version(void) { return "yan-gemm gfx950 6 dense + 8 fp8 tile variants + 2 weight-streaming + 1 split-K fp8 variants + 12 grouped fp8 variants"; }
+const char* yan_gemm_version(void) { return "yan-gemm gfx950 6 dense + 8 fp8 tile variants + 2 weight-streaming + 1 split-K fp8 variants + 12 grouped fp8 variants + 4 quantiser kernels"; }
 
 } // extern "C"

@@ -184,7 +184,15 @@ def prebuild_jit_kernels(num_cus: int = 256, verbose: bool = False) -> int:
             rt = build(name, arg_defs, code)
             if verbose:
                 print(f'built {name} {keys} -> {rt.path}')
-    from .jit_kernels import m_grouped_gemm
+    from .jit_kernels import fp8_cast, m_grouped_gemm
+    for kind in ('per_token', 'per_block'):
+        for dtype in (torch.bfloat16, torch.float32):
+            name, keys, arg_defs, code_template = fp8_cast.cast_kernel_plan(kind, dtype)
+            code = generate(fp8_cast.includes, arg_defs, cpp_format(code_template, keys))
+            seen.add((name, code))
+            rt = build(name, arg_defs, code)
+            if verbose:
+                print(f'built {name} {keys} -> {rt.path}')
     for rows, n, k, pad_blocks in GROUPED_CONTIGUOUS_TEST_CASES:
         m = sum((r + 127) // 128 * 128 for r in rows) + 128 * pad_blocks
         plans = [m_grouped_gemm.grouped_kernel_plan('GroupedContiguous', len(rows), m, n, k, num_cus)]
