@@ -309,6 +309,27 @@ def test_fp8_outlier_16384_cubed():
 
 
 # ----------------------------------------------------------------------------- the ahead-of-time C-ABI library
+def test_tuner_times_a_space_of_tiles_on_the_device():
+    """The empirical half of compile_and_tune (yan/jit_kernels/tuner.py:24-69): every candidate of `space` is built, run
+    once, timed over back-to-back launches after a cache flush, and the fastest is kept and memoised."""
+    from yan_amd.jit_kernels import bf16_gemm
+    from yan_amd.jit_kernels.tuner import JITTuner
+    m = n = k = 1024
+    a, b, c = testing.make_bf16_case(m, n, k, seed=3, device='cuda')
+    args = (m, n, k, a, b, c, torch.cuda.current_stream())
+    space = tuple({'BLOCK_M': bm, 'BLOCK_N': bn} for bm, bn in ((256, 256), (128, 128), (64, 64)))
+    tuner = JITTuner()
+    kw = dict(name='gemm_bf16_tn', keys={'NUM_STAGES': 2}, space=space, includes=bf16_gemm.includes,
+              arg_defs=bf16_gemm._arg_defs(torch.bfloat16), template=bf16_gemm.template, args=args)
+    best = tuner.compile_and_tune(**kw)
+    assert tuner.compile_and_tune(**kw) is best                       # memoised
+    chosen = list(tuner.tuned_keys.values())[0]
+    assert (chosen['BLOCK_M'], chosen['BLOCK_N']) in ((256, 256), (128, 128), (64, 64))
+    c.zero_()
+    assert best(*args) == 0
+    assert float(yan.calc_diff(c.float(), a.float() @ b.float().t())) < 1e-5
+
+
 # ----------------------------------------------------------------------------- quantisers in front of the FP8 GEMM
 def _oracle_per_token(x):
     q, s_ = oracle.per_token_cast_to_fp8(x.float().numpy())
