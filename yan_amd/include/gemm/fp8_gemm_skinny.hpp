@@ -324,14 +324,20 @@ inline SplitKScratch& splitk_scratch() {
     return scratch;
 }
 
-// K blocks per split and number of splits for n weight rows and k depth on `num_cus` compute units: enough splits to
-// give every CU `wgs_per_cu` workgroups, at most `kbs_max` K blocks per split (the LDS slab).
+// K blocks per split and number of splits for n weight rows and k depth on `num_cus` compute units, `wgs_per_cu`
+// workgroups resident per unit, at most `kbs_max` K blocks per split (the LDS slab). Every candidate split count is
+// priced as rounds of workgroups times (K blocks per workgroup + a fixed cost of about 6 blocks for launch, meeting
+// and tail) and the cheapest wins: it fills the chip once where it can and never spills a few workgroups into a
+// second round.
 inline void splitk_plan(int n, int k, int num_cus, int kbs_max, int wgs_per_cu, int* kbs, int* splits) {
-    const int nkb = k / 128, n_tiles = ceil_div(n, 64);
-    int s = max(ceil_div(nkb, kbs_max), ceil_div(num_cus * wgs_per_cu, n_tiles));
-    s = min(s, nkb);
-    *kbs = ceil_div(nkb, s);
-    *splits = ceil_div(nkb, *kbs);
+    const int nkb = k / 128, n_tiles = ceil_div(n, 64), slots = num_cus * wgs_per_cu;
+    int best_cost = 1 << 30;
+    for (int s = ceil_div(nkb, kbs_max); s <= nkb; ++s) {
+        const int per_split = ceil_div(nkb, s), used = ceil_div(nkb, per_split);
+        if (used != s) continue;                            // the same work with fewer workgroups was priced already
+        const int cost = ceil_div(n_tiles * s, slots) * (per_split + 6);
+        if (cost < best_cost) { best_cost = cost; *kbs = per_split; *splits = s; }
+    }
 }
 
 template <int SHAPE_N, int SHAPE_K, int TM, int KBS_MAX = 8>
