@@ -83,8 +83,9 @@ YAN_API int yan_m_grouped_gemm_fp8_fp8_bf16_nt_masked(const void* lhs, const flo
                                               int m_max, int expected_m, int n, int k, void* stream, int num_sms);
 
 /* Quantisers producing the GEMM's operands in one pass over HBM: amax over the group clamped at 1e-4,
- * q = e4m3(x * (448 / amax)) with round to nearest even, scale = amax / 448; bit-identical to the torch op chain
- * callers of this convention use. Sources are bf16 (x_is_fp32 == 0) or fp32, row-major, k % 128 == 0.
+ * q = e4m3(x * (448 / amax)) with round to nearest even, scale = amax / 448, both quotients correctly rounded fp32
+ * divisions (the op chain callers of this convention type in torch, which itself rounds 448 / amax an ulp differently
+ * for some amax). Sources are bf16 (x_is_fp32 == 0) or fp32, row-major, k % 128 == 0.
  * per-token: groups of 1 x 128; scale (i, kb) is written to scales[i*scales_stride_m + kb*scales_stride_k]
  *            ((k/128, 1) for row-major, (1, m) for the token-contiguous layout the GEMM reads fastest).
  * per-block: groups of 128 x 128 (a ragged last block of rows uses the rows that exist); scales [ceil(n/128)][k/128].

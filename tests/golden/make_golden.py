@@ -1,4 +1,5 @@
-"""Writes tests/golden/gemm_small.npz: small seeded inputs and expected outputs for both GEMMs.
+"""Writes tests/golden/gemm_small.npz (small seeded inputs and expected outputs for both GEMMs) and
+tests/golden/grouped_cast_small.npz (the grouped FP8 GEMM layouts and the two quantisers).
 
 The reference cannot produce these (no FP8 entry point, CUDA-only kernels, no fixtures of its own), so the
 expected values come from the closed forms in oracle/gemm_oracle.py evaluated in fp64, cross-checked here against
@@ -42,6 +43,37 @@ def main():
     assert np.array_equal(iexp, c_oracle.gemm_fp8_nt(ia, isa, ib, isb))
     out.update(int_lhs=ia, int_lhs_scales=isa, int_rhs=ib, int_rhs_scales=isb, int_expected=iexp)
     path = os.path.join(ROOT, 'tests', 'golden', 'gemm_small.npz')
+    np.savez_compressed(path, **out)
+    print('wrote', path, os.path.getsize(path), 'bytes')
+
+    out = {}
+    # quantisers: bf16 source, 130 x 256 (a ragged second block of rows for the per-block form), one all-zero group
+    src = (rng.standard_normal((130, 256)) * 2.5).astype(np.float32)
+    src[7, 128:] = 0
+    bits = oracle.f32_to_bf16_bits(src)
+    srcf = oracle.bf16_bits_to_f32(bits)
+    tq, ts = oracle.per_token_cast_to_fp8(srcf)
+    bq, bs = oracle.per_block_cast_to_fp8(srcf)
+    out.update(cast_src_bf16_bits=bits, per_token_codes=tq, per_token_scales=ts, per_block_codes=bq, per_block_scales=bs)
+    # grouped contiguous, exact integers with power-of-two scales: two groups of 128 rows and one block of padding
+    # rows (index -1), n = 192, k = 256; masked: two groups of 40 rows, 40 and 7 of them valid
+    G, n, k = 2, 192, 256
+    wb = np.stack([oracle.e4m3fn_encode(rng.integers(-4, 5, size=(n, k)).astype(np.float32)) for _ in range(G)])
+    wsb = (2.0 ** rng.integers(-2, 3, size=(G, 2, 2))).astype(np.float32)
+    xa = oracle.e4m3fn_encode(rng.integers(-4, 5, size=(384, k)).astype(np.float32))
+    xsa = (2.0 ** rng.integers(-2, 3, size=(384, 2))).astype(np.float32)
+    idx = np.repeat(np.array([1, 0, -1], dtype=np.int32), 128)
+    cexp = oracle.m_grouped_gemm_contiguous_ref(xa, xsa, wb, wsb, idx)
+    for i in (0, 127, 128, 255):
+        assert np.array_equal(cexp[i:i + 1], c_oracle.gemm_fp8_nt(xa[i:i + 1], xsa[i:i + 1], wb[idx[i]], wsb[idx[i]]))
+    ma = np.stack([oracle.e4m3fn_encode(rng.integers(-4, 5, size=(40, k)).astype(np.float32)) for _ in range(G)])
+    msa = (2.0 ** rng.integers(-2, 3, size=(G, 40, 2))).astype(np.float32)
+    masked = np.array([40, 7], dtype=np.int32)
+    mexp = oracle.m_grouped_gemm_masked_ref(ma, msa, wb, wsb, masked)
+    assert np.array_equal(mexp[1, :7], c_oracle.gemm_fp8_nt(ma[1, :7], msa[1, :7], wb[1], wsb[1])) and not mexp[1, 7:].any()
+    out.update(grouped_rhs=wb, grouped_rhs_scales=wsb, contiguous_lhs=xa, contiguous_lhs_scales=xsa, contiguous_m_indices=idx,
+               contiguous_expected=cexp, masked_lhs=ma, masked_lhs_scales=msa, masked_m=masked, masked_expected=mexp)
+    path = os.path.join(ROOT, 'tests', 'golden', 'grouped_cast_small.npz')
     np.savez_compressed(path, **out)
     print('wrote', path, os.path.getsize(path), 'bytes')
 

@@ -114,7 +114,8 @@ def test_quantisers_bounds_and_roundtrip(dist):
 def test_quantisers_match_package_harness():
     from yan_amd import testing
     g = torch.Generator().manual_seed(5)
-    x, w = torch.randn(48, 256, generator=g), torch.randn(160, 256, generator=g)
+    # bf16-valued sources: few mantissa bits, so x * factor lands exactly on rounding ties now and then
+    x, w = torch.randn(48, 256, generator=g).bfloat16().float(), torch.randn(160, 256, generator=g).bfloat16().float()
     qa, sa = testing.per_token_cast_to_fp8(x)
     qb, sb = testing.per_block_cast_to_fp8(w)
     oa, osa = oracle.per_token_cast_to_fp8(x.numpy())
@@ -293,3 +294,27 @@ def test_golden_fixtures_reproduce(repo_root):
     assert np.array_equal(oracle.gemm_bf16_tn_ref(a, b, np.float64), z['bf16_expected_f64'])
     assert np.allclose(c_oracle.gemm_bf16_tn(z['bf16_a_bits'], z['bf16_b_bits']), z['bf16_expected_f64'], rtol=1e-12, atol=1e-12)
     assert np.array_equal(z['int_expected'], oracle.gemm_fp8_block_scaled_ref(z['int_lhs'], z['int_lhs_scales'], z['int_rhs'], z['int_rhs_scales']))
+
+
+def test_grouped_and_cast_fixtures_reproduce(repo_root):
+    import os
+    z = np.load(os.path.join(repo_root, 'tests', 'golden', 'grouped_cast_small.npz'))
+    src = oracle.bf16_bits_to_f32(z['cast_src_bf16_bits'])
+    tq, ts = oracle.per_token_cast_to_fp8(src)
+    bq, bs = oracle.per_block_cast_to_fp8(src)
+    assert np.array_equal(tq, z['per_token_codes']) and np.array_equal(ts, z['per_token_scales'])
+    assert np.array_equal(bq, z['per_block_codes']) and np.array_equal(bs, z['per_block_scales'])
+    # torch's op chain on the same source: `448.0 / amax` is evaluated there as reciprocal(amax) * 448, one ulp away
+    # from the correctly rounded quotient for some amax, so a code moves where x * factor lands on a rounding boundary
+    # (bf16-valued sources make exact ties common); the scales, a plain division, are identical
+    xt = torch.from_numpy(src)
+    amax = xt.view(130, 2, 128).abs().amax(dim=2).clamp(1e-4)
+    q = (xt.view(130, 2, 128) * (448.0 / amax).unsqueeze(2)).to(torch.float8_e4m3fn).view(130, 256)
+    moved = q.view(torch.uint8).numpy() != z['per_token_codes']
+    assert moved.mean() < 2e-3 and np.array_equal((amax / 448.0).numpy(), z['per_token_scales'])
+    exact = (xt.view(130, 2, 128) * (torch.tensor(448.0) / amax).unsqueeze(2)).to(torch.float8_e4m3fn).view(130, 256)
+    assert np.array_equal(exact.view(torch.uint8).numpy(), z['per_token_codes'])      # with a true division: bit for bit
+    assert np.array_equal(oracle.m_grouped_gemm_contiguous_ref(z['contiguous_lhs'], z['contiguous_lhs_scales'], z['grouped_rhs'],
+                                                               z['grouped_rhs_scales'], z['contiguous_m_indices']), z['contiguous_expected'])
+    assert np.array_equal(oracle.m_grouped_gemm_masked_ref(z['masked_lhs'], z['masked_lhs_scales'], z['grouped_rhs'],
+                                                           z['grouped_rhs_scales'], z['masked_m']), z['masked_expected'])

@@ -6,9 +6,9 @@
 //
 // This is the step in front of the GEMM entry whose operand names the reference fixes
 // (yan/jit_kernels/gemm.py:23-30: lhs, lhs_scales, rhs, rhs_scales); the reference itself has no quantiser. The
-// arithmetic is written so that the results are bit-identical to the torch recipe
-// `(x.float() * (448 / amax)).to(torch.float8_e4m3fn)`, `amax / 448`: fp32 IEEE divisions, one fp32 multiply,
-// round-to-nearest-even conversion.
+// arithmetic is the recipe callers of this convention type in torch, `(x.float() * (448 / amax)).to(float8_e4m3fn)`
+// and `amax / 448`, with both quotients correctly rounded: fp32 IEEE divisions, one fp32 multiply, round-to-nearest-
+// even conversion. (torch itself evaluates `448.0 / amax` as reciprocal(amax) * 448, an ulp away for some amax.)
 //
 // Both kernels are bound by HBM traffic: (2 or 4) bytes read + 1 byte written per element, plus 4 bytes per
 // group. Sixteen lanes own one 128-element group at a time, 8 elements per lane, so a wave reads 1 KB (bf16) or

@@ -3,7 +3,10 @@
 The reference names the GEMM's operands (`lhs, lhs_scales, rhs, rhs_scales`, `yan/jit_kernels/gemm.py:23-30`) and has
 no code that produces them; callers of this convention build them with a chain of torch ops
 (`amax = |x|.view(m, -1, 128).amax(-1).clamp(1e-4)`, `q = (x * (448 / amax)).to(float8_e4m3fn)`, `scale = amax / 448`).
-The two entries here do the same arithmetic in one kernel each, one pass over HBM, with bit-identical results.
+The two entries here do the same arithmetic in one kernel each, one pass over HBM. Both quotients are correctly
+rounded fp32 divisions; torch evaluates `448.0 / amax` as `reciprocal(amax) * 448`, which is an ulp away for some
+amax and moves a code where `x * factor` lands on a rounding boundary. With true tensor / tensor divisions the torch
+chain and these kernels agree bit for bit.
 """
 from typing import Tuple
 

@@ -1,7 +1,9 @@
 """Harness-side helpers shared by tests, the smoke entry and the benchmark: FP8 quantisers in the DeepGEMM
 convention and seeded constructors for the benchmark configurations. The reference defines neither (its FP8 path
 has no Python entry or test); the recipes are the ones the benchmark configurations name:
-per-token 1x128 / per-block 128x128 amax, clamp 1e-4, x * 448 / amax -> e4m3fn, scale = amax / 448.
+per-token 1x128 / per-block 128x128 amax, clamp 1e-4, x * (448 / amax) -> e4m3fn, scale = amax / 448.
+Both quotients are tensor / tensor divisions on purpose: torch turns `448.0 / amax` into reciprocal(amax) * 448 and,
+on the GPU, `amax / 448.0` into amax * (1 / 448), each an ulp away from the correctly rounded quotient for some inputs.
 """
 from typing import Tuple
 
@@ -16,8 +18,9 @@ def per_token_cast_to_fp8(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
     m, k = x.shape
     xv = x.float().view(m, k // 128, 128)
     amax = xv.abs().amax(dim=2).clamp(1e-4)
-    q = (xv * (FP8_MAX / amax).unsqueeze(2)).to(torch.float8_e4m3fn)
-    return q.view(m, k), amax / FP8_MAX
+    top = torch.full_like(amax, FP8_MAX)
+    q = (xv * (top / amax).unsqueeze(2)).to(torch.float8_e4m3fn)
+    return q.view(m, k), amax / top
 
 
 def per_block_cast_to_fp8(w: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
@@ -29,8 +32,9 @@ def per_block_cast_to_fp8(w: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
     wp[:n] = w
     wv = wp.view(n_pad // 128, 128, k // 128, 128)
     amax = wv.abs().amax(dim=(1, 3)).clamp(1e-4)
-    q = (wv * (FP8_MAX / amax)[:, None, :, None]).to(torch.float8_e4m3fn)
-    return q.view(n_pad, k)[:n].contiguous(), amax / FP8_MAX
+    top = torch.full_like(amax, FP8_MAX)
+    q = (wv * (top / amax)[:, None, :, None]).to(torch.float8_e4m3fn)
+    return q.view(n_pad, k)[:n].contiguous(), amax / top
 
 
 def dequant_lhs(q: torch.Tensor, scales: torch.Tensor) -> torch.Tensor:
