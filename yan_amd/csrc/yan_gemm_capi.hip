@@ -107,7 +107,7 @@ int yan_gemm_fp8_fp8_bf16_nt(const void* lhs, const float* lhs_scales, long long
     pick(kFp8Tiles, m, n, cus, &bm, &bn);
 #define YAN_FP8_CASE(BM, BN)                                                                                         \
     if (bm == BM && bn == BN)                                                                                        \
-        return int(yan::Gemm<0, 0, BM, BN, 128, 1, 2, 1, yan::GemmType::Normal>::run_sized(                          \
+        return int(yan::Gemm<0, 0, BM, BN, 128, 1, yan::Fp8TileConfig<BM, BN>::MAX_RING_STAGES, 1, yan::GemmType::Normal>::run_sized(                          \
             o, lhs, lhs_scales, int(lhs_scales_stride_m), int(lhs_scales_stride_k), rhs, rhs_scales, m, n, k, s, num_sms, 0));
     YAN_FP8_CASE(256, 256) YAN_FP8_CASE(256, 128) YAN_FP8_CASE(128, 256) YAN_FP8_CASE(128, 128) YAN_FP8_CASE(64, 128) YAN_FP8_CASE(64, 64)
     YAN_FP8_CASE(64, 32) YAN_FP8_CASE(64, 16)
@@ -128,7 +128,7 @@ int yan_m_grouped_gemm_fp8_fp8_bf16_nt_contiguous(const void* lhs, const float* 
     pick_grouped(m, n, cus, 1, 128, num_groups, &bm, &bn);
 #define YAN_GROUPED_CASE(BM, BN)                                                                                     \
     if (bm == BM && bn == BN)                                                                                        \
-        return int(yan::Gemm<0, 0, BM, BN, 128, 1, 2, 1, yan::GemmType::GroupedContiguous>::run_grouped(             \
+        return int(yan::Gemm<0, 0, BM, BN, 128, 1, yan::Fp8TileConfig<BM, BN>::MAX_RING_STAGES, 1, yan::GemmType::GroupedContiguous>::run_grouped(             \
             static_cast<__hip_bfloat16*>(out), lhs, lhs_scales, int(lhs_scales_stride_m), int(lhs_scales_stride_k), 0, rhs, \
             rhs_scales, m_indices, num_groups, m, n, k, static_cast<hipStream_t>(stream)));
     YAN_GROUPED_CASE(256, 256) YAN_GROUPED_CASE(256, 128) YAN_GROUPED_CASE(128, 256) YAN_GROUPED_CASE(128, 128)
@@ -151,7 +151,7 @@ int yan_m_grouped_gemm_fp8_fp8_bf16_nt_masked(const void* lhs, const float* lhs_
     pick_grouped(expected_m < m_max ? expected_m : m_max, n, cus, num_groups, 0, 1, &bm, &bn);
 #define YAN_GROUPED_CASE(BM, BN)                                                                                     \
     if (bm == BM && bn == BN)                                                                                        \
-        return int(yan::Gemm<0, 0, BM, BN, 128, 1, 2, 1, yan::GemmType::GroupedMasked>::run_grouped(                 \
+        return int(yan::Gemm<0, 0, BM, BN, 128, 1, yan::Fp8TileConfig<BM, BN>::MAX_RING_STAGES, 1, yan::GemmType::GroupedMasked>::run_grouped(                 \
             static_cast<__hip_bfloat16*>(out), lhs, lhs_scales, int(lhs_scales_stride_m), int(lhs_scales_stride_k),  \
             int(lhs_scales_stride_g), rhs, rhs_scales, masked_m, num_groups, m_max, n, k, static_cast<hipStream_t>(stream)));
     YAN_GROUPED_CASE(256, 256) YAN_GROUPED_CASE(256, 128) YAN_GROUPED_CASE(128, 256) YAN_GROUPED_CASE(128, 128)

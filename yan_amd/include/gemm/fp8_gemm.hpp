@@ -45,6 +45,13 @@ struct Fp8TileConfig {
     static constexpr int  SCALE_B_PER_SLAB = UNIFORM_SCALE_B ? 1 : (WTN + 112) / 128 + 1;
     static constexpr int  LDS_BYTES = 2 * (BLOCK_M + BLOCK_N) * kRowBytes;
     static_assert(LDS_BYTES <= 160 * 1024, "two stages must fit the 160 KB LDS");
+    // Ring of more than two stages (small tiles, where one k-tile in flight cannot cover the memory latency): a stage
+    // also carries the k-tile's activation scales, one private copy per wave.
+    static constexpr int  RING_SCALE_BYTES = ceil_div(NUM_WAVES * BLOCK_M * 4, 1024) * 1024;
+    static constexpr int  RING_STAGE_BYTES = (BLOCK_M + BLOCK_N) * kRowBytes + RING_SCALE_BYTES;
+    static constexpr bool RING_CAPABLE = NUM_WAVES == 4 && BLOCK_M % 64 == 0 && BLOCK_M <= 128 &&
+                                         (BLOCK_M / 8) % NUM_WAVES == 0 && (BLOCK_N / 8) % NUM_WAVES == 0;
+    static constexpr int  MAX_RING_STAGES = RING_CAPABLE ? (160 * 1024 / RING_STAGE_BYTES < 8 ? 160 * 1024 / RING_STAGE_BYTES : 8) : 2;
 };
 
 // Normal:            lhs [m, K], rhs [N, K], out [m, N]; grouped_layout unused.
@@ -54,7 +61,8 @@ struct Fp8TileConfig {
 // GroupedMasked:     lhs [G, m, K], out [G, m, N], rhs as above; only the first grouped_layout[g] rows of group g
 //                    are computed; lhs_scales of group g start at g * sa_stride_g floats. The grid is G times the
 //                    grid of one [m, N] problem.
-template <int SHAPE_N, int SHAPE_K, int BLOCK_M, int BLOCK_N, GemmType kGemmType = GemmType::Normal>
+// STAGES: 2 = two LDS stages with the next k-tile's scales in registers; 3.. = a ring of that many stages.
+template <int SHAPE_N, int SHAPE_K, int BLOCK_M, int BLOCK_N, GemmType kGemmType = GemmType::Normal, int STAGES = 2>
 __global__ void __launch_bounds__((get_num_waves(BLOCK_M, BLOCK_N) * kWaveSize))
 fp8_gemm_kernel(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_scales,
                 const uint8_t* __restrict__ rhs, const float* __restrict__ rhs_scales,
@@ -69,10 +77,7 @@ fp8_gemm_kernel(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_s
     const int N = SHAPE_N ? SHAPE_N : n_rt, K = SHAPE_K ? SHAPE_K : k_rt;
     const int NUM_K_BLOCKS = K / 128, NUM_N_BLOCKS = ceil_div(N, 128);
 
-    __shared__ __attribute__((aligned(1024))) uint8_t lds_a0[BLOCK_M * kRowBytes];
-    __shared__ __attribute__((aligned(1024))) uint8_t lds_b0[BLOCK_N * kRowBytes];
-    __shared__ __attribute__((aligned(1024))) uint8_t lds_a1[BLOCK_M * kRowBytes];
-    __shared__ __attribute__((aligned(1024))) uint8_t lds_b1[BLOCK_N * kRowBytes];
+    static_assert(STAGES == 2 || (STAGES >= 3 && STAGES <= Cfg::MAX_RING_STAGES), "no ring of this depth for this tile");
 
     const XcdTileScheduler<> sched(m, N, BLOCK_M, BLOCK_N);
     int bid = blockIdx.x;
@@ -145,12 +150,15 @@ fp8_gemm_kernel(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_s
 
     float sa_next[TM];     // activation scales of the k-tile in flight
     float sb_next[NB];     // weight scales of the k-tile in flight (wave-uniform)
+    auto load_weight_scales = [&](int kb) {
+#pragma unroll
+        for (int b = 0; b < NB; ++b) sb_next[b] = rhs_scales[min(base_blk + b, NUM_N_BLOCKS - 1) * NUM_K_BLOCKS + kb];
+    };
     auto load_scales = [&](int kb) {
 #pragma unroll
         for (int j = 0; j < TM; ++j)
             sa_next[j] = buffer_load_f32(rsrc_sa, sa_voff, (kb * sa_stride_k + j * 16 * sa_stride_m) * 4);
-#pragma unroll
-        for (int b = 0; b < NB; ++b) sb_next[b] = rhs_scales[min(base_blk + b, NUM_N_BLOCKS - 1) * NUM_K_BLOCKS + kb];
+        load_weight_scales(kb);
     };
 
     // One k-tile: TN x TM atoms, software-pipelined by hand. Step t issues the MFMA of atom t (fresh zero
@@ -240,6 +248,11 @@ fp8_gemm_kernel(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_s
     for (int i = 0; i < TN; ++i)
 #pragma unroll
         for (int j = 0; j < TM; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+    if constexpr (STAGES == 2) {
+    __shared__ __attribute__((aligned(1024))) uint8_t lds_a0[BLOCK_M * kRowBytes];
+    __shared__ __attribute__((aligned(1024))) uint8_t lds_b0[BLOCK_N * kRowBytes];
+    __shared__ __attribute__((aligned(1024))) uint8_t lds_a1[BLOCK_M * kRowBytes];
+    __shared__ __attribute__((aligned(1024))) uint8_t lds_b1[BLOCK_N * kRowBytes];
     stage_a.issue(rsrc_a, lds_a0, 0, wave);
     stage_b.issue(rsrc_b, lds_b0, 0, wave);
     load_scales(0);
@@ -248,6 +261,55 @@ fp8_gemm_kernel(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_s
         k_step(kb + 1, lds_a1, lds_b1, lds_a0, lds_b0);
     }
     if (NUM_K_BLOCKS % 2 == 1) k_step(NUM_K_BLOCKS - 1, lds_a0, lds_b0, lds_a1, lds_b1);
+    } else {
+    // Ring of STAGES stages, STAGES - 1 k-tiles in flight: what a small tile needs when the problem is bound by
+    // streaming its operands and one k-tile of prefetch cannot cover the memory latency. Every wave issues the same
+    // number of copies per k-tile (OPS), in the same order, so "k-tile kb has landed" is "at most (STAGES - 2) * OPS
+    // of my copies are outstanding". The activation scales of a k-tile travel through the stage as well (a register
+    // load between the copies would make the in-order counter wait for every older copy); each wave keeps a private
+    // copy of the tile's BLOCK_M scales, written by one full-width instruction per 64 rows.
+    constexpr int STAGE_BYTES = Cfg::RING_STAGE_BYTES, TILE_BYTES = (BLOCK_M + BLOCK_N) * kRowBytes;
+    constexpr int SCALE_OPS = BLOCK_M / 64, OPS = StA::PASSES + StB::PASSES + SCALE_OPS;
+    static_assert(Cfg::RING_CAPABLE && (STAGES - 2) * OPS <= 63 && STAGES * STAGE_BYTES <= 160 * 1024);
+    __shared__ __attribute__((aligned(1024))) uint8_t ring[STAGES * STAGE_BYTES];
+    const uint32_t scale_voff = uint32_t(m0 + lane) * sa_stride_m * 4;
+    auto issue_op = [&](int d, int kb, uint8_t* stage) {
+        if (d < StA::PASSES) stage_a.issue_pass(rsrc_a, stage, kb * kRowBytes, wave, d);
+        else if (d < StA::PASSES + StB::PASSES) stage_b.issue_pass(rsrc_b, stage + BLOCK_M * kRowBytes, kb * kRowBytes, wave, d - StA::PASSES);
+        else {
+            const int part = d - StA::PASSES - StB::PASSES;       // rows m0 + 64 * part + lane
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_sa, YAN_LDS_PTR(stage + TILE_BYTES + (wave * BLOCK_M + part * 64) * 4), 4,
+                                                     scale_voff, (kb * sa_stride_k + part * 64 * sa_stride_m) * 4, 0, 0);
+        }
+    };
+#pragma unroll
+    for (int t = 0; t < STAGES - 1; ++t)
+#pragma unroll
+        for (int d = 0; d < OPS; ++d) issue_op(d, t, ring + t * STAGE_BYTES);
+    load_weight_scales(0);
+    int st = 0;
+    for (int kb = 0; kb < NUM_K_BLOCKS; ++kb) {
+#pragma unroll
+        for (int b = 0; b < NB; ++b) sb_cur[b] = sb_next[b];
+        __builtin_amdgcn_s_waitcnt(waitcnt_imm((STAGES - 2) * OPS, kNoWaitLgkm));
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        load_weight_scales(min(kb + 1, NUM_K_BLOCKS - 1));
+        const uint8_t* cur = ring + st * STAGE_BYTES;
+        const int st_nxt = st + STAGES - 1 >= STAGES ? st - 1 : st + STAGES - 1;
+        uint8_t* nxt = ring + st_nxt * STAGE_BYTES;
+        const float* my_scales = reinterpret_cast<const float*>(cur + TILE_BYTES) + wave * BLOCK_M + wm * Cfg::WTM + col;
+#pragma unroll
+        for (int j = 0; j < TM; ++j) sa_cur[j] = my_scales[j * 16];
+        compute_tile(cur, cur + BLOCK_M * kRowBytes, sa_cur, sb_cur, [&](int row) {
+#pragma unroll
+            for (int d = 0; d < OPS; ++d)
+                if (d * SPREAD_ROWS / OPS == row) issue_op(d, kb + STAGES - 1, nxt);
+        });
+        st = st + 1 == STAGES ? 0 : st + 1;
+    }
+    }
 
     // Epilogue: the 4 registers of atom (i, j) are n = n_slab + 16i + 4g + {0..3} of row m = m_slab + 16j + col.
 #pragma unroll
@@ -267,9 +329,9 @@ fp8_gemm_kernel(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_s
 
 // Host side of the kernel, shaped after the class the reference's JIT template instantiates
 // (yan/jit_kernels/gemm.py:20-30: Gemm<N, K, BLOCK_M, BLOCK_N, 128, 1, kNumStages, kNumTMAMulticast, Normal>::run).
-// BLOCK_K is fixed at 128; kNumGroups, kNumStages and kNumTMAMulticast are accepted and unused: the kernel always
-// runs two LDS stages and gfx950 has no multicast copy. `num_sms` and `smem_size` are accepted likewise (one
-// workgroup per tile, static LDS).
+// BLOCK_K is fixed at 128. kNumStages is the number of LDS stages: 2, or a ring of 3 .. Fp8TileConfig::MAX_RING_STAGES
+// for the small tiles that support one. kNumTMAMulticast is accepted and unused (gfx950 has no multicast copy), as
+// are `num_sms` and `smem_size` (one workgroup per tile, static LDS).
 template <uint32_t SHAPE_N, uint32_t SHAPE_K, uint32_t BLOCK_M, uint32_t BLOCK_N, uint32_t BLOCK_K,
           uint32_t kNumGroups, uint32_t kNumStages, uint32_t kNumTMAMulticast, GemmType kGemmType>
 class Gemm {
@@ -306,7 +368,7 @@ public:
         const XcdTileScheduler<> sched(m, n, BLOCK_M, BLOCK_N);
         const uint64_t grid = uint64_t(sched.grid_size()) * (kGemmType == GemmType::GroupedMasked ? num_groups : 1);
         if (grid >= kOutOfRange) return hipErrorInvalidValue;
-        hipLaunchKernelGGL((fp8_gemm_kernel<SHAPE_N, SHAPE_K, BLOCK_M, BLOCK_N, kGemmType>), dim3(uint32_t(grid)),
+        hipLaunchKernelGGL((fp8_gemm_kernel<SHAPE_N, SHAPE_K, BLOCK_M, BLOCK_N, kGemmType, int(kNumStages)>), dim3(uint32_t(grid)),
                            dim3(Cfg::NUM_WAVES * kWaveSize), 0, stream, static_cast<const uint8_t*>(lhs), lhs_scales,
                            static_cast<const uint8_t*>(rhs), rhs_scales, reinterpret_cast<__bf16*>(out), m, n, k,
                            lhs_scales_stride_m, lhs_scales_stride_k, grouped_layout, lhs_scales_stride_g);
@@ -327,7 +389,7 @@ public:
         if (m_pad * k >= kOutOfRange || n_pad * k >= kOutOfRange) return hipErrorInvalidValue;
         using Cfg = Fp8TileConfig<BLOCK_M, BLOCK_N>;
         const XcdTileScheduler<> sched(m, n, BLOCK_M, BLOCK_N);
-        hipLaunchKernelGGL((fp8_gemm_kernel<SHAPE_N, SHAPE_K, BLOCK_M, BLOCK_N>), dim3(sched.grid_size()),
+        hipLaunchKernelGGL((fp8_gemm_kernel<SHAPE_N, SHAPE_K, BLOCK_M, BLOCK_N, GemmType::Normal, int(kNumStages)>), dim3(sched.grid_size()),
                            dim3(Cfg::NUM_WAVES * kWaveSize), 0, stream, static_cast<const uint8_t*>(lhs), lhs_scales,
                            static_cast<const uint8_t*>(rhs), rhs_scales, reinterpret_cast<__bf16*>(out), m, n, k,
                            lhs_scales_stride_m, lhs_scales_stride_k);

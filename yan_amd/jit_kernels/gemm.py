@@ -13,7 +13,7 @@ from typing import Tuple
 
 import torch
 
-from .heuristics import get_best_fp8_config, get_skinny_fp8_config
+from .heuristics import get_best_fp8_config, get_fp8_num_stages, get_skinny_fp8_config
 from .tuner import jit_tuner
 from .utils import get_num_sms, ceil_div, get_col_major_tensor
 
@@ -74,8 +74,9 @@ def fp8_kernel_plan(m: int, n: int, k: int, num_cus: int):
                 'NUM_WAVES': 8}
         return 'gemm_fp8_fp8_bf16_nt', keys, arg_defs, 8 * skinny_atoms * 64 * 16, skinny_template
     block_m, block_n = get_best_fp8_config(m, n, k, num_cus)
-    keys = {'N': n, 'K': k, 'BLOCK_M': block_m, 'BLOCK_N': block_n, 'NUM_STAGES': 2, 'NUM_TMA_MULTICAST': 1}
-    smem_size = 2 * (block_m + block_n) * 128
+    keys = {'N': n, 'K': k, 'BLOCK_M': block_m, 'BLOCK_N': block_n, 'NUM_STAGES': get_fp8_num_stages(block_m, block_n),
+            'NUM_TMA_MULTICAST': 1}
+    smem_size = keys['NUM_STAGES'] * (block_m + block_n) * 128
     return 'gemm_fp8_fp8_bf16_nt', keys, arg_defs, smem_size, template
 
 

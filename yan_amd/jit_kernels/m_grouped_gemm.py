@@ -12,7 +12,7 @@ from typing import Tuple
 import torch
 
 from .gemm import includes
-from .heuristics import get_best_grouped_fp8_config
+from .heuristics import get_best_grouped_fp8_config, get_fp8_num_stages
 from .tuner import jit_tuner
 from .utils import ceil_div, get_m_alignment_for_contiguous_layout, get_num_sms
 
@@ -53,9 +53,10 @@ def grouped_kernel_plan(gemm_type: str, num_groups: int, m: int, n: int, k: int,
     else:
         block_m, block_n = get_best_grouped_fp8_config(m, n, k, num_cus, num_groups)
         name = 'm_grouped_gemm_fp8_fp8_bf16_nt'
-    keys = {'N': n, 'K': k, 'BLOCK_M': block_m, 'BLOCK_N': block_n, 'NUM_GROUPS': num_groups, 'NUM_STAGES': 2,
+    keys = {'N': n, 'K': k, 'BLOCK_M': block_m, 'BLOCK_N': block_n, 'NUM_GROUPS': num_groups,
+            'NUM_STAGES': get_fp8_num_stages(block_m, block_n),
             'NUM_TMA_MULTICAST': 1, 'GEMM_TYPE': gemm_type}
-    return name, keys, arg_defs, 2 * (block_m + block_n) * 128
+    return name, keys, arg_defs, keys['NUM_STAGES'] * (block_m + block_n) * 128
 
 
 def _launch(gemm_type, num_groups, plan_m, m, n, k, lhs, lhs_scales, rhs, rhs_scales, out, layout, strides):
