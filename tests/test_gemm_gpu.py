@@ -346,9 +346,10 @@ def test_tuner_times_a_space_of_tiles_on_the_device():
     m = n = k = 1024
     a, b, c = testing.make_bf16_case(m, n, k, seed=3, device='cuda')
     args = (m, n, k, a, b, c, torch.cuda.current_stream())
-    space = tuple({'BLOCK_M': bm, 'BLOCK_N': bn} for bm, bn in ((256, 256), (128, 128), (64, 64)))
+    from yan_amd.jit_kernels.heuristics import get_dense_num_stages
+    space = tuple({'BLOCK_M': bm, 'BLOCK_N': bn, 'NUM_STAGES': get_dense_num_stages(bm, bn)} for bm, bn in ((256, 256), (128, 128), (64, 64)))
     tuner = JITTuner()
-    kw = dict(name='gemm_bf16_tn', keys={'NUM_STAGES': 2}, space=space, includes=bf16_gemm.includes,
+    kw = dict(name='gemm_bf16_tn', keys={}, space=space, includes=bf16_gemm.includes,
               arg_defs=bf16_gemm._arg_defs(torch.bfloat16), template=bf16_gemm.template, args=args)
     best = tuner.compile_and_tune(**kw)
     assert tuner.compile_and_tune(**kw) is best                       # memoised

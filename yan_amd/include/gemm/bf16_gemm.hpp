@@ -38,19 +38,20 @@ struct DenseTileConfig {
     static_assert(WTN % 32 == 0 && WTM % 32 == 0, "wave slab must be a whole number of 32x32 atoms");
     static constexpr int LDS_BYTES = 2 * (BLOCK_M + BLOCK_N) * kRowBytes;
     static_assert(LDS_BYTES <= 160 * 1024, "two stages must fit the 160 KB LDS");
+    // Deepest ring of LDS stages the 160 KB hold for this tile (at most 8); 2 for the 256 x 256 tile.
+    static constexpr int STAGE_BYTES = (BLOCK_M + BLOCK_N) * kRowBytes;
+    static constexpr int MAX_STAGES  = 160 * 1024 / STAGE_BYTES < 8 ? 160 * 1024 / STAGE_BYTES : 8;
 };
 
-template <typename Atom, typename Elem, int BLOCK_M, int BLOCK_N>
+// STAGES: 2 = two LDS stages, one k-tile of prefetch; 3.. = a ring of that many stages with STAGES - 1 k-tiles in
+// flight, for the smaller tiles, which are picked when a problem is bound by streaming its operands.
+template <typename Atom, typename Elem, int BLOCK_M, int BLOCK_N, int STAGES>
 __device__ __forceinline__ void
 dense_gemm_body(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, Elem* __restrict__ C,
                 int m, int n, int k) {
     using Cfg = DenseTileConfig<BLOCK_M, BLOCK_N>;
     constexpr int NW = Cfg::NUM_WAVES, TN = Cfg::WTN / 32, TM = Cfg::WTM / 32;
-
-    __shared__ __attribute__((aligned(1024))) uint8_t lds_a0[BLOCK_M * kRowBytes];
-    __shared__ __attribute__((aligned(1024))) uint8_t lds_b0[BLOCK_N * kRowBytes];
-    __shared__ __attribute__((aligned(1024))) uint8_t lds_a1[BLOCK_M * kRowBytes];
-    __shared__ __attribute__((aligned(1024))) uint8_t lds_b1[BLOCK_N * kRowBytes];
+    static_assert(STAGES >= 2 && STAGES <= Cfg::MAX_STAGES, "this many stages do not fit the LDS");
 
     const XcdTileScheduler<> sched(m, n, BLOCK_M, BLOCK_N);
     const TileCoord tile = sched.tile_of(blockIdx.x);
@@ -157,14 +158,46 @@ dense_gemm_body(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, El
                 if (d * SPREAD_STEPS / NUM_COPIES == kk) copy_pass(d, kt + 1, a_nxt, b_nxt);
         });
     };
+    if constexpr (STAGES == 2) {
+        __shared__ __attribute__((aligned(1024))) uint8_t lds_a0[BLOCK_M * kRowBytes];
+        __shared__ __attribute__((aligned(1024))) uint8_t lds_b0[BLOCK_N * kRowBytes];
+        __shared__ __attribute__((aligned(1024))) uint8_t lds_a1[BLOCK_M * kRowBytes];
+        __shared__ __attribute__((aligned(1024))) uint8_t lds_b1[BLOCK_N * kRowBytes];
 #pragma unroll
-    for (int d = 0; d < NUM_COPIES; ++d) copy_pass(d, 0, lds_a0, lds_b0);
-    int kt = 0;
-    for (; kt + 1 < num_k_tiles; kt += 2) {
-        k_step(kt, lds_a0, lds_b0, lds_a1, lds_b1);
-        k_step(kt + 1, lds_a1, lds_b1, lds_a0, lds_b0);
+        for (int d = 0; d < NUM_COPIES; ++d) copy_pass(d, 0, lds_a0, lds_b0);
+        int kt = 0;
+        for (; kt + 1 < num_k_tiles; kt += 2) {
+            k_step(kt, lds_a0, lds_b0, lds_a1, lds_b1);
+            k_step(kt + 1, lds_a1, lds_b1, lds_a0, lds_b0);
+        }
+        if (kt < num_k_tiles) k_step(kt, lds_a0, lds_b0, lds_a1, lds_b1);
+    } else {
+        // Ring: every wave issues NUM_COPIES copies per k-tile, in the same order, so "k-tile kt has landed" is "at
+        // most (STAGES - 2) * NUM_COPIES of my copies are outstanding". The copies of k-tile kt + STAGES - 1 go to
+        // the stage that was consumed in iteration kt - 1, which every wave has left once it is past the barrier.
+        static_assert((BLOCK_M / 8) % NW == 0 && (BLOCK_N / 8) % NW == 0 && (STAGES - 2) * NUM_COPIES <= 63);
+        constexpr int STAGE_BYTES = Cfg::STAGE_BYTES;
+        __shared__ __attribute__((aligned(1024))) uint8_t ring[STAGES * STAGE_BYTES];
+#pragma unroll
+        for (int t = 0; t < STAGES - 1; ++t)
+#pragma unroll
+            for (int d = 0; d < NUM_COPIES; ++d) copy_pass(d, t, ring + t * STAGE_BYTES, ring + t * STAGE_BYTES + BLOCK_M * kRowBytes);
+        int st = 0;
+        for (int kt = 0; kt < num_k_tiles; ++kt) {
+            __builtin_amdgcn_s_waitcnt(waitcnt_imm((STAGES - 2) * NUM_COPIES, kNoWaitLgkm));
+            asm volatile("" ::: "memory");
+            __builtin_amdgcn_s_barrier();
+            asm volatile("" ::: "memory");
+            const uint8_t* cur = ring + st * STAGE_BYTES;
+            uint8_t* nxt = ring + (st == 0 ? STAGES - 1 : st - 1) * STAGE_BYTES;
+            compute_tile(cur, cur + BLOCK_M * kRowBytes, [&](int kk) {
+#pragma unroll
+                for (int d = 0; d < NUM_COPIES; ++d)
+                    if (d * SPREAD_STEPS / NUM_COPIES == kk) copy_pass(d, kt + STAGES - 1, nxt, nxt + BLOCK_M * kRowBytes);
+            });
+            st = st + 1 == STAGES ? 0 : st + 1;
+        }
     }
-    if (kt < num_k_tiles) k_step(kt, lds_a0, lds_b0, lds_a1, lds_b1);
 
     // Epilogue: registers 4*q .. 4*q+3 of an atom are n = 8*q + 4*g + {0,1,2,3} of column m = lane % 32.
     const int m_lane = m0 + wm * Cfg::WTM + lane % 32;
@@ -187,18 +220,18 @@ dense_gemm_body(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, El
     }
 }
 
-template <typename Atom, typename Elem, int BLOCK_M, int BLOCK_N>
+template <typename Atom, typename Elem, int BLOCK_M, int BLOCK_N, int STAGES>
 __global__ void __launch_bounds__(4 * kWaveSize)
 dense_gemm_mfma(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, Elem* __restrict__ C, int m, int n, int k) {
-    dense_gemm_body<Atom, Elem, BLOCK_M, BLOCK_N>(A, B, C, m, n, k);
+    dense_gemm_body<Atom, Elem, BLOCK_M, BLOCK_N, STAGES>(A, B, C, m, n, k);
 }
 
 // The fp16 flavour under the name of the reference's kernel (yan/include/gemm/cute_gemm.cuh:20), so that profiler
 // filters written for it (tests/test_cute.py:35 looks for 'fp16_gemm_cute') keep finding it.
-template <int BLOCK_M, int BLOCK_N>
+template <int BLOCK_M, int BLOCK_N, int STAGES>
 __global__ void __launch_bounds__(4 * kWaveSize)
 fp16_gemm_cute(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, _Float16* __restrict__ C, int m, int n, int k) {
-    dense_gemm_body<MfmaF16_32x32x16, _Float16, BLOCK_M, BLOCK_N>(A, B, C, m, n, k);
+    dense_gemm_body<MfmaF16_32x32x16, _Float16, BLOCK_M, BLOCK_N, STAGES>(A, B, C, m, n, k);
 }
 
 // Arguments every dense launcher checks before touching the GPU. Returns hipSuccess or hipErrorInvalidValue.
@@ -212,18 +245,18 @@ inline hipError_t check_dense_args(int m, int n, int k, const void* a, const voi
     return hipSuccess;
 }
 
-template <typename Atom, typename Elem, int BLOCK_M, int BLOCK_N>
+template <typename Atom, typename Elem, int BLOCK_M, int BLOCK_N, int STAGES = DenseTileConfig<BLOCK_M, BLOCK_N>::MAX_STAGES>
 inline hipError_t launch_dense(int m, int n, int k, const void* a, const void* b, void* c, hipStream_t stream) {
     if (m == 0 || n == 0) return hipSuccess;
     if (hipError_t e = check_dense_args(m, n, k, a, b, c, BLOCK_M, BLOCK_N); e != hipSuccess) return e;
     using Cfg = DenseTileConfig<BLOCK_M, BLOCK_N>;
     const XcdTileScheduler<> sched(m, n, BLOCK_M, BLOCK_N);
     if constexpr (__is_same(Elem, _Float16))
-        hipLaunchKernelGGL((fp16_gemm_cute<BLOCK_M, BLOCK_N>), dim3(sched.grid_size()),
+        hipLaunchKernelGGL((fp16_gemm_cute<BLOCK_M, BLOCK_N, STAGES>), dim3(sched.grid_size()),
                            dim3(Cfg::NUM_WAVES * kWaveSize), 0, stream, static_cast<const uint8_t*>(a),
                            static_cast<const uint8_t*>(b), static_cast<Elem*>(c), m, n, k);
     else
-        hipLaunchKernelGGL((dense_gemm_mfma<Atom, Elem, BLOCK_M, BLOCK_N>), dim3(sched.grid_size()),
+        hipLaunchKernelGGL((dense_gemm_mfma<Atom, Elem, BLOCK_M, BLOCK_N, STAGES>), dim3(sched.grid_size()),
                            dim3(Cfg::NUM_WAVES * kWaveSize), 0, stream, static_cast<const uint8_t*>(a),
                            static_cast<const uint8_t*>(b), static_cast<Elem*>(c), m, n, k);
     return hipGetLastError();
@@ -231,16 +264,16 @@ inline hipError_t launch_dense(int m, int n, int k, const void* a, const void* b
 
 } // namespace yan
 
-// bf16 in, fp32 accumulate, bf16 out. NUM_STAGES is accepted for interface parity; the kernel always runs two
-// LDS stages (two 256x256x64 stages are 128 KB of the 160 KB).
+// bf16 in, fp32 accumulate, bf16 out. NUM_STAGES is the number of LDS stages (2 .. DenseTileConfig::MAX_STAGES; two
+// 256x256x64 stages are 128 KB of the 160 KB, smaller tiles can hold a deeper ring).
 template <int BLOCK_M, int BLOCK_N, int NUM_STAGES>
 inline hipError_t gemm_tn(int m, int n, int k, const __hip_bfloat16* A, const __hip_bfloat16* B, __hip_bfloat16* C,
                           hipStream_t stream) {
-    return yan::launch_dense<yan::MfmaBF16_32x32x16, __bf16, BLOCK_M, BLOCK_N>(m, n, k, A, B, C, stream);
+    return yan::launch_dense<yan::MfmaBF16_32x32x16, __bf16, BLOCK_M, BLOCK_N, NUM_STAGES>(m, n, k, A, B, C, stream);
 }
 
 // fp16 in, fp32 accumulate, fp16 out.
 template <int BLOCK_M, int BLOCK_N, int NUM_STAGES>
 inline hipError_t gemm_tn(int m, int n, int k, const __half* A, const __half* B, __half* C, hipStream_t stream) {
-    return yan::launch_dense<yan::MfmaF16_32x32x16, _Float16, BLOCK_M, BLOCK_N>(m, n, k, A, B, C, stream);
+    return yan::launch_dense<yan::MfmaF16_32x32x16, _Float16, BLOCK_M, BLOCK_N, NUM_STAGES>(m, n, k, A, B, C, stream);
 }

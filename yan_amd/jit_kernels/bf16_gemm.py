@@ -8,7 +8,7 @@ keys `BLOCK_M, BLOCK_N, NUM_STAGES`, args `(m, n, k, A, B, C, stream)`.
 """
 import torch
 
-from .heuristics import get_best_dense_config
+from .heuristics import get_best_dense_config, get_dense_num_stages
 from .tuner import jit_tuner
 from .utils import get_num_sms
 
@@ -31,7 +31,7 @@ def dense_kernel_plan(m: int, n: int, k: int, dtype: torch.dtype, num_cus: int):
     """(name, keys, arg_defs) of the JIT kernel a call with these sizes uses; needs no GPU."""
     block_m, block_n = get_best_dense_config(m, n, k, num_cus)
     name = 'gemm_bf16_tn' if dtype == torch.bfloat16 else 'gemm_fp16_tn'
-    return name, {'BLOCK_M': block_m, 'BLOCK_N': block_n, 'NUM_STAGES': 2}, _arg_defs(dtype)
+    return name, {'BLOCK_M': block_m, 'BLOCK_N': block_n, 'NUM_STAGES': get_dense_num_stages(block_m, block_n)}, _arg_defs(dtype)
 
 
 def _gemm_16bit_tn(a: torch.Tensor, b: torch.Tensor, c: torch.Tensor, dtype: torch.dtype) -> None:

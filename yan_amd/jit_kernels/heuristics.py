@@ -34,6 +34,12 @@ def get_best_fp8_config(m: int, n: int, k: int, num_cus: int) -> Tuple[int, int]
     return rank_tiles(m, n, num_cus, _FP8_TILES)[0][1]
 
 
+def get_dense_num_stages(block_m: int, block_n: int) -> int:
+    """LDS stages of the dense kernel for a tile: as many as the 160 KB LDS holds, at most 8
+    (`DenseTileConfig::MAX_STAGES` in bf16_gemm.hpp): 2 for 256 x 256, 3 for 128 x 256, ... 8 for 64 x 64."""
+    return min(8, 160 * 1024 // ((block_m + block_n) * 128))
+
+
 def get_fp8_num_stages(block_m: int, block_n: int) -> int:
     """LDS stages of the tiled FP8 kernel for a tile: a ring as deep as the 160 KB LDS allows (at most 8) for the small
     4-wave tiles that support one (`Fp8TileConfig::MAX_RING_STAGES` in fp8_gemm.hpp), else 2. Small tiles are what the
