@@ -169,8 +169,8 @@ def main():
         decode = lambda: yan.gemm_fp8_fp8_bf16_nt((x8, sx), (w8, sw), o)
         _, wall = _event_time_ms(decode, 200, 20)
         # this kernel is shorter than the host side of a call, so its own device time comes from the profiler
-        ms = yan.bench_kineto(decode, 'fp8_gemm_splitk_kernel', suppress_kineto_output=True) * 1e3
-        ms_cold = yan.bench_kineto(decode, 'fp8_gemm_splitk_kernel', suppress_kineto_output=True, flush_l2=True) * 1e3
+        ms = yan.bench_kineto(decode, 'fp8_gemm_kernel', suppress_kineto_output=True) * 1e3
+        ms_cold = yan.bench_kineto(decode, 'fp8_gemm_kernel', suppress_kineto_output=True, flush_l2=True) * 1e3
         byt = mm * kk + nn * kk + 4 * mm * (kk // 128) + 4 * (nn // 128) * (kk // 128) + 2 * mm * nn
         extra['fp8_decode_64x4096x7168'] = {'kernel_us_warm': round(ms * 1e3, 2), 'kernel_us_cold': round(ms_cold * 1e3, 2),
                                             'call_to_call_us': round(wall * 1e3, 2),

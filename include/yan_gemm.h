@@ -49,11 +49,8 @@ YAN_API int yan_gemm_fp16_tn(int m, int n, int k, const void* a, const void* b, 
  *   out        bf16 [m,n] row-major
  * Requires k % 128 == 0, n % 4 == 0; m arbitrary. `num_sms` is the caller's compute-unit cap (the reference passes
  * it to its persistent kernel, yan/jit_kernels/gemm.py:26-30); this build launches one workgroup per tile and
- * accepts the argument for signature compatibility (the split-K decode kernel uses it to size its grid).
- * For 33..64 activation rows and n >= 8 * CUs the split-K kernel runs: it keeps a library-owned scratch buffer
- * (allocated with hipMalloc on first use, at most ceil(n/64) * splits * 16 KB) and a self-resetting counter per 64
- * output columns, shared by all calls on a device: such calls must not overlap in time on one device, and the
- * first of them cannot be captured into a HIP graph.
+ * accepts the argument for signature compatibility (tile choice uses it as the number of compute units when > 0).
+ * Nothing is allocated and no state is kept between calls.
  * Replaces the FP8 entry the reference only sketches: template yan/jit_kernels/gemm.py:9-31, kernel
  * yan/include/gemm/fp8_gemm.cuh:40-196. */
 YAN_API int yan_gemm_fp8_fp8_bf16_nt(const void* lhs, const float* lhs_scales, long long lhs_scales_stride_m,
@@ -102,7 +99,7 @@ YAN_API int yan_per_block_cast_to_fp8(const void* w, int w_is_fp32, void* q, flo
  * (yan/jit_kernels/cute_gemm.py:41, yan/jit_kernels/gemm.py:13-16). Returns 0, or 1 for an unknown op. */
 YAN_API int yan_gemm_select_tile(int op, int m, int n, int k, int num_cus, int* block_m, int* block_n);
 
-/* "yan-gemm gfx950 <n> dense + <n> fp8 tile variants + <n> weight-streaming + <n> split-K fp8 variants". */
+/* "yan-gemm gfx950 <n> dense + <n> fp8 tile variants + <n> weight-streaming fp8 variant + ...". */
 YAN_API const char* yan_gemm_version(void);
 
 /* The JIT boundary, for reference: signatures of `launch` in the kernel.so of each op

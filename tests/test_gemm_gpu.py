@@ -301,22 +301,26 @@ def test_fp8_decode_shape():
     assert oracle.calc_diff(_np(out), _fp8_ref(a8, sa, b8, sb)) < 1e-5
 
 
-def test_fp8_split_k_decode_kernel_is_repeatable():
-    """33..64 activation rows run the split-K kernel: partial tiles meet in a library-owned scratch buffer and a
-    self-resetting counter picks the workgroup that finishes each column tile. Repeated and interleaved calls must
-    keep giving the same bits (the partials are added in split order, not arrival order)."""
+def test_fp8_decode_shapes_are_repeatable():
+    """The decode shapes (tiled kernel on narrow tiles with a ring of LDS stages; weight-streaming kernel up to 16
+    rows) keep no state between calls: repeated and interleaved calls give the same bits."""
     (a8, sa), (b8, sb), out = testing.make_fp8_case(64, 4096, 7168, seed=3, device='cuda')
     (c8, sc), (d8, sd), out_small = testing.make_fp8_case(40, 2112, 640, seed=4, device='cuda')
+    (e8, se), (f8, sf), out_one = testing.make_fp8_case(1, 4096, 7168, seed=5, device='cuda')
     yan.gemm_fp8_fp8_bf16_nt((a8, sa), (b8, sb), out)
-    first = out.clone()
+    yan.gemm_fp8_fp8_bf16_nt((e8, se), (f8, sf), out_one)
+    first, first_one = out.clone(), out_one.clone()
     ref_small = _fp8_ref(c8, sc, d8, sd)
     for _ in range(5):
         out.fill_(float('nan'))
+        out_one.fill_(float('nan'))
         yan.gemm_fp8_fp8_bf16_nt((a8, sa), (b8, sb), out)
-        yan.gemm_fp8_fp8_bf16_nt((c8, sc), (d8, sd), out_small)      # a different shape through the same scratch
-        assert torch.equal(out, first)
+        yan.gemm_fp8_fp8_bf16_nt((c8, sc), (d8, sd), out_small)
+        yan.gemm_fp8_fp8_bf16_nt((e8, se), (f8, sf), out_one)
+        assert torch.equal(out, first) and torch.equal(out_one, first_one)
         assert oracle.calc_diff(_np(out_small), ref_small) < 1e-5
     assert oracle.calc_diff(_np(first), _fp8_ref(a8, sa, b8, sb)) < 1e-5
+    assert oracle.calc_diff(_np(first_one), _fp8_ref(e8, se, f8, sf)) < 1e-5
 
 
 def test_fp8_outlier_16384_cubed():

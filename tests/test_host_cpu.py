@@ -31,9 +31,13 @@ def test_tile_heuristics_fill_256_cus():
     # a skinny problem must not pick a tile that leaves most CUs idle
     bm, bn = heuristics.get_best_fp8_config(64, 4096, 7168, 256)
     assert bm == 64 and yan.ceil_div(4096, bn) >= 64
-    # ... and the decode shape goes to the weight-streaming kernel: one workgroup per 16 weight rows
-    assert heuristics.get_fp8_tile(64, 4096, 7168, 256) == (64, 16) and heuristics.get_fp8_tile(1, 4096, 7168, 256) == (16, 16)
-    assert heuristics.get_skinny_fp8_config(65, 4096, 7168, 256) == 0 and heuristics.get_skinny_fp8_config(64, 1024, 7168, 256) == 0
+    # ... the decode shape runs the tiled kernel on 64 x 16 tiles with a deep ring of LDS stages, and up to 16 rows go
+    # to the weight-streaming kernel (one workgroup per 16 weight rows) while those workgroups fit the chip at once
+    assert heuristics.get_fp8_tile(64, 4096, 7168, 256) == (64, 16) and heuristics.get_fp8_num_stages(64, 16) == 8
+    assert heuristics.get_fp8_tile(1, 4096, 7168, 256) == (16, 16) and heuristics.get_fp8_tile(16, 2048, 7168, 256) == (16, 16)
+    assert heuristics.get_skinny_fp8_config(17, 4096, 7168, 256) == 0 and heuristics.get_skinny_fp8_config(16, 7168, 7168, 256) == 0
+    assert heuristics.get_fp8_num_stages(256, 256) == 2 and heuristics.get_dense_num_stages(256, 256) == 2
+    assert heuristics.get_dense_num_stages(64, 64) == 8 and heuristics.get_dense_num_stages(128, 256) == 3
     # tiny problems get the smallest tile
     assert heuristics.get_best_dense_config(64, 64, 64, 256) == (64, 64)
     ranked = heuristics.rank_tiles(4096, 7168, 256, heuristics._FP8_TILES)

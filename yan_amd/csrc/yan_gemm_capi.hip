@@ -47,8 +47,7 @@ void pick_grouped(int m, int n, int num_cus, int groups, int m_alignment, int gr
 
 // Activation atoms of the weight-streaming kernel, or 0 for the tiled kernel (get_skinny_fp8_config in heuristics.py).
 int skinny_atoms(int m, int n, int num_cus) {
-    if (m > 0 && m <= 64 && n >= 8 * num_cus) return m <= 16 ? 1 : (m <= 32 ? 2 : 4);
-    return 0;
+    return (m > 0 && m <= 16 && n >= 16 && n <= 16 * num_cus) ? 1 : 0;
 }
 
 int device_cus() {
@@ -97,12 +96,9 @@ int yan_gemm_fp8_fp8_bf16_nt(const void* lhs, const float* lhs_scales, long long
     const int cus = num_sms > 0 ? num_sms : device_cus();
     hipStream_t s = static_cast<hipStream_t>(stream);
     __hip_bfloat16* o = static_cast<__hip_bfloat16*>(out);
-    if (const int atoms = skinny_atoms(m, n, cus)) {
-        const int sm = int(lhs_scales_stride_m), sk = int(lhs_scales_stride_k);
-        if (atoms == 1) return int(yan::launch_fp8_skinny<0, 0, 1, 8>(o, lhs, lhs_scales, sm, sk, rhs, rhs_scales, m, n, k, s));
-        if (atoms == 2) return int(yan::launch_fp8_skinny<0, 0, 2, 8>(o, lhs, lhs_scales, sm, sk, rhs, rhs_scales, m, n, k, s));
-        return int(yan::launch_fp8_splitk<0, 0, 4, 16>(o, lhs, lhs_scales, sm, sk, rhs, rhs_scales, m, n, k, s, cus));
-    }
+    if (skinny_atoms(m, n, cus))
+        return int(yan::launch_fp8_skinny<0, 0, 1, 8>(o, lhs, lhs_scales, int(lhs_scales_stride_m), int(lhs_scales_stride_k), rhs,
+                                                      rhs_scales, m, n, k, s));
     int bm = 0, bn = 0;
     pick(kFp8Tiles, m, n, cus, &bm, &bn);
 #define YAN_FP8_CASE(BM, BN)                                                                                         \
@@ -186,6 +182,6 @@ int yan_gemm_select_tile(int op, int m, int n, int k, int num_cus, int* block_m,
     return 0;
 }
 
-const char* yan_gemm_version(void) { return "yan-gemm gfx950 6 dense + 8 fp8 tile variants + 2 weight-streaming + 1 split-K fp8 variants + 12 grouped fp8 variants + 4 quantiser kernels"; }
+const char* yan_gemm_version(void) { return "yan-gemm gfx950 6 dense + 8 fp8 tile variants + 1 weight-streaming fp8 variant + 12 grouped fp8 variants + 4 quantiser kernels"; }
 
 } // extern "C"

@@ -50,7 +50,7 @@ struct Fp8TileConfig {
     static constexpr int  RING_SCALE_BYTES = ceil_div(NUM_WAVES * BLOCK_M * 4, 1024) * 1024;
     static constexpr int  RING_STAGE_BYTES = (BLOCK_M + BLOCK_N) * kRowBytes + RING_SCALE_BYTES;
     static constexpr bool RING_CAPABLE = NUM_WAVES == 4 && BLOCK_M % 64 == 0 && BLOCK_M <= 128 &&
-                                         (BLOCK_M / 8) % NUM_WAVES == 0 && (BLOCK_N / 8) % NUM_WAVES == 0;
+                                         (BLOCK_M / 8) % NUM_WAVES == 0 && BLOCK_N % 16 == 0;
     static constexpr int  MAX_RING_STAGES = RING_CAPABLE ? (160 * 1024 / RING_STAGE_BYTES < 8 ? 160 * 1024 / RING_STAGE_BYTES : 8) : 2;
 };
 
@@ -263,14 +263,16 @@ fp8_gemm_kernel(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_s
     if (NUM_K_BLOCKS % 2 == 1) k_step(NUM_K_BLOCKS - 1, lds_a0, lds_b0, lds_a1, lds_b1);
     } else {
     // Ring of STAGES stages, STAGES - 1 k-tiles in flight: what a small tile needs when the problem is bound by
-    // streaming its operands and one k-tile of prefetch cannot cover the memory latency. Every wave issues the same
-    // number of copies per k-tile (OPS), in the same order, so "k-tile kb has landed" is "at most (STAGES - 2) * OPS
-    // of my copies are outstanding". The activation scales of a k-tile travel through the stage as well (a register
+    // streaming its operands and one k-tile of prefetch cannot cover the memory latency. A wave issues the same
+    // number of copies for every k-tile (OPS, one fewer for the waves that have no part in the last pass over a narrow
+    // weight tile), in the same order, so "k-tile kb has landed" is "at most (STAGES - 2) * OPS of my copies are
+    // outstanding". The activation scales of a k-tile travel through the stage as well (a register
     // load between the copies would make the in-order counter wait for every older copy); each wave keeps a private
     // copy of the tile's BLOCK_M scales, written by one full-width instruction per 64 rows.
     constexpr int STAGE_BYTES = Cfg::RING_STAGE_BYTES, TILE_BYTES = (BLOCK_M + BLOCK_N) * kRowBytes;
     constexpr int SCALE_OPS = BLOCK_M / 64, OPS = StA::PASSES + StB::PASSES + SCALE_OPS;
     static_assert(Cfg::RING_CAPABLE && (STAGES - 2) * OPS <= 63 && STAGES * STAGE_BYTES <= 160 * 1024);
+    constexpr int FULL_B_WAVES = StB::GROUPS % NW == 0 ? NW : StB::GROUPS % NW;      // waves that take part in the last B pass
     __shared__ __attribute__((aligned(1024))) uint8_t ring[STAGES * STAGE_BYTES];
     const uint32_t scale_voff = uint32_t(m0 + lane) * sa_stride_m * 4;
     auto issue_op = [&](int d, int kb, uint8_t* stage) {
@@ -291,7 +293,8 @@ fp8_gemm_kernel(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_s
     for (int kb = 0; kb < NUM_K_BLOCKS; ++kb) {
 #pragma unroll
         for (int b = 0; b < NB; ++b) sb_cur[b] = sb_next[b];
-        __builtin_amdgcn_s_waitcnt(waitcnt_imm((STAGES - 2) * OPS, kNoWaitLgkm));
+        if (FULL_B_WAVES == NW || wave < FULL_B_WAVES) __builtin_amdgcn_s_waitcnt(waitcnt_imm((STAGES - 2) * OPS, kNoWaitLgkm));
+        else __builtin_amdgcn_s_waitcnt(waitcnt_imm((STAGES - 2) * (OPS - 1), kNoWaitLgkm));
         asm volatile("" ::: "memory");
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");

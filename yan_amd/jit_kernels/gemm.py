@@ -37,8 +37,8 @@ __return_code = static_cast<int>(GemmType::run(out, lhs, lhs_scales, lhs_scales_
                                                rhs, rhs_scales, m, stream, num_sms, smem_size));
 """
 
-# Few activation rows (decode): BLOCK_M / 16 activation atoms per workgroup, 16 weight rows per workgroup, the K blocks
-# of a workgroup shared out over NUM_WAVES waves; no LDS staging, so NUM_STAGES is the per-wave load depth's name only.
+# A handful of activation rows: BLOCK_M / 16 activation atoms and 16 weight rows per workgroup, the K blocks of a
+# workgroup shared out over NUM_WAVES waves; no LDS staging, NUM_STAGES is the per-wave load depth's name only.
 skinny_template = """
 using namespace yan;
 
@@ -50,13 +50,9 @@ constexpr auto kNumStages = {NUM_STAGES};
 constexpr auto kNumTMAMulticast = {NUM_TMA_MULTICAST};
 static_assert(BLOCK_N == 16 && BLOCK_M % 16 == 0);
 
-// Launch kernel: weight-streaming kernel up to 32 activation rows, split-K kernel (library-owned scratch) above
-if constexpr (BLOCK_M <= 32)
-    __return_code = static_cast<int>(launch_fp8_skinny<N, K, BLOCK_M / 16, {NUM_WAVES}>(
-        out, lhs, lhs_scales, lhs_scales_stride_m, lhs_scales_stride_k, rhs, rhs_scales, m, N, K, stream));
-else
-    __return_code = static_cast<int>(launch_fp8_splitk<N, K, BLOCK_M / 16, 16>(
-        out, lhs, lhs_scales, lhs_scales_stride_m, lhs_scales_stride_k, rhs, rhs_scales, m, N, K, stream, num_sms));
+// Launch kernel
+__return_code = static_cast<int>(launch_fp8_skinny<N, K, BLOCK_M / 16, {NUM_WAVES}>(
+    out, lhs, lhs_scales, lhs_scales_stride_m, lhs_scales_stride_k, rhs, rhs_scales, m, N, K, stream));
 """
 
 arg_defs = (('lhs', torch.float8_e4m3fn), ('lhs_scales', torch.float),

@@ -46,7 +46,7 @@ def get_fp8_num_stages(block_m: int, block_n: int) -> int:
     cost model picks when the problem is short on work per CU, i.e. bound by operand streaming, and there one k-tile
     of prefetch does not cover the memory latency."""
     waves = 8 if block_m * block_n >= 256 * 128 else 4
-    capable = waves == 4 and block_m % 64 == 0 and block_m <= 128 and (block_m // 8) % waves == 0 and (block_n // 8) % waves == 0
+    capable = waves == 4 and block_m % 64 == 0 and block_m <= 128 and (block_m // 8) % waves == 0 and block_n % 16 == 0
     if not capable:
         return 2
     stage_bytes = (block_m + block_n) * 128 + ceil_div(waves * block_m * 4, 1024) * 1024
@@ -69,13 +69,14 @@ def get_best_grouped_fp8_config(m: int, n: int, k: int, num_cus: int, groups: in
 
 
 def get_skinny_fp8_config(m: int, n: int, k: int, num_cus: int) -> int:
-    """Number of 16-row activation atoms (1, 2 or 4) when one of the two decode kernels should run instead of the tiled
-    one, else 0: up to 64 activation rows, and enough weight rows that N/16 workgroups fill at least half the CUs.
-    Up to 32 rows (1 or 2 atoms) the weight-streaming kernel runs; 33..64 rows (4 atoms) go to the split-K kernel,
-    whose activations are read N/64 instead of N/16 times (measured: 15 vs 19 us warm, 25 vs 25 us cold at m = 64;
-    6.5-12 vs 8.5-12.7 us warm at m <= 32)."""
-    if 0 < m <= 64 and n >= 8 * num_cus:
-        return 1 if m <= 16 else (2 if m <= 32 else 4)
+    """Number of 16-row activation atoms (1) when the weight-streaming kernel should run instead of the tiled one, else 0:
+    up to 16 activation rows, and few enough weight rows that its n/16 workgroups fit the chip in one round. Measured
+    on 256 CUs (kernel time warm / after a cache flush, weight-streaming vs tiled with its ring of LDS stages):
+    m = 1..16, n = 4096, k = 7168: 7.4-9.3 / 13.4 us vs 13.7-14.0 / 15.3 us; n = 2048: 6.9-9.1 / 9.4-10.4 vs 13.6 / 14.4;
+    n = 7168: 12.9-15.5 / 22 vs 15.5 / 21 (a tie, and two rounds of workgroups). From 17 rows up the tiled kernel wins or
+    ties everywhere (m = 64, n = 4096, k = 7168: 14.5 / 17.2 us)."""
+    if 0 < m <= 16 and 16 <= n <= 16 * num_cus:
+        return 1
     return 0
 
 
