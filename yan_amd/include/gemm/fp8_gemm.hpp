@@ -45,12 +45,11 @@ struct Fp8TileConfig {
     static constexpr int  SCALE_B_PER_SLAB = UNIFORM_SCALE_B ? 1 : (WTN + 112) / 128 + 1;
     static constexpr int  LDS_BYTES = 2 * (BLOCK_M + BLOCK_N) * kRowBytes;
     static_assert(LDS_BYTES <= 160 * 1024, "two stages must fit the 160 KB LDS");
-    // Ring of more than two stages (small tiles, where one k-tile in flight cannot cover the memory latency): a stage
-    // also carries the k-tile's activation scales, one private copy per wave.
-    static constexpr int  RING_SCALE_BYTES = ceil_div(NUM_WAVES * BLOCK_M * 4, 1024) * 1024;
+    // Ring of more than two stages (tiles below 256 x 256, where one k-tile in flight does not cover the memory
+    // latency of an operand-streaming problem): a stage also carries the k-tile's BLOCK_M activation scales.
+    static constexpr int  RING_SCALE_BYTES = ceil_div(BLOCK_M * 4, 1024) * 1024;
     static constexpr int  RING_STAGE_BYTES = (BLOCK_M + BLOCK_N) * kRowBytes + RING_SCALE_BYTES;
-    static constexpr bool RING_CAPABLE = NUM_WAVES == 4 && BLOCK_M % 64 == 0 && BLOCK_M <= 128 &&
-                                         (BLOCK_M / 8) % NUM_WAVES == 0 && BLOCK_N % 16 == 0;
+    static constexpr bool RING_CAPABLE = BLOCK_M % 64 == 0 && (BLOCK_M / 8) % NUM_WAVES == 0 && BLOCK_N % 16 == 0;
     static constexpr int  MAX_RING_STAGES = RING_CAPABLE ? (160 * 1024 / RING_STAGE_BYTES < 8 ? 160 * 1024 / RING_STAGE_BYTES : 8) : 2;
 };
 
@@ -266,11 +265,11 @@ fp8_gemm_kernel(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_s
     // streaming its operands and one k-tile of prefetch cannot cover the memory latency. A wave issues the same
     // number of copies for every k-tile (OPS, one fewer for the waves that have no part in the last pass over a narrow
     // weight tile), in the same order, so "k-tile kb has landed" is "at most (STAGES - 2) * OPS of my copies are
-    // outstanding". The activation scales of a k-tile travel through the stage as well (a register
-    // load between the copies would make the in-order counter wait for every older copy); each wave keeps a private
-    // copy of the tile's BLOCK_M scales, written by one full-width instruction per 64 rows.
+    // outstanding". The activation scales of a k-tile travel through the stage as well (a register load between the
+    // copies would make the in-order counter wait for every older copy): every wave copies one 64-row part of them
+    // with one full-width instruction; waves that share a part write the same bytes twice.
     constexpr int STAGE_BYTES = Cfg::RING_STAGE_BYTES, TILE_BYTES = (BLOCK_M + BLOCK_N) * kRowBytes;
-    constexpr int SCALE_OPS = BLOCK_M / 64, OPS = StA::PASSES + StB::PASSES + SCALE_OPS;
+    constexpr int OPS = StA::PASSES + StB::PASSES + 1, SCALE_PARTS = BLOCK_M / 64;
     static_assert(Cfg::RING_CAPABLE && (STAGES - 2) * OPS <= 63 && STAGES * STAGE_BYTES <= 160 * 1024);
     constexpr int FULL_B_WAVES = StB::GROUPS % NW == 0 ? NW : StB::GROUPS % NW;      // waves that take part in the last B pass
     __shared__ __attribute__((aligned(1024))) uint8_t ring[STAGES * STAGE_BYTES];
@@ -279,8 +278,8 @@ fp8_gemm_kernel(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_s
         if (d < StA::PASSES) stage_a.issue_pass(rsrc_a, stage, kb * kRowBytes, wave, d);
         else if (d < StA::PASSES + StB::PASSES) stage_b.issue_pass(rsrc_b, stage + BLOCK_M * kRowBytes, kb * kRowBytes, wave, d - StA::PASSES);
         else {
-            const int part = d - StA::PASSES - StB::PASSES;       // rows m0 + 64 * part + lane
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_sa, YAN_LDS_PTR(stage + TILE_BYTES + (wave * BLOCK_M + part * 64) * 4), 4,
+            const int part = wave % SCALE_PARTS;                    // rows m0 + 64 * part + lane
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_sa, YAN_LDS_PTR(stage + TILE_BYTES + part * 256), 4,
                                                      scale_voff, (kb * sa_stride_k + part * 64 * sa_stride_m) * 4, 0, 0);
         }
     };
@@ -302,7 +301,7 @@ fp8_gemm_kernel(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_s
         const uint8_t* cur = ring + st * STAGE_BYTES;
         const int st_nxt = st + STAGES - 1 >= STAGES ? st - 1 : st + STAGES - 1;
         uint8_t* nxt = ring + st_nxt * STAGE_BYTES;
-        const float* my_scales = reinterpret_cast<const float*>(cur + TILE_BYTES) + wave * BLOCK_M + wm * Cfg::WTM + col;
+        const float* my_scales = reinterpret_cast<const float*>(cur + TILE_BYTES) + wm * Cfg::WTM + col;
 #pragma unroll
         for (int j = 0; j < TM; ++j) sa_cur[j] = my_scales[j * 16];
         compute_tile(cur, cur + BLOCK_M * kRowBytes, sa_cur, sb_cur, [&](int row) {

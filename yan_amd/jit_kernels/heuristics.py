@@ -41,16 +41,16 @@ def get_dense_num_stages(block_m: int, block_n: int) -> int:
 
 
 def get_fp8_num_stages(block_m: int, block_n: int) -> int:
-    """LDS stages of the tiled FP8 kernel for a tile: a ring as deep as the 160 KB LDS allows (at most 8) for the small
-    4-wave tiles that support one (`Fp8TileConfig::MAX_RING_STAGES` in fp8_gemm.hpp), else 2. Small tiles are what the
-    cost model picks when the problem is short on work per CU, i.e. bound by operand streaming, and there one k-tile
-    of prefetch does not cover the memory latency."""
+    """LDS stages of the tiled FP8 kernel for a tile: a ring as deep as the 160 KB LDS allows, at most 8
+    (`Fp8TileConfig::MAX_RING_STAGES` in fp8_gemm.hpp): 2 for 256 x 256, 3 for 256 x 128 and 128 x 256, up to 8 for the
+    smallest. Tiles below 256 x 256 are what the cost model picks when a problem is short on work per CU, i.e. bound by
+    operand streaming, and there one k-tile of prefetch does not cover the memory latency."""
     waves = 8 if block_m * block_n >= 256 * 128 else 4
-    capable = waves == 4 and block_m % 64 == 0 and block_m <= 128 and (block_m // 8) % waves == 0 and block_n % 16 == 0
+    capable = block_m % 64 == 0 and (block_m // 8) % waves == 0 and block_n % 16 == 0
     if not capable:
         return 2
-    stage_bytes = (block_m + block_n) * 128 + ceil_div(waves * block_m * 4, 1024) * 1024
-    return min(8, 160 * 1024 // stage_bytes)
+    stage_bytes = (block_m + block_n) * 128 + ceil_div(block_m * 4, 1024) * 1024
+    return max(2, min(8, 160 * 1024 // stage_bytes))
 
 
 def get_best_grouped_fp8_config(m: int, n: int, k: int, num_cus: int, groups: int = 1, m_alignment: int = 0,
