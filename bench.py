@@ -95,6 +95,8 @@ def main():
     ap.add_argument('--warmup', type=int, default=100)
     ap.add_argument('--also', action='store_true', help='also time bf16 8192^3, the decode shape and 16384^3 (extra fields)')
     ap.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline leg')
+    ap.add_argument('--ceilings', action='store_true',
+                    help='also measure what the matrix cores sustain with register-resident operands (random and zero bits)')
     ap.add_argument('--calibrate-copy', action='store_true',
                     help='also run a 1 GiB device-to-device copy three times, as the known-size kernel that hardware '
                          'byte counters (FETCH_SIZE / WRITE_SIZE) are scaled by when profiling')
@@ -212,6 +214,13 @@ def main():
                            'frac_of_hbm_peak_cold': round(byt / t_cold / 1e9 / PEAK_HBM_GBPS, 4)}
         del xs, ws
         line['extra'] = extra
+
+    if args.ceilings:
+        from yan_amd import probe
+        line['mfma_only_ceiling_tflops'] = {kind: {data: round(probe.mfma_ceiling(kind, data), 1) for data in ('random', 'zero')}
+                                            for kind in probe.MODES}
+        fold = line['mfma_only_ceiling_tflops']['fp8_16x16x128_zero_c_plus_fold']['random']
+        line['roofline']['frac_of_mfma_only_ceiling'] = round(tflops_kernel / fold, 4)
 
     if not args.no_cpu:
         line['cpu_baseline'] = _cpu_baseline_fp8(a8, sa, b8, sb)

@@ -342,6 +342,15 @@ def test_fp8_outlier_16384_cubed():
 
 
 # ----------------------------------------------------------------------------- the ahead-of-time C-ABI library
+def test_mfma_ceiling_probe_runs_and_stays_below_the_vendor_peak():
+    from yan_amd import probe
+    for kind, peak in (('bf16_32x32x16', 2520.0), ('bf16_16x16x32', 2520.0), ('fp8_16x16x128_accumulate', 5040.0),
+                       ('fp8_16x16x128_zero_c_plus_fold', 5040.0)):
+        zero = probe.mfma_ceiling(kind, 'zero', iters=1000, launches=5)
+        rand = probe.mfma_ceiling(kind, 'random', iters=1000, launches=5)
+        assert 0.3 * peak < rand <= zero * 1.05 and zero < peak * 1.02, (kind, rand, zero)
+
+
 def test_tuner_times_a_space_of_tiles_on_the_device():
     """The empirical half of compile_and_tune (yan/jit_kernels/tuner.py:24-69): every candidate of `space` is built, run
     once, timed over back-to-back launches after a cache flush, and the fastest is kept and memoised."""

@@ -188,7 +188,11 @@ def prebuild_jit_kernels(num_cus: int = 256, verbose: bool = False) -> int:
             rt = build(name, arg_defs, code)
             if verbose:
                 print(f'built {name} {keys} -> {rt.path}')
+    from . import probe
     from .jit_kernels import fp8_cast, m_grouped_gemm
+    name, arg_defs, code = probe.probe_kernel()
+    seen.add((name, code))
+    build(name, arg_defs, code)
     for kind in ('per_token', 'per_block'):
         for dtype in (torch.bfloat16, torch.float32):
             name, keys, arg_defs, code_template = fp8_cast.cast_kernel_plan(kind, dtype)
