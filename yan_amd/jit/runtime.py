@@ -11,7 +11,7 @@ from typing import Dict, Optional
 
 import torch
 
-from .template import map_ctype
+from .template import ctype_map
 
 KERNEL_FILES = ('kernel.cu', 'kernel.args', 'kernel.so')
 
@@ -37,6 +37,8 @@ class Runtime:
             self.args = eval(f.read(), {'torch': torch, '__builtins__': {'bool': bool, 'int': int, 'float': float}})
         if self.args and not isinstance(self.args[0], tuple):
             self.args = (self.args,)      # a single ('name', type) pair evaluates to a flat tuple
+        # Declared once so that ctypes marshals plain Python ints (device pointers, stream handles) and scalars itself.
+        self._launch.argtypes = [ctype_map[dtype] for _, dtype in self.args] + [ctypes.POINTER(ctypes.c_int)]
 
     def __call__(self, *args) -> int:
         if self._launch is None:
@@ -46,11 +48,12 @@ class Runtime:
         for arg, (name, dtype) in zip(args, self.args):
             if isinstance(arg, torch.Tensor):
                 assert arg.dtype == dtype, f'Expected tensor dtype `{dtype}` for `{name}`, got `{arg.dtype}`'
+                cargs.append(arg.data_ptr())
             else:
                 assert isinstance(arg, dtype), f'Expected built-in type `{dtype}` for `{name}`, got `{type(arg)}`'
-            cargs.append(map_ctype(arg))
+                cargs.append(arg.cuda_stream if dtype is torch.cuda.Stream else arg)     # on ROCm the hipStream_t handle
         rc = ctypes.c_int(0)
-        self._launch(*cargs, ctypes.byref(rc))
+        self._launch(*cargs, rc)
         return rc.value
 
 

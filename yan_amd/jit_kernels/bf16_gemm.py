@@ -6,6 +6,8 @@ Same contract as the reference's `gemm_fp16_tn` (`yan/jit_kernels/cute_gemm.py:2
 bf16 and fp16 exist and both accumulate in fp32. Keys and argument order of the JIT kernel are the reference's:
 keys `BLOCK_M, BLOCK_N, NUM_STAGES`, args `(m, n, k, A, B, C, stream)`.
 """
+import functools
+
 import torch
 
 from .heuristics import get_best_dense_config, get_dense_num_stages
@@ -27,6 +29,7 @@ def _arg_defs(dtype: torch.dtype):
     return (('m', int), ('n', int), ('k', int), ('A', dtype), ('B', dtype), ('C', dtype), ('stream', torch.cuda.Stream))
 
 
+@functools.lru_cache(maxsize=None)
 def dense_kernel_plan(m: int, n: int, k: int, dtype: torch.dtype, num_cus: int):
     """(name, keys, arg_defs) of the JIT kernel a call with these sizes uses; needs no GPU."""
     block_m, block_n = get_best_dense_config(m, n, k, num_cus)

@@ -8,6 +8,7 @@ rounded fp32 divisions; torch evaluates `448.0 / amax` as `reciprocal(amax) * 44
 amax and moves a code where `x * factor` lands on a rounding boundary. With true tensor / tensor divisions the torch
 chain and these kernels agree bit for bit.
 """
+import functools
 from typing import Tuple
 
 import torch
@@ -45,6 +46,7 @@ def per_block_arg_defs(dtype: torch.dtype):
             ('stream', torch.cuda.Stream))
 
 
+@functools.lru_cache(maxsize=None)
 def cast_kernel_plan(kind: str, dtype: torch.dtype):
     """(name, keys, arg_defs, template) of the JIT kernel behind a quantiser; needs no GPU."""
     keys = {'SRC': _src_name(dtype)}

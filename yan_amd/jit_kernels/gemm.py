@@ -9,6 +9,7 @@ are passed explicitly, which lets the kernel read them row-major or token-contig
     out[i, j] = bf16( sum_kb lhs_scales[i, kb] * rhs_scales[j // 128, kb]
                               * sum_{t < 128} f32(lhs[i, 128 kb + t]) * f32(rhs[j, 128 kb + t]) )
 """
+import functools
 from typing import Tuple
 
 import torch
@@ -62,6 +63,7 @@ arg_defs = (('lhs', torch.float8_e4m3fn), ('lhs_scales', torch.float),
             ('lhs_scales_stride_m', int), ('lhs_scales_stride_k', int))
 
 
+@functools.lru_cache(maxsize=None)
 def fp8_kernel_plan(m: int, n: int, k: int, num_cus: int):
     """(name, keys, arg_defs, smem_size, template) of the JIT kernel a call with these sizes uses; needs no GPU."""
     skinny_atoms = get_skinny_fp8_config(m, n, k, num_cus)

@@ -7,6 +7,7 @@ The reference carries the hooks for these and no entry point: `GemmType::{Groupe
 The two entries below complete them with the calling convention of the DeepGEMM functions those hooks come from.
 Scales, dtypes and the arithmetic are those of `gemm_fp8_fp8_bf16_nt`, applied per group.
 """
+import functools
 from typing import Tuple
 
 import torch
@@ -43,6 +44,7 @@ arg_defs = (('lhs', torch.float8_e4m3fn), ('lhs_scales', torch.float),
             ('lhs_scales_stride_m', int), ('lhs_scales_stride_k', int), ('lhs_scales_stride_g', int))
 
 
+@functools.lru_cache(maxsize=None)
 def grouped_kernel_plan(gemm_type: str, num_groups: int, m: int, n: int, k: int, num_cus: int):
     """(name, keys, arg_defs, smem_size) of the JIT kernel of a grouped call; needs no GPU. `m` is the total row count
     for 'GroupedContiguous' and the expected rows per group for 'GroupedMasked'."""

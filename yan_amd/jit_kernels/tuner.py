@@ -38,9 +38,17 @@ class JITTuner:
     def __init__(self) -> None:
         self.tuned: Dict[Tuple[str, str], Runtime] = {}
         self.tuned_keys: Dict[Tuple[str, str], Dict[str, Any]] = {}
+        # Callers that pass the very same `keys` object again (the entry points memoise their plans) skip building the
+        # textual signature: (name, id(keys)) -> (keys, runtime); the stored reference both keeps the id from being
+        # reused and is compared on lookup.
+        self._same_object: Dict[Tuple[str, int], Tuple[Dict[str, Any], Runtime]] = {}
 
     def compile_and_tune(self, name: str, keys: Dict[str, Any], space: tuple,
                          includes: tuple, arg_defs: tuple, template: str, args: tuple) -> Runtime:
+        seen = self._same_object.get((name, id(keys)))
+        if seen is not None and seen[0] is keys:
+            return seen[1]
+        caller_keys = keys
         keys = {k: keys[k] for k in sorted(keys)}
         signature = (name, str(keys))
         debug = bool(os.getenv('YAN_JIT_DEBUG'))
@@ -48,6 +56,7 @@ class JITTuner:
         if hit is not None:
             if debug:
                 print(f'Using cached JIT kernel {name} with keys {keys}')
+            self._same_object[(name, id(caller_keys))] = (caller_keys, hit)
             return hit
         if debug:
             print(f'Auto-tuning JIT kernel {name} with keys {keys}')
@@ -80,6 +89,7 @@ class JITTuner:
             print(f'Best JIT kernel {name} with keys {keys} has tuned keys {best[2]} and time {best[0]}')
         self.tuned[signature] = best[1]
         self.tuned_keys[signature] = dict(best[2])
+        self._same_object[(name, id(caller_keys))] = (caller_keys, best[1])
         return best[1]
 
 
