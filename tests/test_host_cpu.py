@@ -114,3 +114,13 @@ def test_tuner_memoises_skips_illegal_and_keeps_the_fastest(monkeypatch):
     # every candidate illegal -> assertion
     with pytest.raises(AssertionError, match='Failed to tune'):
         t.compile_and_tune(name='op2', keys={'KEY': 3}, space=({'T': 'bad'}, {'T': 'bad'}), **kw)
+
+
+def test_reference_package_name_is_an_alias():
+    """Code written against the reference imports `yan` (tests/test_cute.py:5-6 there); here that name resolves to
+    this package, with the names that test uses."""
+    import yan as by_reference_name
+    assert by_reference_name is yan
+    for name in ('gemm_fp16_tn', 'bench_kineto', 'get_col_major_tensor', 'calc_diff', 'jit', 'jit_kernels', 'gemm'):
+        assert hasattr(by_reference_name, name), name
+    assert callable(by_reference_name.jit_kernels.cute_gemm_accuracy_test)
