@@ -6,7 +6,8 @@
 // the reference kernel (cute_gemm.cuh:14-260) is a 128x128x32 cp.async/ldmatrix/mma.sync pipeline with fp16
 // accumulation and no bounds handling. Here:
 //   * macro tile BLOCK_M x BLOCK_N x 64 (128-byte rows), 4 waves, one per SIMD;
-//   * HBM -> LDS with buffer_load ... lds into two static LDS stages (tile_io.hpp);
+//   * HBM -> LDS with buffer_load ... lds (tile_io.hpp) into NUM_STAGES LDS stages: two for the 256 x 256 tile, a ring
+//     of three to eight for the smaller tiles, which run problems bound by operand streaming;
 //   * each wave owns a (BLOCK_N/WAVES_N) x (BLOCK_M/WAVES_M) slab, up to 128 x 128 (256 accumulator registers, which
 //     the compiler keeps in AGPRs), computed with 32x32x16 MFMAs: the larger the slab, the fewer LDS bytes are read
 //     per flop, and on a part whose clock is set by power that is what buys throughput. B rows feed the

@@ -4,9 +4,11 @@
 // kernel signature :40-46, BLOCK_K == 128 :48, one A scale per row and K block and one or two B scales per tile
 // and K block :55-61), which in the reference is an unfinished Hopper kernel built on TMA descriptors, cluster
 // barriers and warpgroup MMAs. This is a different kernel for gfx950:
-//   * macro tile BLOCK_M x BLOCK_N x 128 (one scale block per k-tile, 128-byte rows); 8 waves, two per SIMD, so
-//     one wave's scale arithmetic and LDS traffic hide under the other's MFMAs;
-//   * HBM -> LDS with buffer_load ... lds into two static LDS stages (tile_io.hpp);
+//   * macro tile BLOCK_M x BLOCK_N x 128 (one scale block per k-tile, 128-byte rows); 8 waves, two per SIMD, for
+//     the tiles from 256 x 128 up, so one wave's scale arithmetic and LDS traffic hide under the other's MFMAs;
+//     4 waves below that;
+//   * HBM -> LDS with buffer_load ... lds (tile_io.hpp) into two LDS stages for the 256 x 256 tile and into a ring of
+//     3 to 8 stages for the smaller tiles, which run problems bound by operand streaming;
 //   * 16x16x128 e4m3 MFMAs: one instruction covers a whole scale block, starts from a zero accumulator and
 //     yields 4 partial sums per lane, which the VALU folds into the running fp32 sums as acc += partial * s,
 //     s = sA * sB. Weights feed the MFMA row operand and activations the column operand, so a lane only ever
