@@ -323,6 +323,29 @@ def test_fp8_decode_shapes_are_repeatable():
     assert oracle.calc_diff(_np(first_one), _fp8_ref(e8, se, f8, sf)) < 1e-5
 
 
+@pytest.mark.parametrize('m,n,k', [(128, 4096, 7168), (512, 4096, 2048), (1024, 7168, 1024)])
+def test_ring_of_stages_is_race_free(m, n, k):
+    """Tiles below 256 x 256 keep several k-tiles in flight in a ring of LDS stages, synchronised by counting the
+    wave's outstanding copies. A slip there would show as run-to-run differences: 30 launches, cache flushed between
+    some of them so that the copies land in a different order, must give the same bits, FP8 and bf16."""
+    (a8, sa), (b8, sb), out = testing.make_fp8_case(m, n, k, seed=11, device='cuda', gen_device='cuda')
+    a, b, c = testing.make_bf16_case(m, n, k, seed=12, scale=k ** -0.5, device='cuda', gen_device='cuda')
+    yan.gemm_fp8_fp8_bf16_nt((a8, sa), (b8, sb), out)
+    yan.gemm_bf16_tn(a, b, c)
+    first8, first16 = out.clone(), c.clone()
+    assert float(yan.calc_diff(first8.float(), testing.dequant_lhs(a8, sa) @ testing.dequant_rhs(b8, sb).t())) < 1e-3
+    assert float(yan.calc_diff(first16.float(), a.float() @ b.float().t())) < 1e-5
+    flush = torch.empty(512 << 18, dtype=torch.int, device='cuda')
+    for it in range(30):
+        if it % 3 == 0:
+            flush.zero_()
+        out.fill_(float('nan'))
+        c.fill_(float('nan'))
+        yan.gemm_fp8_fp8_bf16_nt((a8, sa), (b8, sb), out)
+        yan.gemm_bf16_tn(a, b, c)
+        assert torch.equal(out, first8) and torch.equal(c, first16), it
+
+
 def test_fp8_outlier_16384_cubed():
     """cfg5: uniform[-4,4] sources with 1% of entries x50. Sampled rows against the oracle, plus finiteness."""
     m, n, k = testing.BASELINE_FP8['cfg5']

@@ -137,6 +137,7 @@ DENSE_TEST_SHAPES = [
     (128, 256, 256), (64, 64, 64), (1, 64, 64), (255, 132, 72), (300, 520, 8), (33, 4, 200), (257, 1028, 1096),
     (300, 256, 256), (33, 132, 72), (96, 80, 136),
     (256, 5120, 5120), (4096, 2048, 7168), (4096, 7168, 2048), (256, 24576, 1536),
+    (128, 4096, 7168), (512, 4096, 2048), (1024, 7168, 1024),
 ]
 # (m, n, k) of the reference's own dense test (tests/test_cute.py:21-22: m in (256, 4096) x six (k, n) pairs)
 REFERENCE_DENSE_TEST_SHAPES = [(m, n, k) for m in (256, 4096)
@@ -147,6 +148,7 @@ FP8_TEST_SHAPES = [
     (40, 192, 256), (130, 448, 640),
     (257, 2112, 1024), (128, 7168, 2048), (4096, 2048, 7168),
     (1, 4096, 7168), (17, 4096, 1024), (33, 2112, 640), (64, 7168, 2048), (48, 4100, 384), (40, 2112, 640),
+    (128, 4096, 7168), (512, 4096, 2048), (1024, 7168, 1024),
 ]
 # Grouped FP8 GEMMs: (rows per group, n, k, blocks of padding rows) and (groups, m_max, n, k, masked_m, expected_m).
 GROUPED_CONTIGUOUS_TEST_CASES = [
