@@ -79,6 +79,7 @@ dense_gemm_body(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, El
     using StA = TileStager<BLOCK_M, NW>;
     using StB = TileStager<BLOCK_N, NW>;
     constexpr int NUM_COPIES = StA::PASSES + StB::PASSES;
+    static_assert(StA::PADDED_ROWS == BLOCK_M && StB::PADDED_ROWS == BLOCK_N, "tiles are whole copy passes");
     // Copy number `d` (A passes first, then B passes) of k-tile `kt` into the given stage.
     auto copy_pass = [&](int d, int kt, uint8_t* la, uint8_t* lb) {
         const bool tail = kt == tail_tile;

@@ -45,12 +45,14 @@ struct Fp8TileConfig {
     static constexpr bool UNIFORM_SCALE_B = (128 % WTN == 0);
     // Number of 128-wide scale blocks a slab of 16-aligned start can touch.
     static constexpr int  SCALE_B_PER_SLAB = UNIFORM_SCALE_B ? 1 : (WTN + 112) / 128 + 1;
-    static constexpr int  LDS_BYTES = 2 * (BLOCK_M + BLOCK_N) * kRowBytes;
+    // LDS rows of the two operand tiles: whole copy passes (tile_io.hpp), i.e. rounded up to 8 rows per wave.
+    static constexpr int  LDS_ROWS_A = TileStager<BLOCK_M, NUM_WAVES>::PADDED_ROWS, LDS_ROWS_B = TileStager<BLOCK_N, NUM_WAVES>::PADDED_ROWS;
+    static constexpr int  LDS_BYTES = 2 * (LDS_ROWS_A + LDS_ROWS_B) * kRowBytes;
     static_assert(LDS_BYTES <= 160 * 1024, "two stages must fit the 160 KB LDS");
     // Ring of more than two stages (tiles below 256 x 256, where one k-tile in flight does not cover the memory
     // latency of an operand-streaming problem): a stage also carries the k-tile's BLOCK_M activation scales.
     static constexpr int  RING_SCALE_BYTES = ceil_div(BLOCK_M * 4, 1024) * 1024;
-    static constexpr int  RING_STAGE_BYTES = (BLOCK_M + BLOCK_N) * kRowBytes + RING_SCALE_BYTES;
+    static constexpr int  RING_STAGE_BYTES = (LDS_ROWS_A + LDS_ROWS_B) * kRowBytes + RING_SCALE_BYTES;
     static constexpr bool RING_CAPABLE = BLOCK_M % 64 == 0 && (BLOCK_M / 8) % NUM_WAVES == 0 && BLOCK_N % 16 == 0;
     static constexpr int  MAX_RING_STAGES = RING_CAPABLE ? (160 * 1024 / RING_STAGE_BYTES < 8 ? 160 * 1024 / RING_STAGE_BYTES : 8) : 2;
 };
@@ -139,6 +141,7 @@ fp8_gemm_kernel(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_s
     const uint32_t sa_voff = uint32_t(m_slab + col) * sa_stride_m * 4;
     // Weight scales: rows base_blk .. base_blk+NB-1 of the [N/128, K/128] table cover the slab.
     const int base_blk = n_slab / 128;
+    [[maybe_unused]] const int rows_in_first_block = (128 - (n_slab & 127)) / 16;     // only for slabs that straddle blocks
 
     const int off0 = frag_offset<16>(lane, 2 * g), off1 = frag_offset<16>(lane, 2 * g + 1);
     auto read_frag = [&](const uint8_t* atom_rows) {
@@ -177,6 +180,7 @@ fp8_gemm_kernel(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_s
 #pragma unroll
         for (int j = 0; j < TM; ++j) mf[j] = read_frag(pa + j * 16 * kRowBytes);
         float s[TM];
+        [[maybe_unused]] float s_first[TM], s_second[TM];
         f32x4 p[RING];
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -189,19 +193,26 @@ fp8_gemm_kernel(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_s
             }
             if (t >= DEPTH) {
                 const int u = t - DEPTH, i = u / TM, j = u % TM;
-                if (j == 0) {
-                    // (re)compute s = sA * sB on entering the slab and whenever rows i cross into the next 128-block
-                    const bool fresh = (i == 0) || (!Cfg::UNIFORM_SCALE_B && ((n_slab + i * 16) & 127) == 0);
-                    if (fresh) {
-                        float sbv = sb[0];
-                        if constexpr (NB > 1) {
-                            const int rel = (n_slab + i * 16) / 128 - base_blk;
+                if constexpr (Cfg::UNIFORM_SCALE_B) {
+                    if (u == 0) {
 #pragma unroll
-                            for (int b = 1; b < NB; ++b) sbv = (rel == b) ? sb[b] : sbv;
-                        }
-#pragma unroll
-                        for (int jj = 0; jj < TM; ++jj) s[jj] = sa[jj] * sbv;
+                        for (int jj = 0; jj < TM; ++jj) s[jj] = sa[jj] * sb[0];
                     }
+                } else if (j == 0) {
+                    // A slab that is not a divisor of 128 wide crosses at most one boundary between weight-scale
+                    // blocks: rows of atoms below `rows_in_first_block` take block 0's scale, the others block 1's.
+                    // Both products are formed once per k-tile and each row picks its own with a bit select under a
+                    // wave-uniform mask: no branch, so the steps stay in one basic block.
+                    static_assert(NB == 2, "a slab narrower than 128 touches at most two scale blocks");
+                    if (i == 0) {
+#pragma unroll
+                        for (int jj = 0; jj < TM; ++jj) { s_first[jj] = sa[jj] * sb[0]; s_second[jj] = sa[jj] * sb[1]; }
+                    }
+                    const uint32_t pick_second = i >= rows_in_first_block ? 0xffffffffu : 0u;
+#pragma unroll
+                    for (int jj = 0; jj < TM; ++jj)
+                        s[jj] = __builtin_bit_cast(float, (__builtin_bit_cast(uint32_t, s_second[jj]) & pick_second) |
+                                                          (__builtin_bit_cast(uint32_t, s_first[jj]) & ~pick_second));
                 }
 #pragma unroll
                 for (int r = 0; r < 4; ++r) acc[i][j][r] = __builtin_fmaf(p[u % RING][r], s[j], acc[i][j][r]);
@@ -250,10 +261,10 @@ fp8_gemm_kernel(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_s
 #pragma unroll
         for (int j = 0; j < TM; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
     if constexpr (STAGES == 2) {
-    __shared__ __attribute__((aligned(1024))) uint8_t lds_a0[BLOCK_M * kRowBytes];
-    __shared__ __attribute__((aligned(1024))) uint8_t lds_b0[BLOCK_N * kRowBytes];
-    __shared__ __attribute__((aligned(1024))) uint8_t lds_a1[BLOCK_M * kRowBytes];
-    __shared__ __attribute__((aligned(1024))) uint8_t lds_b1[BLOCK_N * kRowBytes];
+    __shared__ __attribute__((aligned(1024))) uint8_t lds_a0[Cfg::LDS_ROWS_A * kRowBytes];
+    __shared__ __attribute__((aligned(1024))) uint8_t lds_b0[Cfg::LDS_ROWS_B * kRowBytes];
+    __shared__ __attribute__((aligned(1024))) uint8_t lds_a1[Cfg::LDS_ROWS_A * kRowBytes];
+    __shared__ __attribute__((aligned(1024))) uint8_t lds_b1[Cfg::LDS_ROWS_B * kRowBytes];
     stage_a.issue(rsrc_a, lds_a0, 0, wave);
     stage_b.issue(rsrc_b, lds_b0, 0, wave);
     load_scales(0);
@@ -264,21 +275,19 @@ fp8_gemm_kernel(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_s
     if (NUM_K_BLOCKS % 2 == 1) k_step(NUM_K_BLOCKS - 1, lds_a0, lds_b0, lds_a1, lds_b1);
     } else {
     // Ring of STAGES stages, STAGES - 1 k-tiles in flight: what a small tile needs when the problem is bound by
-    // streaming its operands and one k-tile of prefetch cannot cover the memory latency. A wave issues the same
-    // number of copies for every k-tile (OPS, one fewer for the waves that have no part in the last pass over a narrow
-    // weight tile), in the same order, so "k-tile kb has landed" is "at most (STAGES - 2) * OPS of my copies are
-    // outstanding". The activation scales of a k-tile travel through the stage as well (a register load between the
+    // streaming its operands and one k-tile of prefetch cannot cover the memory latency. Every wave issues the same
+    // number of copies for every k-tile (OPS), in the same order, so "k-tile kb has landed" is "at most
+    // (STAGES - 2) * OPS of my copies are outstanding". The activation scales of a k-tile travel through the stage as well (a register load between the
     // copies would make the in-order counter wait for every older copy): every wave copies one 64-row part of them
     // with one full-width instruction; waves that share a part write the same bytes twice.
-    constexpr int STAGE_BYTES = Cfg::RING_STAGE_BYTES, TILE_BYTES = (BLOCK_M + BLOCK_N) * kRowBytes;
+    constexpr int STAGE_BYTES = Cfg::RING_STAGE_BYTES, A_BYTES = Cfg::LDS_ROWS_A * kRowBytes, TILE_BYTES = A_BYTES + Cfg::LDS_ROWS_B * kRowBytes;
     constexpr int OPS = StA::PASSES + StB::PASSES + 1, SCALE_PARTS = BLOCK_M / 64;
     static_assert(Cfg::RING_CAPABLE && (STAGES - 2) * OPS <= 63 && STAGES * STAGE_BYTES <= 160 * 1024);
-    constexpr int FULL_B_WAVES = StB::GROUPS % NW == 0 ? NW : StB::GROUPS % NW;      // waves that take part in the last B pass
     __shared__ __attribute__((aligned(1024))) uint8_t ring[STAGES * STAGE_BYTES];
     const uint32_t scale_voff = uint32_t(m0 + lane) * sa_stride_m * 4;
     auto issue_op = [&](int d, int kb, uint8_t* stage) {
         if (d < StA::PASSES) stage_a.issue_pass(rsrc_a, stage, kb * kRowBytes, wave, d);
-        else if (d < StA::PASSES + StB::PASSES) stage_b.issue_pass(rsrc_b, stage + BLOCK_M * kRowBytes, kb * kRowBytes, wave, d - StA::PASSES);
+        else if (d < StA::PASSES + StB::PASSES) stage_b.issue_pass(rsrc_b, stage + A_BYTES, kb * kRowBytes, wave, d - StA::PASSES);
         else {
             const int part = wave % SCALE_PARTS;                    // rows m0 + 64 * part + lane
             __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_sa, YAN_LDS_PTR(stage + TILE_BYTES + part * 256), 4,
@@ -294,8 +303,7 @@ fp8_gemm_kernel(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_s
     for (int kb = 0; kb < NUM_K_BLOCKS; ++kb) {
 #pragma unroll
         for (int b = 0; b < NB; ++b) sb_cur[b] = sb_next[b];
-        if (FULL_B_WAVES == NW || wave < FULL_B_WAVES) __builtin_amdgcn_s_waitcnt(waitcnt_imm((STAGES - 2) * OPS, kNoWaitLgkm));
-        else __builtin_amdgcn_s_waitcnt(waitcnt_imm((STAGES - 2) * (OPS - 1), kNoWaitLgkm));
+        __builtin_amdgcn_s_waitcnt(waitcnt_imm((STAGES - 2) * OPS, kNoWaitLgkm));
         asm volatile("" ::: "memory");
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
@@ -306,7 +314,7 @@ fp8_gemm_kernel(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_s
         const float* my_scales = reinterpret_cast<const float*>(cur + TILE_BYTES) + wm * Cfg::WTM + col;
 #pragma unroll
         for (int j = 0; j < TM; ++j) sa_cur[j] = my_scales[j * 16];
-        compute_tile(cur, cur + BLOCK_M * kRowBytes, sa_cur, sb_cur, [&](int row) {
+        compute_tile(cur, cur + A_BYTES, sa_cur, sb_cur, [&](int row) {
 #pragma unroll
             for (int d = 0; d < OPS; ++d)
                 if (d * SPREAD_ROWS / OPS == row) issue_op(d, kb + STAGES - 1, nxt);

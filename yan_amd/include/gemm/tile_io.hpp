@@ -51,6 +51,10 @@ struct TileStager {
     static_assert(ROWS % 16 == 0 && NUM_WAVES % 2 == 0);
     static constexpr int GROUPS = ROWS / 8;                       // 8-row groups, one instruction each
     static constexpr int PASSES = ceil_div(GROUPS, NUM_WAVES);
+    // Every wave issues every pass, so that the steady state of a k-loop has no wave-dependent branch and every wave
+    // has the same number of copies in flight. A wave whose group lies past the tile (only possible in the last
+    // pass) is sent out of range and moves zeros into rows ROWS .. PADDED_ROWS - 1, which the LDS tile must have.
+    static constexpr int PADDED_ROWS = PASSES * NUM_WAVES * 8;
 
     uint32_t voff;        // byte offset of this lane's chunk for pass 0 at K = 0
     uint32_t pass_pitch;  // bytes between the rows of consecutive passes (uniform)
@@ -83,9 +87,9 @@ struct TileStager {
     __device__ __forceinline__ void issue_pass_from(__amdgpu_buffer_rsrc_t rsrc, uint8_t* lds_tile, int k_byte0, int wave, int j,
                                                     uint32_t lane_voff) const {
         const int q = j * NUM_WAVES + wave;
-        if (GROUPS % NUM_WAVES == 0 || q < GROUPS)
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, YAN_LDS_PTR(lds_tile + q * 8 * kRowBytes), kChunk, lane_voff,
-                                                     k_byte0 + j * pass_pitch, 0, 0);
+        const uint32_t past_tile = (GROUPS % NUM_WAVES == 0 || q < GROUPS) ? 0u : kOutOfRange;
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, YAN_LDS_PTR(lds_tile + q * 8 * kRowBytes), kChunk, lane_voff | past_tile,
+                                                 k_byte0 + j * pass_pitch, 0, 0);
     }
 
     __device__ __forceinline__ void issue_from(__amdgpu_buffer_rsrc_t rsrc, uint8_t* lds_tile, int k_byte0, int wave,
@@ -93,9 +97,9 @@ struct TileStager {
 #pragma unroll
         for (int j = 0; j < PASSES; ++j) {
             const int q = j * NUM_WAVES + wave;
-            if (GROUPS % NUM_WAVES == 0 || q < GROUPS)
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, YAN_LDS_PTR(lds_tile + q * 8 * kRowBytes), kChunk,
-                                                         lane_voff, k_byte0 + j * pass_pitch, 0, 0);
+            const uint32_t past_tile = (GROUPS % NUM_WAVES == 0 || q < GROUPS) ? 0u : kOutOfRange;
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, YAN_LDS_PTR(lds_tile + q * 8 * kRowBytes), kChunk,
+                                                     lane_voff | past_tile, k_byte0 + j * pass_pitch, 0, 0);
         }
     }
 };

@@ -49,7 +49,8 @@ def get_fp8_num_stages(block_m: int, block_n: int) -> int:
     capable = block_m % 64 == 0 and (block_m // 8) % waves == 0 and block_n % 16 == 0
     if not capable:
         return 2
-    stage_bytes = (block_m + block_n) * 128 + ceil_div(block_m * 4, 1024) * 1024
+    rows = ceil_div(block_m, 8 * waves) * 8 * waves + ceil_div(block_n, 8 * waves) * 8 * waves      # whole copy passes
+    stage_bytes = rows * 128 + ceil_div(block_m * 4, 1024) * 1024
     return max(2, min(8, 160 * 1024 // stage_bytes))
 
 
