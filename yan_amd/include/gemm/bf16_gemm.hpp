@@ -146,33 +146,73 @@ dense_gemm_body(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, El
         }
     };
 
-    // Two LDS stages; the copy of tile kt+1 is in flight while tile kt is consumed. The barrier both publishes
-    // the tile that just landed and retires every wave's reads of the stage about to be overwritten. The copies
-    // are started a few at a time during the first two of the four steps rather than in one burst after the
-    // barrier, so the memory pipeline's issue time hides under MFMAs and the copies still get half a k-tile to
-    // land. The steady-state body is branch-free: a copy started for a tile past the end is never consumed.
-    auto k_step = [&](int kt, const uint8_t* a_cur, const uint8_t* b_cur, uint8_t* a_nxt, uint8_t* b_nxt) {
-        wait_for_copies();
-        __syncthreads();
-        compute_tile(a_cur, b_cur, [&](int kk) {
-#pragma unroll
-            for (int d = 0; d < NUM_COPIES; ++d)
-                if (d * SPREAD_STEPS / NUM_COPIES == kk) copy_pass(d, kt + 1, a_nxt, b_nxt);
-        });
-    };
     if constexpr (STAGES == 2) {
         __shared__ __attribute__((aligned(1024))) uint8_t lds_a0[BLOCK_M * kRowBytes];
         __shared__ __attribute__((aligned(1024))) uint8_t lds_b0[BLOCK_N * kRowBytes];
         __shared__ __attribute__((aligned(1024))) uint8_t lds_a1[BLOCK_M * kRowBytes];
         __shared__ __attribute__((aligned(1024))) uint8_t lds_b1[BLOCK_N * kRowBytes];
+        // The barrier that publishes k-tile kt+1 sits before the LAST of the four steps of k-tile kt, not at the tile
+        // boundary: the MFMAs of that step have their operands in registers already, so the first fragment reads of
+        // the new tile (and the time the waves need to meet) hide under sixteen MFMAs instead of stalling the matrix
+        // core of a SIMD that has no second wave to run. The copies of k-tile kt+2 go to the stage k-tile kt used,
+        // which every wave has finished reading when it is past that barrier; half of them are started in that last
+        // step and half in the first step of the next tile, which leaves them two to three steps to land, as before.
+        using Frag = typename Atom::Frag;
+        Frag nf[2][TN], mf[2][TM];
+        auto fetch_from = [&](const uint8_t* la, const uint8_t* lb, int kk) {
+            const uint8_t* pa = la + wm * Cfg::WTM * kRowBytes;
+            const uint8_t* pb = lb + wn * Cfg::WTN * kRowBytes;
+#pragma unroll
+            for (int i = 0; i < TN; ++i) nf[kk & 1][i] = *reinterpret_cast<const Frag*>(pb + i * 32 * kRowBytes + koff[kk]);
+#pragma unroll
+            for (int j = 0; j < TM; ++j) mf[kk & 1][j] = *reinterpret_cast<const Frag*>(pa + j * 32 * kRowBytes + koff[kk]);
+        };
+        auto mma_step = [&](int kk, int copies) {
+#pragma unroll
+            for (int i = 0; i < TN; ++i)
+#pragma unroll
+                for (int j = 0; j < TM; ++j) acc[i][j] = Atom::mma(nf[kk & 1][i], mf[kk & 1][j], acc[i][j]);
+            constexpr int kDsRead = 0x100, kVmem = 0x020, kMfma = 0x008;
+#pragma unroll
+            for (int x = 0; x < TN * TM; ++x) {
+                if (x < TN + TM) __builtin_amdgcn_sched_group_barrier(kDsRead, 1, 0);
+                if (x < copies) __builtin_amdgcn_sched_group_barrier(kVmem, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(kMfma, 1, 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        };
+        constexpr int FIRST_HALF = NUM_COPIES / 2;
+        // On entry the fragments of (kt, step 0) are in registers and the first half of k-tile kt+1's copies is under way.
+        auto rotated_tile = [&](int kt, uint8_t* a_cur, uint8_t* b_cur, uint8_t* a_nxt, uint8_t* b_nxt) {
+#pragma unroll
+            for (int kk = 0; kk < 3; ++kk) {
+                if (kk == 0) {
+#pragma unroll
+                    for (int d = FIRST_HALF; d < NUM_COPIES; ++d) copy_pass(d, kt + 1, a_nxt, b_nxt);
+                }
+                fetch_from(a_cur, b_cur, kk + 1);
+                mma_step(kk, kk == 0 ? NUM_COPIES - FIRST_HALF : 0);
+            }
+            __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 0));      // my reads of this stage and my copies of k-tile kt+1 are done
+            __syncthreads();
+#pragma unroll
+            for (int d = 0; d < FIRST_HALF; ++d) copy_pass(d, kt + 2, a_cur, b_cur);
+            fetch_from(a_nxt, b_nxt, 0);
+            mma_step(3, FIRST_HALF);
+        };
 #pragma unroll
         for (int d = 0; d < NUM_COPIES; ++d) copy_pass(d, 0, lds_a0, lds_b0);
+        wait_for_copies();
+        __syncthreads();
+        fetch_from(lds_a0, lds_b0, 0);
+#pragma unroll
+        for (int d = 0; d < FIRST_HALF; ++d) copy_pass(d, 1, lds_a1, lds_b1);
         int kt = 0;
         for (; kt + 1 < num_k_tiles; kt += 2) {
-            k_step(kt, lds_a0, lds_b0, lds_a1, lds_b1);
-            k_step(kt + 1, lds_a1, lds_b1, lds_a0, lds_b0);
+            rotated_tile(kt, lds_a0, lds_b0, lds_a1, lds_b1);
+            rotated_tile(kt + 1, lds_a1, lds_b1, lds_a0, lds_b0);
         }
-        if (kt < num_k_tiles) k_step(kt, lds_a0, lds_b0, lds_a1, lds_b1);
+        if (kt < num_k_tiles) rotated_tile(kt, lds_a0, lds_b0, lds_a1, lds_b1);
     } else {
         // Ring: every wave issues NUM_COPIES copies per k-tile, in the same order, so "k-tile kt has landed" is "at
         // most (STAGES - 2) * NUM_COPIES of my copies are outstanding". The copies of k-tile kt + STAGES - 1 go to
