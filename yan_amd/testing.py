@@ -163,62 +163,57 @@ GROUPED_MASKED_TEST_CASES = [
 ]
 
 
-def prebuild_jit_kernels(num_cus: int = 256, verbose: bool = False) -> int:
-    """Compile every JIT kernel the shapes above select (hipcc cross-compiles for gfx950 without a GPU) into the
-    current kernel cache. Returns the number of distinct kernels."""
-    from .jit import build, cpp_format, generate
-    from .jit_kernels import bf16_gemm, gemm
-    seen = set()
+def jit_kernels_in_use(num_cus: int = 256):
+    """(name, arg_defs, code) of every distinct JIT kernel the shapes above, the quantisers and the probe select."""
+    from . import probe
+    from .jit import cpp_format, generate
+    from .jit_kernels import bf16_gemm, fp8_cast, gemm, m_grouped_gemm
+    kernels = {}
+
+    def add(name, arg_defs, includes, code_template, keys):
+        code = generate(includes, arg_defs, cpp_format(code_template, keys))
+        kernels.setdefault((name, code), (name, arg_defs, code))
+
     for m, n, k in DENSE_TEST_SHAPES + REFERENCE_DENSE_TEST_SHAPES:
         for dtype in (torch.bfloat16, torch.half):
-            if m == 0 or n == 0:
-                continue
-            name, keys, arg_defs = bf16_gemm.dense_kernel_plan(m, n, k, dtype, num_cus)
-            code = generate(bf16_gemm.includes, arg_defs, cpp_format(bf16_gemm.template, keys))
-            if (name, code) not in seen:
-                seen.add((name, code))
-                rt = build(name, arg_defs, code)
-                if verbose:
-                    print(f'built {name} {keys} -> {rt.path}')
+            if m and n:
+                name, keys, arg_defs = bf16_gemm.dense_kernel_plan(m, n, k, dtype, num_cus)
+                add(name, arg_defs, bf16_gemm.includes, bf16_gemm.template, keys)
     for m, n, k in FP8_TEST_SHAPES:
-        if m == 0:
-            continue
-        name, keys, arg_defs, _, code_template = gemm.fp8_kernel_plan(m, n, k, num_cus)
-        code = generate(gemm.includes, arg_defs, cpp_format(code_template, keys))
-        if (name, code) not in seen:
-            seen.add((name, code))
-            rt = build(name, arg_defs, code)
-            if verbose:
-                print(f'built {name} {keys} -> {rt.path}')
-    from . import probe
-    from .jit_kernels import fp8_cast, m_grouped_gemm
+        if m:
+            name, keys, arg_defs, _, code_template = gemm.fp8_kernel_plan(m, n, k, num_cus)
+            add(name, arg_defs, gemm.includes, code_template, keys)
     name, arg_defs, code = probe.probe_kernel()
-    seen.add((name, code))
-    build(name, arg_defs, code)
+    kernels.setdefault((name, code), (name, arg_defs, code))
     for kind in ('per_token', 'per_block'):
         for dtype in (torch.bfloat16, torch.float32):
             name, keys, arg_defs, code_template = fp8_cast.cast_kernel_plan(kind, dtype)
-            code = generate(fp8_cast.includes, arg_defs, cpp_format(code_template, keys))
-            seen.add((name, code))
-            rt = build(name, arg_defs, code)
-            if verbose:
-                print(f'built {name} {keys} -> {rt.path}')
+            add(name, arg_defs, fp8_cast.includes, code_template, keys)
     for rows, n, k, pad_blocks in GROUPED_CONTIGUOUS_TEST_CASES:
         m = sum((r + 127) // 128 * 128 for r in rows) + 128 * pad_blocks
-        plans = [m_grouped_gemm.grouped_kernel_plan('GroupedContiguous', len(rows), m, n, k, num_cus)]
-        for name, keys, arg_defs, _ in plans:
-            code = generate(m_grouped_gemm.includes, arg_defs, cpp_format(m_grouped_gemm.template, keys))
-            if (name, code) not in seen:
-                seen.add((name, code))
-                rt = build(name, arg_defs, code)
-                if verbose:
-                    print(f'built {name} {keys} -> {rt.path}')
+        name, keys, arg_defs, _ = m_grouped_gemm.grouped_kernel_plan('GroupedContiguous', len(rows), m, n, k, num_cus)
+        add(name, arg_defs, m_grouped_gemm.includes, m_grouped_gemm.template, keys)
     for groups, m_max, n, k, _, expected_m in GROUPED_MASKED_TEST_CASES:
         name, keys, arg_defs, _ = m_grouped_gemm.grouped_kernel_plan('GroupedMasked', groups, min(expected_m, m_max), n, k, num_cus)
-        code = generate(m_grouped_gemm.includes, arg_defs, cpp_format(m_grouped_gemm.template, keys))
-        if (name, code) not in seen:
-            seen.add((name, code))
-            rt = build(name, arg_defs, code)
-            if verbose:
-                print(f'built {name} {keys} -> {rt.path}')
-    return len(seen)
+        add(name, arg_defs, m_grouped_gemm.includes, m_grouped_gemm.template, keys)
+    return list(kernels.values())
+
+
+def prebuild_jit_kernels(num_cus: int = 256, verbose: bool = False, jobs: int = 0) -> int:
+    """Compile every JIT kernel of `jit_kernels_in_use` (hipcc cross-compiles for gfx950 without a GPU) into the
+    current kernel cache, `jobs` compilers at a time (default: one per CPU, at most 8). Returns the number of kernels."""
+    import os
+    from concurrent.futures import ThreadPoolExecutor
+    from .jit import build
+    kernels = jit_kernels_in_use(num_cus)
+    jobs = jobs or max(1, min(8, os.cpu_count() or 1))
+
+    def one(kernel):
+        runtime = build(*kernel)
+        if verbose:
+            print(f'built {kernel[0]} -> {runtime.path}')
+        return runtime
+
+    with ThreadPoolExecutor(max_workers=jobs) as pool:
+        list(pool.map(one, kernels))
+    return len(kernels)
