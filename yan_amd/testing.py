@@ -150,16 +150,22 @@ FP8_TEST_SHAPES = [
     (1, 4096, 7168), (17, 4096, 1024), (33, 2112, 640), (64, 7168, 2048), (48, 4100, 384), (40, 2112, 640),
     (128, 4096, 7168), (512, 4096, 2048), (1024, 7168, 1024),
 ]
+# Plain FP8 calls the grouped and quantiser tests make on the side (first group through the plain entry, quantise-then-
+# multiply): listed so that their kernels are compiled ahead of time as well.
+FP8_SIDE_SHAPES = [(1024, 4096, 7168), (8192, 4096, 7168), (200, 384, 512), (1152, 512, 512), (128, 4096, 1024), (128, 320, 384),
+                   (256, 200, 128)]
 # Grouped FP8 GEMMs: (rows per group, n, k, blocks of padding rows) and (groups, m_max, n, k, masked_m, expected_m).
 GROUPED_CONTIGUOUS_TEST_CASES = [
     ((100, 128, 1, 300), 320, 384, 1), ((128, 128), 4096, 1024, 0), ((129,), 200, 128, 2),
     ((1024, 1024, 1024, 1024), 4096, 7168, 0), ((8192, 8192, 8192, 8192), 4096, 7168, 0),
     # long groups whose boundaries fall in the middle of 256-row tiles (two-pass tiles), with a trailing padding block
     ((1150, 900, 1300, 1100), 512, 512, 1),
+    ((128, 128), 192, 256, 1),                       # the committed fixture
 ]
 GROUPED_MASKED_TEST_CASES = [
     (3, 200, 320, 384, (200, 0, 77), 128), (4, 256, 4096, 1024, (1, 256, 130, 64), 64), (2, 64, 200, 128, (64, 3), 32),
     (4, 1024, 4096, 7168, (1024, 900, 512, 1), 1024),
+    (2, 40, 192, 256, (40, 7), 40),                  # the committed fixture
 ]
 
 
@@ -179,7 +185,7 @@ def jit_kernels_in_use(num_cus: int = 256):
             if m and n:
                 name, keys, arg_defs = bf16_gemm.dense_kernel_plan(m, n, k, dtype, num_cus)
                 add(name, arg_defs, bf16_gemm.includes, bf16_gemm.template, keys)
-    for m, n, k in FP8_TEST_SHAPES:
+    for m, n, k in FP8_TEST_SHAPES + FP8_SIDE_SHAPES:
         if m:
             name, keys, arg_defs, _, code_template = gemm.fp8_kernel_plan(m, n, k, num_cus)
             add(name, arg_defs, gemm.includes, code_template, keys)
