@@ -96,7 +96,8 @@ def main():
     ap.add_argument('--also', action='store_true', help='also time bf16 8192^3, the decode shape and 16384^3 (extra fields)')
     ap.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline leg')
     ap.add_argument('--ceilings', action='store_true',
-                    help='also measure what the matrix cores sustain with register-resident operands (random and zero bits)')
+                    help='also measure what the matrix cores sustain with register-resident operands, and what the main loop of the '
+                         'block-scaled kernel sustains on a tile that never changes (random and zero bits)')
     ap.add_argument('--calibrate-copy', action='store_true',
                     help='also run a 1 GiB device-to-device copy three times, as the known-size kernel that hardware '
                          'byte counters (FETCH_SIZE / WRITE_SIZE) are scaled by when profiling')
@@ -217,10 +218,12 @@ def main():
 
     if args.ceilings:
         from yan_amd import probe
-        line['mfma_only_ceiling_tflops'] = {kind: {data: round(probe.mfma_ceiling(kind, data), 1) for data in ('random', 'zero')}
-                                            for kind in probe.MODES}
-        fold = line['mfma_only_ceiling_tflops']['fp8_16x16x128_zero_c_plus_fold']['random']
-        line['roofline']['frac_of_mfma_only_ceiling'] = round(tflops_kernel / fold, 4)
+        line['ceilings_tflops'] = {kind: {data: round(probe.mfma_ceiling(kind, data), 1) for data in ('random', 'zero')}
+                                   for kind in probe.MODES}
+        line['roofline']['frac_of_mfma_only_ceiling'] = round(
+            tflops_kernel / line['ceilings_tflops']['fp8_16x16x128_zero_c_plus_fold']['random'], 4)
+        line['roofline']['frac_of_fed_loop_ceiling'] = round(
+            tflops_kernel / line['ceilings_tflops']['fp8_fold_plus_lds_reads_barrier_copies']['random'], 4)
 
     if not args.no_cpu:
         line['cpu_baseline'] = _cpu_baseline_fp8(a8, sa, b8, sb)

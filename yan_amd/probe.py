@@ -12,8 +12,9 @@ _body = """
 using namespace yan;
 __return_code = static_cast<int>(launch_mfma_ceiling(mode, src, out, num_cus, iters, stream));
 """
-MODES = {'bf16_32x32x16': 0, 'bf16_16x16x32': 1, 'fp8_16x16x128_accumulate': 2, 'fp8_16x16x128_zero_c_plus_fold': 3}
-_FLOPS_PER_WAVE_ITER = {0: 16 * 2 * 32 * 32 * 16, 1: 16 * 2 * 16 * 16 * 32, 2: 32 * 2 * 16 * 16 * 128, 3: 32 * 2 * 16 * 16 * 128}
+MODES = {'bf16_32x32x16': 0, 'bf16_16x16x32': 1, 'fp8_16x16x128_accumulate': 2, 'fp8_16x16x128_zero_c_plus_fold': 3,
+         'fp8_fold_plus_lds_reads': 4, 'fp8_fold_plus_lds_reads_barrier': 5, 'fp8_fold_plus_lds_reads_barrier_copies': 6}
+_FLOPS_PER_WAVE_ITER = {0: 16 * 2 * 32 * 32 * 16, 1: 16 * 2 * 16 * 16 * 32, **{mode: 32 * 2 * 16 * 16 * 128 for mode in range(2, 7)}}
 
 
 def probe_kernel():
