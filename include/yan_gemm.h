@@ -41,6 +41,16 @@ YAN_API int yan_gemm_bf16_tn(int m, int n, int k, const void* a, const void* b, 
 /* Same contraction for IEEE fp16 in / fp16 out, fp32 accumulate (the reference's dtype, cute_gemm.py:26). */
 YAN_API int yan_gemm_fp16_tn(int m, int n, int k, const void* a, const void* b, void* c, void* stream);
 
+/* c = alpha * a . b^T + beta * c in fp32 (fp32 MFMA accumulation).
+ *   a  m x k with M contiguous: element (i, kk) at a[i + kk*lda];   b  n x k with N contiguous: b[j + kk*ldb];
+ *   c  m x n row-major: c[i*ldc + j].  beta == 0 does not read c.
+ * Requires m, n, lda, ldb, ldc multiples of 4, lda >= m, ldb >= n, ldc >= n, 16-byte aligned pointers and
+ * (k + 144) * lda * 4 < 2^31 bytes, same for ldb. k == 0 scales c by beta.
+ * Replaces gemm_float_nt -> gemm_nt of the reference (yan/jit_kernels/simple_gemm.py:18-57,
+ * yan/include/gemm/simple_gemm.cuh:194-247), same argument order and memory convention. */
+YAN_API int yan_gemm_float_nt(int m, int n, int k, float alpha, const float* a, int lda, const float* b, int ldb,
+                              float beta, float* c, int ldc, void* stream);
+
 /* out[i,j] = bf16( sum_kb lhs_scales(i,kb) * rhs_scales[j/128][kb] * sum_{t<128} lhs[i][128kb+t] * rhs[j][128kb+t] )
  *   lhs        e4m3 (OCP, max 448) [m,k] row-major
  *   lhs_scales fp32, element (i,kb) at lhs_scales[i*lhs_scales_stride_m + kb*lhs_scales_stride_k]
@@ -93,13 +103,13 @@ YAN_API int yan_per_token_cast_to_fp8(const void* x, int x_is_fp32, void* q, flo
 YAN_API int yan_per_block_cast_to_fp8(const void* w, int w_is_fp32, void* q, float* scales, int n, int k, void* stream);
 
 /* Macro tile the library uses for a problem: op 0 = dense 16-bit, 1 = FP8 block-scaled, 2 = FP8 grouped contiguous
- * (m = total rows, and `k` carries the number of groups instead of the depth). Writes BLOCK_M / BLOCK_N.
+ * (m = total rows, and `k` carries the number of groups instead of the depth), 3 = fp32. Writes BLOCK_M / BLOCK_N.
  * For op 1 with few activation rows the answer is (16 * atoms, 16): the weight-streaming kernel.
  * Host-only (no device call). Stands where the reference leaves tile choice to the caller's keys
  * (yan/jit_kernels/cute_gemm.py:41, yan/jit_kernels/gemm.py:13-16). Returns 0, or 1 for an unknown op. */
 YAN_API int yan_gemm_select_tile(int op, int m, int n, int k, int num_cus, int* block_m, int* block_n);
 
-/* "yan-gemm gfx950 <n> dense + <n> fp8 tile variants + <n> weight-streaming fp8 variant + ...". */
+/* "yan-gemm gfx950 <n> dense + <n> fp32 + <n> fp8 tile variants + <n> weight-streaming fp8 variant + ...". */
 YAN_API const char* yan_gemm_version(void);
 
 /* The JIT boundary, for reference: signatures of `launch` in the kernel.so of each op

@@ -45,3 +45,17 @@ def gemm_fp8_nt(a: np.ndarray, sa: np.ndarray, b: np.ndarray, sb: np.ndarray) ->
                               ctypes.c_long(sa.strides[0] // 4), ctypes.c_long(sa.strides[1] // 4),
                               _ptr(b), _ptr(sb), _ptr(c))
     return c
+
+
+def gemm_float_nt(m: int, n: int, k: int, alpha: float, a_buf: np.ndarray, lda: int, b_buf: np.ndarray, ldb: int,
+                  beta: float, c_buf: np.ndarray, ldc: int) -> np.ndarray:
+    """Raw fp32 buffers in the C-ABI's memory convention; returns a float64 buffer shaped like `c_buf` (elements
+    outside the m x n window are left as zeros)."""
+    a_buf, b_buf = np.ascontiguousarray(a_buf, np.float32).ravel(), np.ascontiguousarray(b_buf, np.float32).ravel()
+    c_in = np.ascontiguousarray(c_buf, np.float32).ravel()
+    assert a_buf.size >= (k - 1) * lda + m and b_buf.size >= (k - 1) * ldb + n and c_in.size >= (m - 1) * ldc + n
+    c_out = np.zeros(c_in.size, np.float64)
+    load().oracle_gemm_float_nt(ctypes.c_int(m), ctypes.c_int(n), ctypes.c_int(k), ctypes.c_double(alpha), _ptr(a_buf),
+                                ctypes.c_int(lda), _ptr(b_buf), ctypes.c_int(ldb), ctypes.c_double(beta), _ptr(c_in),
+                                _ptr(c_out), ctypes.c_int(ldc))
+    return c_out

@@ -7,6 +7,9 @@
  *   oracle_gemm_fp8_nt    : c[i][j] = sum_kb sa[i][kb] * sb[j/128][kb] * sum_{t<128} A[i][128kb+t] * B[j][128kb+t]
  *                           (operands of yan/jit_kernels/gemm.py:23-30; scale granularity of
  *                            yan/include/gemm/fp8_gemm.cuh:48-61)
+ *   oracle_gemm_float_nt  : c[i*ldc + j] = alpha * sum_t a[i + t*lda] * b[j + t*ldb] + beta * c[i*ldc + j] on raw
+ *                           buffers, in the memory convention of yan/include/gemm/simple_gemm.cuh:210-214
+ *                           (A and B with their row index contiguous, C row-major); beta == 0 ignores c's old values
  */
 #include <math.h>
 #include <stdint.h>
@@ -52,5 +55,15 @@ void oracle_gemm_fp8_nt(int m, int n, int k, const uint8_t* a, const float* sa, 
                 acc += (double)sa[i * sa_stride_m + kb * sa_stride_k] * (double)sb[(size_t)(j / 128) * kblocks + kb] * part;
             }
             c[(size_t)i * n + j] = acc;
+        }
+}
+
+void oracle_gemm_float_nt(int m, int n, int k, double alpha, const float* a, int lda, const float* b, int ldb,
+                          double beta, const float* c_in, double* c_out, int ldc) {
+    for (int i = 0; i < m; ++i)
+        for (int j = 0; j < n; ++j) {
+            double acc = 0.0;
+            for (int t = 0; t < k; ++t) acc += (double)a[i + (size_t)t * lda] * (double)b[j + (size_t)t * ldb];
+            c_out[(size_t)i * ldc + j] = alpha * acc + (beta != 0.0 ? beta * (double)c_in[(size_t)i * ldc + j] : 0.0);
         }
 }

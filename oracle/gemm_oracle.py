@@ -8,6 +8,8 @@ What each function restates (paths relative to the reference tree):
                              yan/include/gemm/fp8_gemm.cuh:48-61        one A scale per row per 128-K, one B scale per
                                                                        128x128 block; the reference has no executable FP8
                                                                        path, so the closed form is the oracle
+  gemm_float_nt_ref          yan/jit_kernels/simple_gemm.py:18-57, yan/include/gemm/simple_gemm.cuh:191 (axpby):
+                             alpha * a @ b.T + beta * c on logical [m,k] / [n,k] / [m,n] arrays, in fp64
   m_grouped_gemm_contiguous_ref,
   m_grouped_gemm_masked_ref  yan/include/gemm/scheduler.cuh:7-11,31-48, yan/include/gemm/fp8_gemm.cuh:41 (the GemmType
                              enumerators and grouped_layout hook; the reference has no grouped entry point and no test):
@@ -23,13 +25,15 @@ scales giving exact integer results, single-K-block scale isolation), the indepe
 gemm_oracle.c, brute force on tiny inputs, the 256-entry e4m3 table against torch's CPU cast, and the committed
 fixtures under tests/golden/. The reference holds no golden vectors for this path. The grouped forms are pinned
 against a row-by-row brute force (every row multiplied with the weight matrix its index names, one row at a time),
-against the plain form for a single group, and by permuting the groups.
+against the plain form for a single group, and by permuting the groups. gemm_float_nt_ref is pinned by closed forms
+(identity, the ones pattern, alpha / beta linearity) and, together with the memory convention of the C ABI, by the
+raw-buffer triple loop oracle_gemm_float_nt in gemm_oracle.c.
 """
 import numpy as np
 
 __all__ = ['calc_diff', 'e4m3fn_decode_table', 'e4m3fn_decode', 'e4m3fn_encode', 'bf16_bits_to_f32', 'f32_to_bf16_bits',
            'bf16_round', 'per_token_cast_to_fp8', 'per_block_cast_to_fp8', 'dequant_lhs', 'dequant_rhs',
-           'gemm_bf16_tn_ref', 'gemm_fp8_block_scaled_ref', 'gemm_fp8_blockwise_f32',
+           'gemm_bf16_tn_ref', 'gemm_float_nt_ref', 'gemm_fp8_block_scaled_ref', 'gemm_fp8_blockwise_f32',
            'm_grouped_gemm_contiguous_ref', 'm_grouped_gemm_masked_ref']
 
 FP8_MAX = 448.0
@@ -138,6 +142,15 @@ def dequant_rhs(codes, scales) -> np.ndarray:
 def gemm_bf16_tn_ref(a, b, dtype=np.float32) -> np.ndarray:
     """a [m,k], b [n,k] given as fp32 arrays holding bf16-representable values (or any fp32): a @ b.T."""
     return np.asarray(a, dtype=dtype) @ np.asarray(b, dtype=dtype).T
+
+
+def gemm_float_nt_ref(a, b, c=None, alpha=1.0, beta=0.0) -> np.ndarray:
+    """a [m,k], b [n,k], c [m,n] (logical arrays, any storage order): alpha * a @ b.T + beta * c in fp64; beta == 0
+    ignores c."""
+    out = float(alpha) * (np.asarray(a, dtype=np.float64) @ np.asarray(b, dtype=np.float64).T)
+    if beta != 0.0:
+        out = out + float(beta) * np.asarray(c, dtype=np.float64)
+    return out
 
 
 def gemm_fp8_block_scaled_ref(lhs, lhs_scales, rhs, rhs_scales, dtype=np.float32) -> np.ndarray:

@@ -23,7 +23,7 @@ def _declared(repo_root):
 
 def test_library_exports_every_declared_symbol(lib, repo_root):
     declared = _declared(repo_root)
-    assert declared == sorted(capi.SYMBOLS) and len(declared) == 9
+    assert declared == sorted(capi.SYMBOLS) and len(declared) == 10
     for name in declared:
         assert hasattr(lib, name), name
     out = subprocess.check_output(['nm', '-D', '--defined-only', os.path.join(repo_root, 'yan_amd', 'csrc', 'libyan_gemm.so')], text=True)
@@ -50,6 +50,9 @@ def test_version_and_tile_selection_match_python(lib):
         for cus in (256, 80):
             for groups in (1, 4, 64):
                 assert capi.select_tile(2, m, n, groups, cus) == heuristics.get_best_grouped_fp8_config(m, n, 1024, cus, 1, 128, groups)
+    for m, n in [(128, 2112), (128, 24576), (4096, 7168), (4096, 32768), (128, 64), (5120, 2048), (256, 256)]:
+        for cus in (256, 80):
+            assert capi.select_tile(3, m, n, 512, cus) == heuristics.get_best_float_config(m, n, cus), (m, n, cus)
     bm, bn = ctypes.c_int(), ctypes.c_int()
     assert lib.yan_gemm_select_tile(7, 1, 1, 1, 256, ctypes.byref(bm), ctypes.byref(bn)) == 1
     assert lib.yan_gemm_select_tile(0, 1, 1, 1, 0, ctypes.byref(bm), ctypes.byref(bn)) == 1
@@ -63,6 +66,15 @@ def test_compute_entry_points_validate_before_touching_a_device(lib):
     assert lib.yan_gemm_bf16_tn(64, 62, 64, null, null, null, null) != 0         # n % 4
     assert lib.yan_gemm_bf16_tn(64, 64, 60, null, null, null, null) != 0         # k % 8
     assert lib.yan_gemm_bf16_tn(64, 64, 64, null, null, null, null) != 0         # null operands
+    f = ctypes.c_float
+    assert lib.yan_gemm_float_nt(0, 64, 16, f(1), null, 0, null, 64, f(0), null, 64, null) == 0            # empty problem
+    assert lib.yan_gemm_float_nt(128, 64, 16, f(1), null, 128, null, 64, f(0), null, 64, null) != 0        # null operands
+    aligned = ctypes.c_void_p(4096)
+    assert lib.yan_gemm_float_nt(126, 64, 16, f(1), aligned, 128, aligned, 64, f(0), aligned, 64, null) != 0   # m % 4
+    assert lib.yan_gemm_float_nt(128, 64, 16, f(1), aligned, 64, aligned, 64, f(0), aligned, 64, null) != 0    # lda < m
+    assert lib.yan_gemm_float_nt(128, 64, 16, f(1), aligned, 128, aligned, 64, f(0), aligned, 60, null) != 0   # ldc < n
+    assert lib.yan_gemm_float_nt(128, 64, 16, f(1), ctypes.c_void_p(4100), 128, aligned, 64, f(0), aligned, 64, null) != 0   # alignment
+    assert lib.yan_gemm_float_nt(128, 64, 1 << 22, f(1), aligned, 128, aligned, 64, f(0), aligned, 64, null) != 0   # beyond 32-bit offsets
     assert lib.yan_gemm_fp8_fp8_bf16_nt(null, null, 1, 1, null, null, null, 0, 128, 128, null, 256) == 0
     assert lib.yan_gemm_fp8_fp8_bf16_nt(null, null, 1, 1, null, null, null, 4, 128, 64, null, 256) != 0    # k % 128
     assert lib.yan_gemm_fp8_fp8_bf16_nt(null, null, 1, 1, null, null, null, 4, 126, 128, null, 256) != 0   # n % 4

@@ -177,6 +177,105 @@ def test_fp16_kernel_answers_to_the_reference_kernel_name():
     assert yan.jit_kernels.cute_gemm_accuracy_test is yan.jit_kernels.bf16_gemm_accuracy_test
 
 
+# ----------------------------------------------------------------------------- fp32 GEMM with alpha / beta
+FLOAT_TOL = 1e-10       # calc_diff against the fp64 product; fp32 accumulation of N(0,1) data sits near 1e-14
+
+
+def _float_close(got, want, k):
+    return np.allclose(got, want, rtol=1e-5, atol=1e-5 * max(1.0, float(np.abs(want).max())))
+
+
+@pytest.mark.parametrize('m,n,k', testing.FLOAT_TEST_SHAPES)
+def test_float_gemm_parity_vs_oracle_with_alpha_beta(m, n, k):
+    _announce('fp32', m, n, k)
+    a, b, c = testing.make_float_case(m, n, k, seed=5, device='cuda')
+    assert yan.gemm_float_nt(a, b, c) is None
+    want = oracle.gemm_float_nt_ref(_np(a), _np(b))
+    assert oracle.calc_diff(_np(c), want) < FLOAT_TOL and _float_close(_np(c), want, k)
+    # alpha and beta: c <- alpha * a b^T + beta * c, on top of what the first call left
+    before = _np(c)
+    yan.gemm_float_nt(a, b, c, alpha=-0.5, beta=2.0)
+    want2 = oracle.gemm_float_nt_ref(_np(a), _np(b), before, -0.5, 2.0)
+    assert oracle.calc_diff(_np(c), want2) < FLOAT_TOL and _float_close(_np(c), want2, k)
+    # beta == 0 does not read c: NaNs in it do not propagate
+    c.fill_(float('nan'))
+    yan.gemm_float_nt(a, b, c, alpha=1.0, beta=0.0)
+    assert oracle.calc_diff(_np(c), want) < FLOAT_TOL
+
+
+@pytest.mark.parametrize('m,n,k', testing.REFERENCE_FLOAT_TEST_SHAPES)
+def test_float_entry_on_the_reference_test_shapes(m, n, k):
+    """The flow of the reference's fp32 test (tests/test_simple.py:9-27): randn operands made col-major with
+    `get_col_major_tensor`, zeroed output, `gemm_float_nt`, calc_diff < 1e-3 against `x @ y.t()`; and the bar of this
+    build: 1e-10 against the fp64 product on the device and against the oracle on a seeded sample of rows."""
+    _announce('fp32 reference shape', m, n, k)
+    g = torch.Generator(device='cuda').manual_seed(42 + m + n + k)
+    x = torch.randn(m, k, device='cuda', dtype=torch.float32, generator=g)
+    y = torch.randn(n, k, device='cuda', dtype=torch.float32, generator=g)
+    out = torch.zeros(m, n, device='cuda', dtype=torch.float32)
+    ref_out = x @ y.t()
+    assert yan.gemm_float_nt(yan.get_col_major_tensor(x), yan.get_col_major_tensor(y), out) is None
+    assert float(yan.calc_diff(out, ref_out)) < 1e-3
+    assert float(yan.calc_diff(out.double(), x.double() @ y.double().t())) < FLOAT_TOL
+    rows = np.random.default_rng(m + n + k).choice(m, size=8, replace=False)
+    want = oracle.gemm_float_nt_ref(_np(x[rows]), _np(y))
+    assert oracle.calc_diff(_np(out[rows]), want) < FLOAT_TOL and _float_close(_np(out[rows]), want, k)
+
+
+def test_float_gemm_closed_forms_are_exact_and_kernel_name():
+    # the ones pattern: c = ceil(k / 12) everywhere, exactly; alpha = 0.5, beta = -2 on top of it stays exact
+    m, n, k = 256, 320, 252
+    a, b = torch.zeros(k, m, device='cuda').t(), torch.zeros(k, n, device='cuda').t()
+    a[:, ::4] = 1
+    b[:, ::3] = 1
+    c = torch.zeros(m, n, device='cuda')
+    yan.gemm_float_nt(a, b, c)
+    assert torch.equal(c, torch.full_like(c, 21.0))
+    yan.gemm_float_nt(a, b, c, alpha=0.5, beta=-2.0)
+    assert torch.equal(c, torch.full_like(c, 10.5 - 42.0))
+    # identity on the B side returns A: a transposed operand or a swapped leading dimension cannot pass
+    x, _, _ = testing.make_float_case(128, 64, 64, seed=2, device='cuda')
+    eye = torch.eye(64, device='cuda').t()
+    out = torch.zeros(128, 64, device='cuda')
+    yan.gemm_float_nt(x, eye, out)
+    assert torch.equal(out, x)
+    # k == 0: c <- beta * c
+    out2 = out.clone()
+    yan.gemm_float_nt(torch.zeros(0, 128, device='cuda').t(), torch.zeros(0, 64, device='cuda').t(), out2, alpha=1.0, beta=3.0)
+    assert torch.equal(out2, 3.0 * out)
+    # tests/test_simple.py:35 times the kernel whose name contains 'gemm_cute'
+    big = testing.make_float_case(4096, 4096, 1024, seed=3, device='cuda')
+    t = yan.bench_kineto(lambda: yan.gemm_float_nt(*big), 'gemm_cute', suppress_kineto_output=True)
+    assert 0 < t < 5e-3
+
+
+@pytest.mark.parametrize('m,n,k,lda,ldb,ldc', [(132, 68, 37, 140, 72, 80), (4, 4, 1, 4, 4, 4), (260, 516, 129, 260, 516, 516),
+                                               (128, 64, 16, 128, 64, 64), (1024, 2112, 300, 1032, 2112, 2116)])
+def test_capi_float_matches_raw_buffer_oracle(m, n, k, lda, ldb, ldc):
+    """The C entry on raw buffers with leading dimensions, any m and n that are multiples of 4: against the C triple
+    loop that indexes A[i + t*lda], B[j + t*ldb], C[i*ldc + j]; what lies outside the m x n window is left alone."""
+    from oracle import c_oracle
+    _announce('capi fp32', m, n, k, lda, ldb, ldc)
+    g = torch.Generator().manual_seed(11)
+    a_buf, b_buf = torch.randn(k, lda, generator=g), torch.randn(k, ldb, generator=g)
+    c_buf = torch.randn(m, ldc, generator=g)
+    da, db, dc = a_buf.cuda(), b_buf.cuda(), c_buf.cuda()
+    lib = capi.load()
+    for alpha, beta in ((1.0, 0.0), (0.75, -1.5)):
+        dc.copy_(c_buf)
+        assert lib.yan_gemm_float_nt(m, n, k, alpha, da.data_ptr(), lda, db.data_ptr(), ldb, beta, dc.data_ptr(), ldc, None) == 0
+        got = dc.cpu().numpy().astype(np.float64)
+        want = c_oracle.gemm_float_nt(m, n, k, alpha, a_buf.numpy(), lda, b_buf.numpy(), ldb, beta, c_buf.numpy(), ldc).reshape(m, ldc)
+        assert _float_close(got[:, :n], want[:, :n], k) and oracle.calc_diff(got[:, :n], want[:, :n]) < FLOAT_TOL
+        assert np.array_equal(got[:, n:], c_buf.numpy()[:, n:].astype(np.float64))
+    if m % 128 == 0 and n % 64 == 0 and lda == m and ldb == n and ldc == n:
+        a, b = da.t()[:m], db.t()[:n]
+        via_jit, via_lib = torch.zeros(m, n, device='cuda'), torch.zeros(m, n, device='cuda')
+        yan.gemm_float_nt(a, b, via_jit)
+        assert capi.gemm_float_nt(a, b, via_lib) == 0
+        assert torch.equal(via_jit, via_lib)            # same kernel source, same tile choice: same bits
+
+
 @pytest.mark.parametrize('m,n,k', [s for s in testing.FP8_TEST_SHAPES if s[0] * s[1] * s[2] <= 7e10])
 @pytest.mark.parametrize('col_major', [False, True])
 def test_fp8_parity_vs_oracle(m, n, k, col_major):

@@ -4,7 +4,7 @@ import pytest
 import torch
 
 import yan_amd as yan
-from yan_amd.jit_kernels import heuristics, tuner as tuner_mod, bf16_gemm, gemm
+from yan_amd.jit_kernels import heuristics, tuner as tuner_mod, bf16_gemm, gemm, simple_gemm
 
 
 def test_ceil_div_and_alignment():
@@ -53,6 +53,9 @@ def test_kernel_plans_keep_reference_keys_and_argument_order():
     assert name == 'gemm_fp8_fp8_bf16_nt'
     assert sorted(keys) == ['BLOCK_M', 'BLOCK_N', 'K', 'N', 'NUM_STAGES', 'NUM_TMA_MULTICAST']
     assert [d[0] for d in defs][:9] == ['lhs', 'lhs_scales', 'rhs', 'rhs_scales', 'out', 'm', 'stream', 'num_sms', 'smem_size']
+    name, fkeys, defs = simple_gemm.float_kernel_plan(4096, 7168, 256)
+    assert name == 'gemm_float_nt' and sorted(fkeys) == ['BLOCK_M', 'BLOCK_N']
+    assert [d[0] for d in defs] == ['m', 'n', 'k', 'alpha', 'A', 'ldA', 'B', 'ldB', 'beta', 'C', 'ldC', 'stream']
     assert keys['N'] == 7168 and keys['K'] == 7168 and smem == 2 * (keys['BLOCK_M'] + keys['BLOCK_N']) * 128 <= 160 * 1024
 
 
@@ -67,6 +70,19 @@ def test_entry_points_reject_bad_arguments_before_touching_a_device():
     # empty problems return before any device call
     yan.gemm_bf16_tn(torch.zeros(0, 16, dtype=torch.bfloat16), b, torch.zeros(0, 4, dtype=torch.bfloat16))
     yan.gemm_fp16_tn(torch.zeros(8, 16, dtype=torch.half), torch.zeros(0, 16, dtype=torch.half), torch.zeros(8, 0, dtype=torch.half))
+    # fp32 GEMM (yan/jit_kernels/simple_gemm.py:25-32): m % 128, n % 64, dtypes, shapes; operands M- / N-contiguous
+    x, y = yan.get_col_major_tensor(torch.zeros(128, 16)), yan.get_col_major_tensor(torch.zeros(64, 16))
+    with pytest.raises(AssertionError):
+        yan.gemm_float_nt(x[:100], y, torch.zeros(100, 64))
+    with pytest.raises(AssertionError):
+        yan.gemm_float_nt(x, y[:32], torch.zeros(128, 32))
+    with pytest.raises(AssertionError):
+        yan.gemm_float_nt(x, y, torch.zeros(128, 128))
+    with pytest.raises(AssertionError):
+        yan.gemm_float_nt(x.double(), y, torch.zeros(128, 64))
+    with pytest.raises(AssertionError):     # row-major operands would be read as their transposes
+        yan.gemm_float_nt(torch.zeros(128, 16), y, torch.zeros(128, 64))
+    yan.gemm_float_nt(yan.get_col_major_tensor(torch.zeros(0, 16)), y, torch.zeros(0, 64))
     q = torch.zeros(0, 128, dtype=torch.float8_e4m3fn)
     w = torch.zeros(128, 128, dtype=torch.float8_e4m3fn)
     yan.gemm_fp8_fp8_bf16_nt((q, torch.zeros(0, 1)), (w, torch.ones(1, 1)), torch.zeros(0, 128, dtype=torch.bfloat16))

@@ -165,6 +165,41 @@ def test_bf16_gemm_numpy_vs_c_triple_loop_vs_bruteforce():
     assert np.allclose(oracle.gemm_bf16_tn_ref(2 * a, b, np.float64), 2 * full)
 
 
+# ----------------------------------------------------------------------------- fp32 GEMM with alpha / beta
+def test_float_gemm_closed_forms_and_memory_convention():
+    rng = np.random.default_rng(21)
+    # the ones pattern again: exact small integers, so alpha and beta show up exactly
+    m, n, k = 8, 12, 48
+    a, b = np.zeros((m, k), np.float32), np.zeros((n, k), np.float32)
+    a[:, ::4] = 1
+    b[:, ::3] = 1
+    c = np.arange(m * n, dtype=np.float32).reshape(m, n)
+    assert np.array_equal(oracle.gemm_float_nt_ref(a, b), np.full((m, n), 4.0))
+    assert np.array_equal(oracle.gemm_float_nt_ref(a, b, c, alpha=0.5, beta=-2.0), 2.0 - 2.0 * c)
+    # beta == 0 ignores what c held (NaN included); identity on the B side returns alpha * A
+    a = rng.standard_normal((7, 16)).astype(np.float32)
+    assert np.array_equal(oracle.gemm_float_nt_ref(a, np.eye(16, dtype=np.float32), np.full((7, 16), np.nan), 3.0, 0.0), 3.0 * a.astype(np.float64))
+    # raw-buffer triple loop in the C ABI's convention (A[i + t*lda], B[j + t*ldb], C[i*ldc + j]) against the
+    # logical-array form: a swapped leading dimension or a transposed operand fails this
+    m, n, k, lda, ldb, ldc = 8, 12, 5, 12, 16, 20
+    a_buf = rng.standard_normal((k, lda)).astype(np.float32)
+    b_buf = rng.standard_normal((k, ldb)).astype(np.float32)
+    c_buf = rng.standard_normal((m, ldc)).astype(np.float32)
+    for alpha, beta in ((1.0, 0.0), (0.5, 2.0), (-1.25, 1.0)):
+        got = c_oracle.gemm_float_nt(m, n, k, alpha, a_buf, lda, b_buf, ldb, beta, c_buf, ldc).reshape(m, ldc)
+        want = oracle.gemm_float_nt_ref(a_buf[:, :m].T, b_buf[:, :n].T, c_buf[:, :n], alpha, beta)
+        assert np.allclose(got[:, :n], want, rtol=1e-14, atol=1e-14)
+        assert not got[:, n:].any()                     # outside the m x n window nothing is written
+        brute = np.array([[alpha * sum(float(a_buf[t, i]) * float(b_buf[t, j]) for t in range(k)) + (beta * float(c_buf[i, j]) if beta else 0.0)
+                           for j in range(n)] for i in range(m)])
+        assert np.allclose(want, brute, rtol=1e-13, atol=1e-13)
+    # linearity in alpha and in beta, K-split additivity
+    a, b, c = a_buf[:, :m].T, b_buf[:, :n].T, c_buf[:, :n]
+    full = oracle.gemm_float_nt_ref(a, b, c, 1.0, 1.0)
+    assert np.allclose(full, oracle.gemm_float_nt_ref(a[:, :2], b[:, :2]) + oracle.gemm_float_nt_ref(a[:, 2:], b[:, 2:], c, 1.0, 1.0))
+    assert np.allclose(oracle.gemm_float_nt_ref(a, b, c, 2.0, 3.0), 2.0 * oracle.gemm_float_nt_ref(a, b) + 3.0 * c.astype(np.float64))
+
+
 # ----------------------------------------------------------------------------- FP8 block-scaled GEMM
 def _small_int_codes(rng, shape):
     """e4m3 codes of values in {-4..4}: every product and every 128-term sum is an exact small integer in fp32."""

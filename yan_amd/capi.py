@@ -8,7 +8,7 @@ import torch
 _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), 'csrc', 'libyan_gemm.so')
 _lib = None
 
-SYMBOLS = ('yan_gemm_bf16_tn', 'yan_gemm_fp16_tn', 'yan_gemm_fp8_fp8_bf16_nt', 'yan_m_grouped_gemm_fp8_fp8_bf16_nt_contiguous',
+SYMBOLS = ('yan_gemm_bf16_tn', 'yan_gemm_fp16_tn', 'yan_gemm_float_nt', 'yan_gemm_fp8_fp8_bf16_nt', 'yan_m_grouped_gemm_fp8_fp8_bf16_nt_contiguous',
            'yan_m_grouped_gemm_fp8_fp8_bf16_nt_masked', 'yan_per_token_cast_to_fp8', 'yan_per_block_cast_to_fp8',
            'yan_gemm_select_tile', 'yan_gemm_version')
 
@@ -21,6 +21,7 @@ def load() -> ctypes.CDLL:
         lib = ctypes.CDLL(_LIB_PATH)
         vp, ci, ll = ctypes.c_void_p, ctypes.c_int, ctypes.c_longlong
         lib.yan_gemm_bf16_tn.argtypes = lib.yan_gemm_fp16_tn.argtypes = [ci, ci, ci, vp, vp, vp, vp]
+        lib.yan_gemm_float_nt.argtypes = [ci, ci, ci, ctypes.c_float, vp, ci, vp, ci, ctypes.c_float, vp, ci, vp]
         lib.yan_gemm_fp8_fp8_bf16_nt.argtypes = [vp, vp, ll, ll, vp, vp, vp, ci, ci, ci, vp, ci]
         lib.yan_gemm_select_tile.argtypes = [ci, ci, ci, ci, ci, ctypes.POINTER(ci), ctypes.POINTER(ci)]
         lib.yan_m_grouped_gemm_fp8_fp8_bf16_nt_contiguous.argtypes = [vp, vp, ll, ll, vp, vp, vp, vp, ci, ci, ci, ci, vp, ci]
@@ -46,6 +47,15 @@ def gemm_bf16_tn(a: torch.Tensor, b: torch.Tensor, c: torch.Tensor) -> int:
 def gemm_fp16_tn(a: torch.Tensor, b: torch.Tensor, c: torch.Tensor) -> int:
     (m, k), n = a.shape, b.shape[0]
     return load().yan_gemm_fp16_tn(m, n, k, a.data_ptr(), b.data_ptr(), c.data_ptr(), _stream_handle())
+
+
+def gemm_float_nt(a: torch.Tensor, b: torch.Tensor, c: torch.Tensor, alpha: float = 1.0, beta: float = 0.0) -> int:
+    """`a` [m, k] and `b` [n, k] with their first dimension contiguous, `c` [m, n] row-major."""
+    (m, k), n = a.shape, b.shape[0]
+    lda = a.stride(1) if k > 1 else m
+    ldb = b.stride(1) if k > 1 else n
+    return load().yan_gemm_float_nt(m, n, k, alpha, a.data_ptr(), lda, b.data_ptr(), ldb, beta, c.data_ptr(), c.stride(0),
+                                    _stream_handle())
 
 
 def gemm_fp8_fp8_bf16_nt(lhs, rhs, out: torch.Tensor, num_sms: int = 0) -> int:

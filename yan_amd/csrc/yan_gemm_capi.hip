@@ -6,6 +6,7 @@
 #include "gemm/fp8_gemm.hpp"
 #include "gemm/fp8_gemm_skinny.hpp"
 #include "gemm/fp8_cast.hpp"
+#include "gemm/simple_gemm.hpp"
 
 namespace {
 
@@ -83,6 +84,11 @@ int yan_gemm_bf16_tn(int m, int n, int k, const void* a, const void* b, void* c,
 
 int yan_gemm_fp16_tn(int m, int n, int k, const void* a, const void* b, void* c, void* stream) {
     return dense<yan::MfmaF16_32x32x16, _Float16>(m, n, k, a, b, c, stream);
+}
+
+int yan_gemm_float_nt(int m, int n, int k, float alpha, const float* a, int lda, const float* b, int ldb, float beta,
+                      float* c, int ldc, void* stream) {
+    return int(gemm_nt(m, n, k, alpha, a, lda, b, ldb, beta, c, ldc, static_cast<hipStream_t>(stream), device_cus()));
 }
 
 int yan_gemm_fp8_fp8_bf16_nt(const void* lhs, const float* lhs_scales, long long lhs_scales_stride_m,
@@ -178,10 +184,11 @@ int yan_gemm_select_tile(int op, int m, int n, int k, int num_cus, int* block_m,
         else pick(kFp8Tiles, m, n, num_cus, block_m, block_n);
     }
     else if (op == 2) pick_grouped(m, n, num_cus, 1, 128, k, block_m, block_n);
+    else if (op == 3) { const yan::FloatTile t = yan::pick_float_tile(m, n, num_cus); *block_m = t.block_m; *block_n = t.block_n; }
     else return 1;
     return 0;
 }
 
-const char* yan_gemm_version(void) { return "yan-gemm gfx950 6 dense + 8 fp8 tile variants + 1 weight-streaming fp8 variant + 12 grouped fp8 variants + 4 quantiser kernels"; }
+const char* yan_gemm_version(void) { return "yan-gemm gfx950 6 dense + 4 fp32 + 8 fp8 tile variants + 1 weight-streaming fp8 variant + 12 grouped fp8 variants + 4 quantiser kernels"; }
 
 } // extern "C"

@@ -85,3 +85,19 @@ def get_fp8_tile(m: int, n: int, k: int, num_cus: int) -> Tuple[int, int]:
     """(BLOCK_M, BLOCK_N) of the FP8 kernel that runs: (16 * atoms, 16) for the weight-streaming kernel."""
     atoms = get_skinny_fp8_config(m, n, k, num_cus)
     return (16 * atoms, 16) if atoms else get_best_fp8_config(m, n, k, num_cus)
+
+
+_FLOAT_TILES = ((256, 256), (128, 256), (128, 128), (128, 64))
+
+
+def get_best_float_config(m: int, n: int, num_cus: int) -> Tuple[int, int]:
+    """(BLOCK_M, BLOCK_N) of the fp32 GEMM: the matrix cores run at the same rate for every tile, so the cost is rounds
+    of workgroups over the CUs times the tile's area; ties go to the larger tile, which moves fewer operand bytes per
+    flop. Same rule as `yan::pick_float_tile` in gemm/simple_gemm.hpp."""
+    best, best_cost = None, None
+    for bm, bn in _FLOAT_TILES:
+        tiles = ceil_div(m, bm) * ceil_div(n, bn)
+        cost = ceil_div(tiles, num_cus) * bm * bn
+        if best_cost is None or cost < best_cost:
+            best, best_cost = (bm, bn), cost
+    return best

@@ -66,6 +66,15 @@ def make_bf16_case(m: int, n: int, k: int, seed: int = 42, scale: float = 1.0, d
     return a, b, torch.zeros(m, n, dtype=dtype, device=device)
 
 
+def make_float_case(m: int, n: int, k: int, seed: int = 42, device='cpu', gen_device='cpu'):
+    """A [m,k] and B [n,k] ~ N(0,1) in fp32, stored with their first dimension contiguous (what `gemm_float_nt`
+    takes), plus a zeroed row-major C [m,n]."""
+    gen = torch.Generator(device=gen_device).manual_seed(seed)
+    a = torch.randn(k, m, generator=gen, device=gen_device).to(device).t()
+    b = torch.randn(k, n, generator=gen, device=gen_device).to(device).t()
+    return a, b, torch.zeros(m, n, dtype=torch.float32, device=device)
+
+
 def make_fp8_case(m: int, n: int, k: int, seed: int = 42, dist: str = 'normal', device='cpu', gen_device='cpu',
                   col_major_scales: bool = False):
     """((A8, sA), (B8, sB), out) for the block-scaled GEMM, quantised from seeded fp32 sources.
@@ -142,6 +151,12 @@ DENSE_TEST_SHAPES = [
 # (m, n, k) of the reference's own dense test (tests/test_cute.py:21-22: m in (256, 4096) x six (k, n) pairs)
 REFERENCE_DENSE_TEST_SHAPES = [(m, n, k) for m in (256, 4096)
                                for k, n in ((5120, 5120), (1536, 24576), (512, 32768), (16384, 7168), (7168, 2048), (2048, 7168))]
+# (m, n, k) of the reference's fp32 test (tests/test_simple.py:22-23: m in (128, 4096) x six (k, n) pairs)
+REFERENCE_FLOAT_TEST_SHAPES = [(m, n, k) for m in (128, 4096)
+                               for k, n in ((7168, 2112), (1536, 24576), (512, 32768), (16384, 7168), (7168, 4096), (2048, 7168))]
+# small fp32 cases compared in full: k tails, every tile variant (128x64, 128x128, 128x256, 256x256)
+FLOAT_TEST_SHAPES = [(128, 64, 16), (128, 64, 1), (128, 192, 17), (256, 320, 100), (384, 1024, 260), (128, 24576, 40),
+                     (256, 32768, 24), (4096, 32768, 8)]
 FP8_TEST_SHAPES = [
     (4096, 7168, 7168), (64, 4096, 7168), (16384, 16384, 16384),
     (64, 256, 384), (512, 1024, 1024), (1, 128, 128), (63, 192, 256), (129, 320, 128), (300, 96, 640),
@@ -173,7 +188,7 @@ def jit_kernels_in_use(num_cus: int = 256):
     """(name, arg_defs, code) of every distinct JIT kernel the shapes above, the quantisers and the probe select."""
     from . import probe
     from .jit import cpp_format, generate
-    from .jit_kernels import bf16_gemm, fp8_cast, gemm, m_grouped_gemm
+    from .jit_kernels import bf16_gemm, fp8_cast, gemm, m_grouped_gemm, simple_gemm
     kernels = {}
 
     def add(name, arg_defs, includes, code_template, keys):
@@ -185,6 +200,9 @@ def jit_kernels_in_use(num_cus: int = 256):
             if m and n:
                 name, keys, arg_defs = bf16_gemm.dense_kernel_plan(m, n, k, dtype, num_cus)
                 add(name, arg_defs, bf16_gemm.includes, bf16_gemm.template, keys)
+    for m, n, k in REFERENCE_FLOAT_TEST_SHAPES + FLOAT_TEST_SHAPES + [(5120, 2048, 4096)]:
+        name, keys, arg_defs = simple_gemm.float_kernel_plan(m, n, num_cus)
+        add(name, arg_defs, simple_gemm.includes, simple_gemm.template, keys)
     for m, n, k in FP8_TEST_SHAPES + FP8_SIDE_SHAPES:
         if m:
             name, keys, arg_defs, _, code_template = gemm.fp8_kernel_plan(m, n, k, num_cus)
