@@ -22,6 +22,7 @@ METRIC = 'TFLOPS & % of MFMA peak, fp8 block-scaled GEMM 4096x7168x7168, 1 MI355
 PEAK_FP8_TFLOPS = 5000.0
 PEAK_BF16_TFLOPS = 2500.0
 PEAK_HBM_GBPS = 8000.0
+PEAK_FP32_TFLOPS = 157.3
 
 
 def _event_time_ms(fn, steps, warmup):
@@ -93,7 +94,7 @@ def main():
     ap.add_argument('--gpus', type=int, default=1)
     ap.add_argument('--steps', type=int, default=1000)
     ap.add_argument('--warmup', type=int, default=100)
-    ap.add_argument('--also', action='store_true', help='also time bf16 8192^3, the decode shape and 16384^3 (extra fields)')
+    ap.add_argument('--also', action='store_true', help='also time bf16 8192^3, the decode shape, 16384^3, the grouped GEMMs, the quantisers and the fp32 GEMM (extra fields)')
     ap.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline leg')
     ap.add_argument('--ceilings', action='store_true',
                     help='also measure what the matrix cores sustain with register-resident operands, and what the main loop of the '
@@ -214,6 +215,18 @@ def main():
                            'algorithmic_bytes': byt, 'gb_per_s_cold': round(byt / t_cold / 1e9, 1),
                            'frac_of_hbm_peak_cold': round(byt / t_cold / 1e9 / PEAK_HBM_GBPS, 4)}
         del xs, ws
+        # fp32 GEMM (fp32 MFMA, 157.3 TFLOP/s peak): a large square, the largest shape of the reference's fp32 test and
+        # its m = 128 shape with the fewest outputs, each next to torch.matmul (hipBLASLt) on the same operands
+        for mm, nn, kk in ((8192, 8192, 8192), (4096, 7168, 16384), (128, 2112, 7168)):
+            a, b, c = testing.make_float_case(mm, nn, kk, seed=42, device='cuda', gen_device='cuda')
+            reps = 10 if mm > 128 else 200
+            ms, _ = _event_time_ms(lambda: yan.gemm_float_nt(a, b, c), reps, 3)
+            ms_t, _ = _event_time_ms(lambda: torch.matmul(a, b.t(), out=c), reps, 3)
+            fl = 2.0 * mm * nn * kk
+            extra[f'fp32_{mm}x{nn}x{kk}'] = {'us': round(ms * 1e3, 1), 'tflops': round(fl / ms / 1e9, 1),
+                                             'frac_of_fp32_peak': round(fl / ms / 1e9 / PEAK_FP32_TFLOPS, 4),
+                                             'torch_hipblaslt_us': round(ms_t * 1e3, 1)}
+            del a, b, c
         line['extra'] = extra
 
     if args.ceilings:

@@ -50,7 +50,8 @@ def test_version_and_tile_selection_match_python(lib):
         for cus in (256, 80):
             for groups in (1, 4, 64):
                 assert capi.select_tile(2, m, n, groups, cus) == heuristics.get_best_grouped_fp8_config(m, n, 1024, cus, 1, 128, groups)
-    for m, n in [(128, 2112), (128, 24576), (4096, 7168), (4096, 32768), (128, 64), (5120, 2048), (256, 256)]:
+    for m, n in [(128, 2112), (128, 24576), (128, 32768), (128, 7168), (4096, 7168), (4096, 2112), (4096, 32768), (128, 64), (5120, 2048),
+                 (256, 256), (512, 4096), (1024, 1024), (2048, 2048), (256, 32768)]:
         for cus in (256, 80):
             assert capi.select_tile(3, m, n, 512, cus) == heuristics.get_best_float_config(m, n, cus), (m, n, cus)
     bm, bn = ctypes.c_int(), ctypes.c_int()

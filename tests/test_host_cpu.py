@@ -40,6 +40,11 @@ def test_tile_heuristics_fill_256_cus():
     assert heuristics.get_dense_num_stages(64, 64) == 8 and heuristics.get_dense_num_stages(128, 256) == 3
     # tiny problems get the smallest tile
     assert heuristics.get_best_dense_config(64, 64, 64, 256) == (64, 64)
+    # fp32: full tiles for large problems, K-split tiles (below 128 rows) when a 128-row tiling leaves CUs idle
+    assert heuristics.get_best_float_config(8192, 8192, 256) == (256, 256)
+    assert heuristics.get_best_float_config(4096, 7168, 256) == (128, 128)          # 1792 tiles: exactly 7 rounds
+    assert heuristics.get_best_float_config(128, 2112, 256) == (32, 64)             # 33 tiles of 128 x 64 would use 33 CUs
+    assert heuristics.get_best_float_config(128, 64, 256) == (32, 32)
     ranked = heuristics.rank_tiles(4096, 7168, 256, heuristics._FP8_TILES)
     assert ranked == sorted(ranked) and len(ranked) == len(heuristics._FP8_TILES)
 

@@ -5,7 +5,7 @@
 // contiguous (element (i, kk) at A[i + kk * ldA]), B is n x k with N contiguous (B[j + kk * ldB]), C is m x n
 // row-major (C[i * ldC + j]), work is enqueued on `stream`. The reference kernel (simple_gemm.cuh:16-192) is a
 // 128 x 64 x 16 cp.async pipeline of scalar FMAs; here:
-//   * macro tile BLOCK_M x BLOCK_N x 16, 4 waves in a 2 x 2 arrangement, one per SIMD, each with a
+//   * macro tile BLOCK_M x BLOCK_N, 16 to 128 k-rows per LDS stage, 4 waves in a 2 x 2 arrangement, one per SIMD, each with a
 //     (BLOCK_M / 2) x (BLOCK_N / 2) slab of 32x32x2 fp32 MFMAs (up to 128 x 128: 256 accumulator registers);
 //   * a k-row of a tile is contiguous in memory, so one buffer_load ... lds instruction moves 1 KB of it (or two
 //     k-rows of a 128-wide tile) to where the fragments are read from; a ring of LDS stages keeps
@@ -13,6 +13,10 @@
 //   * a lane reads VM = BLOCK_M / 64 consecutive floats of one k-row as the row operands of VM MFMAs (and VN
 //     floats for the columns), which makes MFMA t of a slab cover the rows VM * i + t: a lane's VN column
 //     accumulators are VN consecutive n of one m, one 16-byte access in C;
+//   * tiles below 128 rows (64 x 64, 32 x 64, 32 x 32) are for problems with too few outputs to give every CU a
+//     large tile: there the four waves split K instead of the tile (each takes a quarter of every 64-deep k-tile
+//     over the whole tile) and their partial sums are added through LDS in a fixed order at the end, so results do
+//     not depend on timing;
 //   * rows past m / n are not written, k rows past the end read as zero: any m, n, k with m, n, ldA, ldB, ldC
 //     multiples of 4 and 16-byte aligned bases.
 // beta == 0 does not read C (the BLAS convention).
@@ -29,7 +33,13 @@ namespace yan {
 
 template <int BLOCK_M, int BLOCK_N>
 struct FloatTileConfig {
-    static constexpr int NUM_WAVES = 4, WAVES_M = 2, WAVES_N = 2, BLOCK_K = 16;
+    static constexpr int NUM_WAVES = 4;
+    static constexpr int K_SPLIT = BLOCK_M < 128 ? 4 : 1;                    // waves that share one tile along K
+    static constexpr int WAVES_M = K_SPLIT == 4 ? 1 : 2, WAVES_N = WAVES_M;
+    // k-rows per LDS stage: deeper for the smaller tiles, so that a stage is 24-32 KB and the barrier between k-tiles
+    // comes once per some thousands of MFMA cycles
+    static constexpr int BLOCK_K = K_SPLIT == 4 ? 64 : (BLOCK_M + BLOCK_N >= 384 ? 16 : 32);
+    static constexpr int KP_PER_WAVE = BLOCK_K / 2 / K_SPLIT;                // k-pairs (one MFMA deep) per wave per k-tile
     static constexpr int WTM = BLOCK_M / WAVES_M, WTN = BLOCK_N / WAVES_N;
     static constexpr int VM = WTM / 32, VN = WTN / 32;                       // floats per lane per operand read
     static_assert((VM == 1 || VM == 2 || VM == 4) && (VN == 1 || VN == 2 || VN == 4), "slabs of 32, 64 or 128 per side");
@@ -38,8 +48,12 @@ struct FloatTileConfig {
     static constexpr int A_COPIES = A_BYTES / 1024, B_COPIES = B_BYTES / 1024;     // wave instructions per stage
     static_assert(A_COPIES % NUM_WAVES == 0 && B_COPIES % NUM_WAVES == 0);
     static constexpr int OPS = (A_COPIES + B_COPIES) / NUM_WAVES;                // per wave per k-tile
-    static constexpr int MAX_STAGES = 128 * 1024 / STAGE_BYTES < 8 ? 128 * 1024 / STAGE_BYTES : 8;
-    static_assert(MAX_STAGES >= 3);
+    static_assert(OPS <= KP_PER_WAVE, "one copy per k-pair");
+    // The two smallest tiles keep their ring within 72 KB so that two workgroups fit a CU and cover each other's
+    // waits (measured: 5-25 % faster than one workgroup with a deeper ring).
+    static constexpr int RING_BUDGET = BLOCK_M == 32 ? 72 * 1024 : 128 * 1024;
+    static constexpr int MAX_STAGES = RING_BUDGET / STAGE_BYTES < 3 ? 3 : (RING_BUDGET / STAGE_BYTES < 8 ? RING_BUDGET / STAGE_BYTES : 8);
+    static_assert(K_SPLIT == 1 || 3 * VM * VN * 16 * 256 <= 3 * STAGE_BYTES, "partial sums of three waves fit the ring");
 };
 
 template <int N> struct FloatVec;
@@ -71,7 +85,7 @@ gemm_cute(const float* __restrict__ A, const float* __restrict__ B, float* __res
 
     const int lane = get_lane_id();
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWaveSize);
-    const int wm = wave / Cfg::WAVES_N, wn = wave % Cfg::WAVES_N;
+    const int wm = Cfg::K_SPLIT == 4 ? 0 : wave / Cfg::WAVES_N, wn = Cfg::K_SPLIT == 4 ? 0 : wave % Cfg::WAVES_N;
 
     // Descriptors end with the last element of the last k-row, so every k-row past k reads as zero.
     const __amdgpu_buffer_rsrc_t rsrc_a = make_rsrc(A, k > 0 ? (uint32_t(k - 1) * uint32_t(ldA) + uint32_t(m)) * 4u : 0u);
@@ -105,8 +119,10 @@ gemm_cute(const float* __restrict__ A, const float* __restrict__ B, float* __res
     // Lane (h, i) = (lane / 32, lane % 32) supplies k-row 2 * kp + h of k-pair kp: VM floats from column VM * i of
     // its slab of the A part, VN floats from column VN * i of its slab of the B part.
     const int h = lane / 32, i = lane % 32;
-    const int frag_a = (h * BLOCK_M + wm * Cfg::WTM + VM * i) * 4;
-    const int frag_b = Cfg::A_BYTES + (h * BLOCK_N + wn * Cfg::WTN + VN * i) * 4;
+    // With K split over the waves, wave w owns k-pairs KP_PER_WAVE * w .. of every k-tile.
+    const int first_kp = Cfg::K_SPLIT == 4 ? wave * Cfg::KP_PER_WAVE : 0;
+    const int frag_a = ((2 * first_kp + h) * BLOCK_M + wm * Cfg::WTM + VM * i) * 4;
+    const int frag_b = Cfg::A_BYTES + ((2 * first_kp + h) * BLOCK_N + wn * Cfg::WTN + VN * i) * 4;
 
     __shared__ __attribute__((aligned(1024))) uint8_t ring[STAGES * Cfg::STAGE_BYTES];
     const int num_k_tiles = ceil_div(k, BLOCK_K);
@@ -131,8 +147,8 @@ gemm_cute(const float* __restrict__ A, const float* __restrict__ B, float* __res
         fa[0] = *reinterpret_cast<const VecM*>(cur + frag_a);
         fb[0] = *reinterpret_cast<const VecN*>(cur + frag_b);
 #pragma unroll
-        for (int kp = 0; kp < BLOCK_K / 2; ++kp) {
-            if (kp + 1 < BLOCK_K / 2) {
+        for (int kp = 0; kp < Cfg::KP_PER_WAVE; ++kp) {
+            if (kp + 1 < Cfg::KP_PER_WAVE) {
                 fa[(kp + 1) & 1] = *reinterpret_cast<const VecM*>(cur + frag_a + (kp + 1) * 2 * BLOCK_M * 4);
                 fb[(kp + 1) & 1] = *reinterpret_cast<const VecN*>(cur + frag_b + (kp + 1) * 2 * BLOCK_N * 4);
             }
@@ -144,8 +160,36 @@ gemm_cute(const float* __restrict__ A, const float* __restrict__ B, float* __res
                 for (int u = 0; u < VN; ++u)
                     acc[t][u] = __builtin_amdgcn_mfma_f32_32x32x2f32(vec_at<VM>(fa[kp & 1], t), vec_at<VN>(fb[kp & 1], u), acc[t][u], 0, 0, 0);
         }
-        static_assert(OPS <= BLOCK_K / 2, "one copy per k-pair");
         st = st + 1 == STAGES ? 0 : st + 1;
+    }
+
+    if constexpr (Cfg::K_SPLIT == 4) {
+        // Partial sums of waves 1..3 go through LDS (register-major, lane-minor: no bank conflicts) and wave 0 adds
+        // them in the order 1, 2, 3. The ring is free once nobody reads it and no copy is still on its way into it.
+        constexpr int REGS = VM * VN * 16;
+        wait_for_copies();
+        __syncthreads();
+        float* partial = reinterpret_cast<float*>(ring);
+        if (wave != 0) {
+#pragma unroll
+            for (int t = 0; t < VM; ++t)
+#pragma unroll
+                for (int u = 0; u < VN; ++u)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r)
+                        partial[((wave - 1) * REGS + (t * VN + u) * 16 + r) * kWaveSize + lane] = acc[t][u][r];
+        }
+        __syncthreads();
+        if (wave != 0) return;
+#pragma unroll
+        for (int w = 0; w < 3; ++w)
+#pragma unroll
+            for (int t = 0; t < VM; ++t)
+#pragma unroll
+                for (int u = 0; u < VN; ++u)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r)
+                        acc[t][u][r] += partial[(w * REGS + (t * VN + u) * 16 + r) * kWaveSize + lane];
     }
 
     // Epilogue: register r of an atom is MFMA row 8 * (r / 4) + 4 * h + r % 4 of MFMA column i; MFMA (t, u) holds
@@ -179,9 +223,9 @@ inline hipError_t check_float_args(int m, int n, int k, const void* a, int ldA, 
     if (ldA < m || ldB < n || ldC < n || (ldA % 4) != 0 || (ldB % 4) != 0 || (ldC % 4) != 0) return hipErrorInvalidValue;
     if (!c || (k > 0 && (!a || !b))) return hipErrorInvalidValue;          // with k == 0 the operands are never read
     if ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b) | reinterpret_cast<uintptr_t>(c)) & 15) return hipErrorInvalidValue;
-    // 32-bit descriptor offsets: the last k-row the ring prefetches (up to 7 k-tiles past the end), tile overhang
+    // 32-bit descriptor offsets: the last k-row the ring prefetches (up to 8 k-tiles of at most 128 rows past the end), tile overhang
     // included, must stay below 2 GiB
-    const uint64_t k_pad = uint64_t(ceil_div(k, 16)) * 16 + 8 * 16;
+    const uint64_t k_pad = uint64_t(k) + 8 * 128;
     if ((k_pad * ldA + block_m) * 4 >= kOutOfRange || (k_pad * ldB + block_n) * 4 >= kOutOfRange) return hipErrorInvalidValue;
     return hipSuccess;
 }
@@ -197,17 +241,19 @@ inline hipError_t launch_float_nt(int m, int n, int k, float alpha, const float*
     return hipGetLastError();
 }
 
-// Tile for a problem when the caller names none: the largest of 256x256, 128x256, 128x128, 128x64 whose count of
-// rounds of workgroups over `num_cus` CUs, times its area, is smallest (the matrix cores run at the same rate for
-// all four; larger tiles move fewer operand bytes per flop).
-struct FloatTile { int block_m, block_n; };
+// Tile for a problem when the caller names none: the one whose count of rounds of workgroups over `num_cus` CUs,
+// times its area, times a measured cost per area, is smallest (the matrix cores run at nearly the same rate for all
+// of them; larger tiles move fewer operand bytes per flop, and the K-split tiles pay for their reduction). Ties go
+// to the earlier, larger tile.
+struct FloatTile { int block_m, block_n; double per_area; };
+constexpr FloatTile kFloatTiles[] = {{256, 256, 1.00}, {128, 256, 1.015}, {128, 128, 1.04}, {128, 64, 1.09},
+                                     {64, 64, 1.13}, {32, 64, 1.13}, {32, 32, 1.25}};
 inline FloatTile pick_float_tile(int m, int n, int num_cus) {
-    constexpr FloatTile kTiles[] = {{256, 256}, {128, 256}, {128, 128}, {128, 64}};
-    FloatTile best = kTiles[0];
-    long long best_cost = -1;
-    for (const FloatTile& t : kTiles) {
+    FloatTile best = kFloatTiles[0];
+    double best_cost = -1;
+    for (const FloatTile& t : kFloatTiles) {
         const long long tiles = static_cast<long long>(ceil_div(m, t.block_m)) * ceil_div(n, t.block_n);
-        const long long cost = ceil_div<long long>(tiles, num_cus) * t.block_m * t.block_n;
+        const double cost = double(ceil_div<long long>(tiles, num_cus)) * t.block_m * t.block_n * t.per_area;
         if (best_cost < 0 || cost < best_cost) { best = t; best_cost = cost; }
     }
     return best;
@@ -232,8 +278,9 @@ inline hipError_t gemm_nt(int m, int n, int k, float alpha, float const* A, int 
             num_cus = 256;
     }
     const yan::FloatTile t = yan::pick_float_tile(m, n, num_cus);
-    if (t.block_m == 256) return gemm_nt<256, 256>(m, n, k, alpha, A, ldA, B, ldB, beta, C, ldC, stream);
-    if (t.block_n == 256) return gemm_nt<128, 256>(m, n, k, alpha, A, ldA, B, ldB, beta, C, ldC, stream);
-    if (t.block_n == 128) return gemm_nt<128, 128>(m, n, k, alpha, A, ldA, B, ldB, beta, C, ldC, stream);
-    return gemm_nt<128, 64>(m, n, k, alpha, A, ldA, B, ldB, beta, C, ldC, stream);
+#define YAN_FLOAT_CASE(BM, BN) if (t.block_m == BM && t.block_n == BN) return gemm_nt<BM, BN>(m, n, k, alpha, A, ldA, B, ldB, beta, C, ldC, stream);
+    YAN_FLOAT_CASE(256, 256) YAN_FLOAT_CASE(128, 256) YAN_FLOAT_CASE(128, 128) YAN_FLOAT_CASE(128, 64)
+    YAN_FLOAT_CASE(64, 64) YAN_FLOAT_CASE(32, 64) YAN_FLOAT_CASE(32, 32)
+#undef YAN_FLOAT_CASE
+    return hipErrorInvalidValue;
 }

@@ -87,17 +87,18 @@ def get_fp8_tile(m: int, n: int, k: int, num_cus: int) -> Tuple[int, int]:
     return (16 * atoms, 16) if atoms else get_best_fp8_config(m, n, k, num_cus)
 
 
-_FLOAT_TILES = ((256, 256), (128, 256), (128, 128), (128, 64))
+# (BLOCK_M, BLOCK_N) -> cost per unit of tile area; tiles below 128 rows split K over their four waves.
+_FLOAT_TILES = {(256, 256): 1.00, (128, 256): 1.015, (128, 128): 1.04, (128, 64): 1.09, (64, 64): 1.13, (32, 64): 1.13, (32, 32): 1.25}
 
 
 def get_best_float_config(m: int, n: int, num_cus: int) -> Tuple[int, int]:
-    """(BLOCK_M, BLOCK_N) of the fp32 GEMM: the matrix cores run at the same rate for every tile, so the cost is rounds
-    of workgroups over the CUs times the tile's area; ties go to the larger tile, which moves fewer operand bytes per
-    flop. Same rule as `yan::pick_float_tile` in gemm/simple_gemm.hpp."""
+    """(BLOCK_M, BLOCK_N) of the fp32 GEMM: rounds of workgroups over the CUs times the tile's area times its cost
+    per area; ties go to the earlier, larger tile. Same table and rule as `yan::pick_float_tile` in
+    gemm/simple_gemm.hpp (a CPU test keeps the two in step)."""
     best, best_cost = None, None
-    for bm, bn in _FLOAT_TILES:
+    for (bm, bn), per_area in _FLOAT_TILES.items():
         tiles = ceil_div(m, bm) * ceil_div(n, bn)
-        cost = ceil_div(tiles, num_cus) * bm * bn
+        cost = ceil_div(tiles, num_cus) * bm * bn * per_area
         if best_cost is None or cost < best_cost:
             best, best_cost = (bm, bn), cost
     return best

@@ -154,9 +154,10 @@ REFERENCE_DENSE_TEST_SHAPES = [(m, n, k) for m in (256, 4096)
 # (m, n, k) of the reference's fp32 test (tests/test_simple.py:22-23: m in (128, 4096) x six (k, n) pairs)
 REFERENCE_FLOAT_TEST_SHAPES = [(m, n, k) for m in (128, 4096)
                                for k, n in ((7168, 2112), (1536, 24576), (512, 32768), (16384, 7168), (7168, 4096), (2048, 7168))]
-# small fp32 cases compared in full: k tails, every tile variant (128x64, 128x128, 128x256, 256x256)
+# small fp32 cases compared in full: k tails, and with the reference's shapes every tile variant (32x32, 32x64 and
+# 64x64 with K split over the waves; 128x64, 128x128, 128x256, 256x256)
 FLOAT_TEST_SHAPES = [(128, 64, 16), (128, 64, 1), (128, 192, 17), (256, 320, 100), (384, 1024, 260), (128, 24576, 40),
-                     (256, 32768, 24), (4096, 32768, 8)]
+                     (512, 4096, 40), (256, 32768, 24), (4096, 32768, 8)]
 FP8_TEST_SHAPES = [
     (4096, 7168, 7168), (64, 4096, 7168), (16384, 16384, 16384),
     (64, 256, 384), (512, 1024, 1024), (1, 128, 128), (63, 192, 256), (129, 320, 128), (300, 96, 640),
