@@ -36,9 +36,8 @@ struct FloatTileConfig {
     static constexpr int NUM_WAVES = 4;
     static constexpr int K_SPLIT = BLOCK_M < 128 ? 4 : 1;                    // waves that share one tile along K
     static constexpr int WAVES_M = K_SPLIT == 4 ? 1 : 2, WAVES_N = WAVES_M;
-    // k-rows per LDS stage: deeper for the smaller tiles, so that a stage is 24-32 KB and the barrier between k-tiles
-    // comes once per some thousands of MFMA cycles
-    static constexpr int BLOCK_K = K_SPLIT == 4 ? 64 : (BLOCK_M + BLOCK_N >= 384 ? 16 : 32);
+    // k-rows per LDS stage: 16 to 32 KB of operands, and a barrier between k-tiles once per 2000-8000 MFMA cycles
+    static constexpr int BLOCK_K = K_SPLIT == 4 ? 64 : (BLOCK_M + BLOCK_N >= 256 ? 16 : 32);
     static constexpr int KP_PER_WAVE = BLOCK_K / 2 / K_SPLIT;                // k-pairs (one MFMA deep) per wave per k-tile
     static constexpr int WTM = BLOCK_M / WAVES_M, WTN = BLOCK_N / WAVES_N;
     static constexpr int VM = WTM / 32, VN = WTN / 32;                       // floats per lane per operand read
@@ -49,9 +48,10 @@ struct FloatTileConfig {
     static_assert(A_COPIES % NUM_WAVES == 0 && B_COPIES % NUM_WAVES == 0);
     static constexpr int OPS = (A_COPIES + B_COPIES) / NUM_WAVES;                // per wave per k-tile
     static_assert(OPS <= KP_PER_WAVE, "one copy per k-pair");
-    // The two smallest tiles keep their ring within 72 KB so that two workgroups fit a CU and cover each other's
-    // waits (measured: 5-25 % faster than one workgroup with a deeper ring).
-    static constexpr int RING_BUDGET = BLOCK_M == 32 ? 72 * 1024 : 128 * 1024;
+    // The 128 x 128 and 128 x 64 tiles and the two smallest ones keep their ring within 72 KB so that two workgroups
+    // fit a CU and cover each other's barriers (measured: 2-10 % and 5-25 % faster than one workgroup with a
+    // deeper ring).
+    static constexpr int RING_BUDGET = (BLOCK_M == 32 || (BLOCK_M == 128 && BLOCK_N <= 128)) ? 72 * 1024 : 128 * 1024;
     static constexpr int MAX_STAGES = RING_BUDGET / STAGE_BYTES < 3 ? 3 : (RING_BUDGET / STAGE_BYTES < 8 ? RING_BUDGET / STAGE_BYTES : 8);
     static_assert(K_SPLIT == 1 || 3 * VM * VN * 16 * 256 <= 3 * STAGE_BYTES, "partial sums of three waves fit the ring");
 };
@@ -246,7 +246,7 @@ inline hipError_t launch_float_nt(int m, int n, int k, float alpha, const float*
 // of them; larger tiles move fewer operand bytes per flop, and the K-split tiles pay for their reduction). Ties go
 // to the earlier, larger tile.
 struct FloatTile { int block_m, block_n; double per_area; };
-constexpr FloatTile kFloatTiles[] = {{256, 256, 1.00}, {128, 256, 1.015}, {128, 128, 1.04}, {128, 64, 1.09},
+constexpr FloatTile kFloatTiles[] = {{256, 256, 1.00}, {128, 256, 1.015}, {128, 128, 1.03}, {128, 64, 1.04},
                                      {64, 64, 1.13}, {32, 64, 1.13}, {32, 32, 1.25}};
 inline FloatTile pick_float_tile(int m, int n, int num_cus) {
     FloatTile best = kFloatTiles[0];

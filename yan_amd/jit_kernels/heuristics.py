@@ -88,7 +88,7 @@ def get_fp8_tile(m: int, n: int, k: int, num_cus: int) -> Tuple[int, int]:
 
 
 # (BLOCK_M, BLOCK_N) -> cost per unit of tile area; tiles below 128 rows split K over their four waves.
-_FLOAT_TILES = {(256, 256): 1.00, (128, 256): 1.015, (128, 128): 1.04, (128, 64): 1.09, (64, 64): 1.13, (32, 64): 1.13, (32, 32): 1.25}
+_FLOAT_TILES = {(256, 256): 1.00, (128, 256): 1.015, (128, 128): 1.03, (128, 64): 1.04, (64, 64): 1.13, (32, 64): 1.13, (32, 32): 1.25}
 
 
 def get_best_float_config(m: int, n: int, num_cus: int) -> Tuple[int, int]:
