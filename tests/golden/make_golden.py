@@ -1,5 +1,6 @@
-"""Writes tests/golden/gemm_small.npz (small seeded inputs and expected outputs for both GEMMs) and
-tests/golden/grouped_cast_small.npz (the grouped FP8 GEMM layouts and the two quantisers).
+"""Writes tests/golden/gemm_small.npz (small seeded inputs and expected outputs for both GEMMs),
+tests/golden/grouped_cast_small.npz (the grouped FP8 GEMM layouts and the two quantisers) and
+tests/golden/float_small.npz (the fp32 GEMM with alpha / beta on raw buffers with leading dimensions).
 
 The reference cannot produce these (no FP8 entry point, CUDA-only kernels, no fixtures of its own), so the
 expected values come from the closed forms in oracle/gemm_oracle.py evaluated in fp64, cross-checked here against
@@ -78,5 +79,30 @@ def main():
     print('wrote', path, os.path.getsize(path), 'bytes')
 
 
+def float_fixture():
+    """fp32 GEMM in the memory convention of the C ABI: A[i + t*lda], B[j + t*ldb], C[i*ldc + j]; 132 x 68 x 37 with
+    padded leading dimensions, and an exact-integer 128 x 64 x 48 case."""
+    rng = np.random.default_rng(20240921)
+    m, n, k, lda, ldb, ldc = 132, 68, 37, 140, 72, 80
+    a_buf = rng.standard_normal((k, lda)).astype(np.float32)
+    b_buf = rng.standard_normal((k, ldb)).astype(np.float32)
+    c_buf = rng.standard_normal((m, ldc)).astype(np.float32)
+    alpha, beta = 0.75, -1.5
+    exp = c_oracle.gemm_float_nt(m, n, k, alpha, a_buf, lda, b_buf, ldb, beta, c_buf, ldc).reshape(m, ldc)
+    want = oracle.gemm_float_nt_ref(a_buf[:, :m].T, b_buf[:, :n].T, c_buf[:, :n], alpha, beta)
+    assert np.allclose(exp[:, :n], want, rtol=1e-14, atol=1e-14)
+    ia = rng.integers(-4, 5, size=(48, 128)).astype(np.float32)        # [k, m]: M contiguous
+    ib = rng.integers(-4, 5, size=(48, 64)).astype(np.float32)
+    ic = rng.integers(-8, 9, size=(128, 64)).astype(np.float32)
+    iexp = oracle.gemm_float_nt_ref(ia.T, ib.T, ic, 0.5, 2.0)
+    assert np.array_equal(iexp, iexp.astype(np.float32).astype(np.float64))       # exactly representable in fp32
+    path = os.path.join(ROOT, 'tests', 'golden', 'float_small.npz')
+    np.savez_compressed(path, dims=np.array([m, n, k, lda, ldb, ldc]), alpha_beta=np.array([alpha, beta]), a_buf=a_buf,
+                        b_buf=b_buf, c_buf=c_buf, expected_f64=exp[:, :n], int_a=ia, int_b=ib, int_c=ic,
+                        int_alpha_beta=np.array([0.5, 2.0]), int_expected=iexp)
+    print('wrote', path, os.path.getsize(path), 'bytes')
+
+
 if __name__ == '__main__':
     main()
+    float_fixture()

@@ -249,6 +249,23 @@ def test_float_gemm_closed_forms_are_exact_and_kernel_name():
     assert 0 < t < 5e-3
 
 
+def test_float_golden_fixture(repo_root):
+    """The committed fp32 fixture: raw buffers with padded leading dimensions through the C entry, and the
+    exact-integer case through the JIT entry, bit for bit."""
+    z = np.load(os.path.join(repo_root, 'tests', 'golden', 'float_small.npz'))
+    m, n, k, lda, ldb, ldc = (int(v) for v in z['dims'])
+    alpha, beta = (float(v) for v in z['alpha_beta'])
+    da, db, dc = (torch.from_numpy(z[name]).cuda() for name in ('a_buf', 'b_buf', 'c_buf'))
+    assert capi.load().yan_gemm_float_nt(m, n, k, alpha, da.data_ptr(), lda, db.data_ptr(), ldb, beta, dc.data_ptr(), ldc, None) == 0
+    got = dc.cpu().numpy().astype(np.float64)
+    assert oracle.calc_diff(got[:, :n], z['expected_f64']) < FLOAT_TOL and _float_close(got[:, :n], z['expected_f64'], k)
+    assert np.array_equal(got[:, n:], z['c_buf'][:, n:].astype(np.float64))
+    a, b, c = torch.from_numpy(z['int_a']).cuda().t(), torch.from_numpy(z['int_b']).cuda().t(), torch.from_numpy(z['int_c']).cuda()
+    ia, ib = (float(v) for v in z['int_alpha_beta'])
+    yan.gemm_float_nt(a, b, c, alpha=ia, beta=ib)
+    assert np.array_equal(c.cpu().numpy().astype(np.float64), z['int_expected'])
+
+
 @pytest.mark.parametrize('m,n,k,lda,ldb,ldc', [(132, 68, 37, 140, 72, 80), (4, 4, 1, 4, 4, 4), (260, 516, 129, 260, 516, 516),
                                                (128, 64, 16, 128, 64, 64), (1024, 2112, 300, 1032, 2112, 2116)])
 def test_capi_float_matches_raw_buffer_oracle(m, n, k, lda, ldb, ldc):

@@ -331,6 +331,19 @@ def test_golden_fixtures_reproduce(repo_root):
     assert np.array_equal(z['int_expected'], oracle.gemm_fp8_block_scaled_ref(z['int_lhs'], z['int_lhs_scales'], z['int_rhs'], z['int_rhs_scales']))
 
 
+def test_float_fixture_reproduces(repo_root):
+    import os
+    z = np.load(os.path.join(repo_root, 'tests', 'golden', 'float_small.npz'))
+    m, n, k, lda, ldb, ldc = (int(v) for v in z['dims'])
+    alpha, beta = (float(v) for v in z['alpha_beta'])
+    got = c_oracle.gemm_float_nt(m, n, k, alpha, z['a_buf'], lda, z['b_buf'], ldb, beta, z['c_buf'], ldc).reshape(m, ldc)
+    assert np.array_equal(got[:, :n], z['expected_f64'])
+    want = oracle.gemm_float_nt_ref(z['a_buf'][:, :m].T, z['b_buf'][:, :n].T, z['c_buf'][:, :n], alpha, beta)
+    assert np.allclose(want, z['expected_f64'], rtol=1e-14, atol=1e-14)
+    ia, ib = (float(v) for v in z['int_alpha_beta'])
+    assert np.array_equal(oracle.gemm_float_nt_ref(z['int_a'].T, z['int_b'].T, z['int_c'], ia, ib), z['int_expected'])
+
+
 def test_grouped_and_cast_fixtures_reproduce(repo_root):
     import os
     z = np.load(os.path.join(repo_root, 'tests', 'golden', 'grouped_cast_small.npz'))
