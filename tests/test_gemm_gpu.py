@@ -719,6 +719,59 @@ def test_capi_fp8_matches_oracle_and_jit(m, n, k):
     assert torch.equal(out, out_cm) and torch.equal(out, out_jit)
 
 
+def test_entry_points_replay_correctly_from_a_captured_graph():
+    """No entry point allocates, synchronises or keeps state, so a chain of them (quantiser -> FP8 GEMM, bf16 GEMM,
+    fp32 GEMM with beta, masked grouped GEMM) can be captured once and replayed; every replay, with new contents in the
+    static input buffers and eager work in between, must give the bits of an eager run on the same inputs."""
+    _announce('graph replay')
+    m, n, k = 256, 512, 512
+    g = torch.Generator(device='cuda').manual_seed(77)
+    x = torch.randn(m, k, device='cuda', generator=g).bfloat16()
+    w = torch.randn(n, k, device='cuda', generator=g).bfloat16()
+    w8, sw = yan.per_block_cast_to_fp8(w)
+    xf_buf, wf_buf = torch.randn(k, m, device='cuda', generator=g), torch.randn(k, n, device='cuda', generator=g)
+    (ga8, gsa), (gb8, gsb), _, masked = testing.make_grouped_masked_case(2, 128, n, k, (128, 40), seed=3, device='cuda')
+    outs = {'fp8': torch.zeros(m, n, dtype=torch.bfloat16, device='cuda'), 'bf16': torch.zeros(m, n, dtype=torch.bfloat16, device='cuda'),
+            'fp32': torch.zeros(m, n, device='cuda'), 'masked': torch.zeros(2, 128, n, dtype=torch.bfloat16, device='cuda')}
+
+    def chain():
+        a8, sa = yan.per_token_cast_to_fp8(x, col_major_scales=True)
+        yan.gemm_fp8_fp8_bf16_nt((a8, sa), (w8, sw), outs['fp8'])
+        yan.gemm_bf16_tn(x, w, outs['bf16'])
+        yan.gemm_float_nt(xf_buf.t(), wf_buf.t(), outs['fp32'], alpha=0.5, beta=0.25)
+        yan.m_grouped_gemm_fp8_fp8_bf16_nt_masked((ga8, gsa), (gb8, gsb), outs['masked'], masked, 128)
+
+    def reset():
+        for name, t in outs.items():
+            t.fill_(1.0 if name == 'fp32' else 0.0)        # the fp32 GEMM reads c (beta != 0)
+
+    reset()
+    chain()                                                # loads every kernel before anything is captured
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        chain()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        chain()
+    for rep in range(3):
+        x.copy_(torch.randn(m, k, device='cuda', generator=g).bfloat16())
+        xf_buf.copy_(torch.randn(k, m, device='cuda', generator=g))
+        reset()
+        graph.replay()
+        torch.cuda.synchronize()
+        replayed = {name: t.clone() for name, t in outs.items()}
+        reset()
+        chain()
+        torch.cuda.synchronize()
+        for name, t in outs.items():
+            assert torch.equal(replayed[name], t), (rep, name)
+        assert float(replayed['fp8'].float().abs().sum()) > 0 and float(replayed['masked'][1, 40:].float().abs().sum()) == 0
+
+
 def test_capi_rejects_bad_sizes_on_device():
     from yan_amd import capi
     a = torch.zeros(64, 64, dtype=torch.bfloat16, device='cuda')

@@ -169,7 +169,7 @@ FP8_TEST_SHAPES = [
 # Plain FP8 calls the grouped and quantiser tests make on the side (first group through the plain entry, quantise-then-
 # multiply): listed so that their kernels are compiled ahead of time as well.
 FP8_SIDE_SHAPES = [(1024, 4096, 7168), (8192, 4096, 7168), (200, 384, 512), (1152, 512, 512), (128, 4096, 1024), (128, 320, 384),
-                   (256, 200, 128)]
+                   (256, 200, 128), (256, 512, 512)]
 # Grouped FP8 GEMMs: (rows per group, n, k, blocks of padding rows) and (groups, m_max, n, k, masked_m, expected_m).
 GROUPED_CONTIGUOUS_TEST_CASES = [
     ((100, 128, 1, 300), 320, 384, 1), ((128, 128), 4096, 1024, 0), ((129,), 200, 128, 2),
@@ -182,6 +182,7 @@ GROUPED_MASKED_TEST_CASES = [
     (3, 200, 320, 384, (200, 0, 77), 128), (4, 256, 4096, 1024, (1, 256, 130, 64), 64), (2, 64, 200, 128, (64, 3), 32),
     (4, 1024, 4096, 7168, (1024, 900, 512, 1), 1024),
     (2, 40, 192, 256, (40, 7), 40),                  # the committed fixture
+    (2, 128, 512, 512, (128, 40), 128),              # the group of the graph-replay test
 ]
 
 
@@ -196,7 +197,7 @@ def jit_kernels_in_use(num_cus: int = 256):
         code = generate(includes, arg_defs, cpp_format(code_template, keys))
         kernels.setdefault((name, code), (name, arg_defs, code))
 
-    for m, n, k in DENSE_TEST_SHAPES + REFERENCE_DENSE_TEST_SHAPES:
+    for m, n, k in DENSE_TEST_SHAPES + REFERENCE_DENSE_TEST_SHAPES + [(256, 512, 512)]:
         for dtype in (torch.bfloat16, torch.half):
             if m and n:
                 name, keys, arg_defs = bf16_gemm.dense_kernel_plan(m, n, k, dtype, num_cus)
