@@ -38,6 +38,26 @@ struct MfmaF16_32x32x16 {
     }
 };
 
+// 16x16x32, bf16 / f16 in, fp32 accumulate: 4 passes, 4 accumulator registers per lane; a lane holds 8 consecutive
+// K values (16 bytes) of row l % 16, K group l / 16.
+struct MfmaBF16_16x16x32 {
+    static constexpr int R = 16, K_BYTES = 64, ACC = 4;
+    using Frag = bf16x8;
+    using Acc  = f32x4;
+    __device__ __forceinline__ static Acc mma(Frag rows, Frag cols, Acc c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(rows, cols, c, 0, 0, 0);
+    }
+};
+
+struct MfmaF16_16x16x32 {
+    static constexpr int R = 16, K_BYTES = 64, ACC = 4;
+    using Frag = f16x8;
+    using Acc  = f32x4;
+    __device__ __forceinline__ static Acc mma(Frag rows, Frag cols, Acc c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(rows, cols, c, 0, 0, 0);
+    }
+};
+
 // 16x16x128 over OCP e4m3 bytes (cbsz = blgp = 0 selects e4m3 for both operands; zero scale operands select
 // the unscaled instruction): 8 passes, a whole 128-deep scale block per instruction, 4 accumulator registers.
 struct MfmaFP8_16x16x128 {
