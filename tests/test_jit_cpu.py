@@ -96,6 +96,29 @@ def test_build_layout_cache_and_export(cache_dir):
         assert 'gfx950' in objs.stdout
 
 
+def test_concurrent_builds_of_one_kernel_leave_one_valid_entry(cache_dir):
+    """Several processes that miss the cache at the same moment each compile into a temporary of their own and rename
+    it into place (yan/jit/compiler.py:131-151, 228-250 does the same): all succeed, one directory remains, and it
+    loads."""
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    prog = ("import sys, torch; sys.path.insert(0, %r); from yan_amd import jit; "
+            "args = (('x', torch.float), ('n', int)); "
+            "rt = jit.build('racer', args, jit.generate((), args, '\\n__return_code = n + 1;\\n')); print(rt.path)") % root
+    env = dict(os.environ, YAN_CACHE_DIR=str(cache_dir))
+    procs = [subprocess.Popen([sys.executable, '-c', prog], env=env, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True)
+             for _ in range(3)]
+    outs = [p.communicate(timeout=300) for p in procs]
+    assert all(p.returncode == 0 for p in procs), [e[-500:] for _, e in outs]
+    paths = {o.strip().splitlines()[-1] for o, _ in outs}
+    assert len(paths) == 1
+    path = paths.pop()
+    assert os.listdir(cache_dir / 'cache') == [os.path.basename(path)]
+    assert sorted(os.listdir(path)) == ['kernel.args', 'kernel.cu', 'kernel.so']
+    assert os.listdir(cache_dir / 'tmp') == []
+    assert hasattr(ctypes.CDLL(os.path.join(path, 'kernel.so')), 'launch')
+
+
 def test_runtime_call_marshals_and_checks_arguments(cache_dir):
     # a host-only body: the launch wrapper itself needs no device
     args = (('n', int), ('x', float), ('flag', bool), ('data', torch.int))
