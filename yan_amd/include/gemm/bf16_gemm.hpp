@@ -196,7 +196,11 @@ dense_gemm_body(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, El
 
 // The same contraction with 8 waves (two per SIMD) and 16x16x32 atoms: each wave owns a (BLOCK_N/2) x (BLOCK_M/4) slab,
 // 128 accumulator registers for the 256 x 256 tile. Two LDS stages; while one wave of a SIMD waits at the barrier or
-// issues its copies, the other keeps the matrix core busy.
+// issues its copies, the other keeps the matrix core busy. The kernel is persistent: a workgroup walks the tiles
+// blockIdx.x, blockIdx.x + gridDim.x, ... (the launcher starts one workgroup per CU), starts the copies of the next
+// tile's first k-tile during the last k-tile of the current one, and its output stores drain while the next tile is
+// already computing. With one workgroup per tile the drain and the first loads of every tile were exposed: 11 % of the
+// time at 8192^3.
 template <typename Atom, typename Elem, int BLOCK_M, int BLOCK_N>
 __device__ __forceinline__ void
 dense_gemm_body_8w(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, Elem* __restrict__ C, int m, int n, int k) {
@@ -204,11 +208,14 @@ dense_gemm_body_8w(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
     constexpr int TN = WTN / 16, TM = WTM / 16, STEPS = 2 * TN;
     static_assert(WTN % 16 == 0 && WTM % 16 == 0 && TN * TM * 4 <= 128);
     using Frag = typename Atom::Frag;
+    using StA = TileStager<BLOCK_M, NW>;
+    using StB = TileStager<BLOCK_N, NW>;
+    static_assert(StA::PADDED_ROWS == BLOCK_M && StB::PADDED_ROWS == BLOCK_N, "tiles are whole copy passes");
+    constexpr int NUM_COPIES = StA::PASSES + StB::PASSES;
+    static_assert(NUM_COPIES <= STEPS);
 
     const XcdTileScheduler<> sched(m, n, BLOCK_M, BLOCK_N);
-    const TileCoord tile = sched.tile_of(blockIdx.x);
-    if (!tile.valid) return;
-    const int m0 = tile.m_idx * BLOCK_M, n0 = tile.n_idx * BLOCK_N;
+    const int num_slots = sched.grid_size();
     const int lane = get_lane_id();
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWaveSize);
     const int wn = wave % WAVES_N, wm = wave / WAVES_N;
@@ -217,44 +224,73 @@ dense_gemm_body_8w(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
     const uint32_t ld_bytes = uint32_t(k) * 2;
     const __amdgpu_buffer_rsrc_t rsrc_a = make_rsrc(A, uint32_t(m) * ld_bytes);
     const __amdgpu_buffer_rsrc_t rsrc_b = make_rsrc(B, uint32_t(n) * ld_bytes);
-    using StA = TileStager<BLOCK_M, NW>;
-    using StB = TileStager<BLOCK_N, NW>;
-    static_assert(StA::PADDED_ROWS == BLOCK_M && StB::PADDED_ROWS == BLOCK_N, "tiles are whole copy passes");
-    StA stage_a;
-    StB stage_b;
-    stage_a.init(m0, ld_bytes, wave, lane);
-    stage_b.init(n0, ld_bytes, wave, lane);
     const int k_bytes = k * 2;
     const int num_k_tiles = ceil_div(k_bytes, kRowBytes);
     const int tail_tile = (k_bytes % kRowBytes) ? num_k_tiles - 1 : -1;
-    const uint32_t tail_a = stage_a.tail_voff(k_bytes % kRowBytes), tail_b = stage_b.tail_voff(k_bytes % kRowBytes);
-    constexpr int NUM_COPIES = StA::PASSES + StB::PASSES;
-    auto copy_pass = [&](int d, int kt, uint8_t* la, uint8_t* lb) {
-        const bool tail = kt == tail_tile;
-        if (d < StA::PASSES) stage_a.issue_pass_from(rsrc_a, la, kt * kRowBytes, wave, d, tail ? tail_a : stage_a.voff);
-        else stage_b.issue_pass_from(rsrc_b, lb, kt * kRowBytes, wave, d - StA::PASSES, tail ? tail_b : stage_b.voff);
+    // An output larger than the L2s together (8 x 4 MB) is stored with the non-temporal hint: kept in L2 it pushes
+    // out the operand panels the other workgroups of the XCD are about to read (8192^3: 805 -> 754 us).
+    const bool stream_out = size_t(m) * n * sizeof(Elem) > (size_t(32) << 20);
+
+    // What a wave needs to know of a tile to copy its k-tiles.
+    struct TileIo {
+        StA a;
+        StB b;
+        uint32_t tail_a, tail_b;
+        int m0, n0;
+        bool valid;
+    };
+    auto open_tile = [&](int slot) {
+        TileIo t;
+        const TileCoord coord = slot < num_slots ? sched.tile_of(slot) : TileCoord{0, 0, false};
+        t.valid = coord.valid;
+        t.m0 = coord.m_idx * BLOCK_M;
+        t.n0 = coord.n_idx * BLOCK_N;
+        t.a.init(t.m0, ld_bytes, wave, lane);
+        t.b.init(t.n0, ld_bytes, wave, lane);
+        t.tail_a = t.a.tail_voff(k_bytes % kRowBytes);
+        t.tail_b = t.b.tail_voff(k_bytes % kRowBytes);
+        return t;
+    };
+    // Every tile runs an even number of k-tiles, so that it starts in stage 0 and the stage of every k-step is known
+    // at compile time (the compiler then sees that the copies into one stage cannot touch the fragments it reads from
+    // the other, and does not wait for them): an odd count gets one more k-tile whose copies are sent out of range
+    // and move zeros.
+    const int k_tiles_run = (num_k_tiles + 1) & ~1;
+    auto copy_pass = [&](const TileIo& t, int d, int kt, uint8_t* la, uint8_t* lb) {
+        const bool tail = kt == tail_tile, past = kt >= num_k_tiles;
+        if (d < StA::PASSES) t.a.issue_pass_from(rsrc_a, la, kt * kRowBytes, wave, d, past ? kOutOfRange : (tail ? t.tail_a : t.a.voff));
+        else t.b.issue_pass_from(rsrc_b, lb, kt * kRowBytes, wave, d - StA::PASSES, past ? kOutOfRange : (tail ? t.tail_b : t.b.voff));
     };
 
     // The two 32-deep halves of a 64-deep k-tile: chunk 4 * half + g of the lane's row.
     const int koff[2] = {frag_offset<16>(lane, g), frag_offset<16>(lane, 4 + g)};
 
-    f32x4 acc[TN][TM];
-#pragma unroll
-    for (int i = 0; i < TN; ++i)
-#pragma unroll
-        for (int j = 0; j < TM; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+    // One array for both stages: with a separate array per stage the compiler knows which copies feed which fragment
+    // reads and guards the reads with a wait for every outstanding vector-memory operation, the output stores of the
+    // previous tile included; the waits below are exact instead.
+    constexpr int A_BYTES = BLOCK_M * kRowBytes, STAGE_BYTES = (BLOCK_M + BLOCK_N) * kRowBytes;
+    __shared__ __attribute__((aligned(1024))) uint8_t stages[2 * STAGE_BYTES];
+    uint8_t* const lds_a0 = stages;
+    uint8_t* const lds_b0 = stages + A_BYTES;
+    uint8_t* const lds_a1 = stages + STAGE_BYTES;
+    uint8_t* const lds_b1 = stages + STAGE_BYTES + A_BYTES;
 
-    __shared__ __attribute__((aligned(1024))) uint8_t lds_a0[BLOCK_M * kRowBytes];
-    __shared__ __attribute__((aligned(1024))) uint8_t lds_b0[BLOCK_N * kRowBytes];
-    __shared__ __attribute__((aligned(1024))) uint8_t lds_a1[BLOCK_M * kRowBytes];
-    __shared__ __attribute__((aligned(1024))) uint8_t lds_b1[BLOCK_N * kRowBytes];
+    f32x4 acc[TN][TM];
 
     // One k-tile: STEPS = 2 * TN steps of TM MFMAs (one row of atoms, one half of K); the fragments of the next step are
-    // fetched before the MFMAs of this one issue (fetching two steps ahead measured no faster), the copies of the next
-    // k-tile go out one per step from the start.
-    auto k_step = [&](int kt, const uint8_t* a_cur, const uint8_t* b_cur, uint8_t* a_nxt, uint8_t* b_nxt) {
-        wait_for_copies();
-        __syncthreads();
+    // fetched before the MFMAs of this one issue (fetching two steps ahead measured no faster); `copy(s)` runs once per
+    // step from the start of the tile and is where the copies of whatever comes next are started, one per step.
+    // `stores_behind`: the last STORES_PER_TILE vector-memory operations of this wave are the previous tile's output
+    // stores, issued after the copies this k-tile needs; the in-order counter then only has to drop to that many,
+    // and the stores drain while the new tile computes.
+    constexpr int STORES_PER_TILE = TM * 4;
+    auto k_step = [&](const uint8_t* a_cur, const uint8_t* b_cur, bool stores_behind, auto&& copy) {
+        if (stores_behind) __builtin_amdgcn_s_waitcnt(waitcnt_imm(STORES_PER_TILE, kNoWaitLgkm));
+        else wait_for_copies();
+        // a bare barrier: __syncthreads() carries a fence that would wait for the stores after all
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
         const uint8_t* pa = a_cur + wm * WTM * kRowBytes;
         const uint8_t* pb = b_cur + wn * WTN * kRowBytes;
         Frag nf[2], mf[2][TM];
@@ -269,37 +305,91 @@ dense_gemm_body_8w(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
 #pragma unroll
         for (int s = 0; s < STEPS; ++s) {
             const int half = s / TN, i = s % TN;
-            if (s < NUM_COPIES) copy_pass(s, kt + 1, a_nxt, b_nxt);
+            if (s < NUM_COPIES) copy(s);
             if (s + 1 < STEPS) fetch_n(s + 1);
             if (s + 1 == TN) fetch_m(1);
 #pragma unroll
             for (int j = 0; j < TM; ++j) acc[i][j] = Atom::mma(nf[s & 1], mf[half][j], acc[i][j]);
             __builtin_amdgcn_sched_barrier(0);        // without it the compiler hoists the reads and copies of the whole k-tile
         }
-        static_assert(NUM_COPIES <= STEPS);
     };
 
+    int slot = blockIdx.x;
+    TileIo cur = open_tile(slot);
+    if (!cur.valid) return;
 #pragma unroll
-    for (int d = 0; d < NUM_COPIES; ++d) copy_pass(d, 0, lds_a0, lds_b0);
-    int kt = 0;
-    for (; kt + 1 < num_k_tiles; kt += 2) {
-        k_step(kt, lds_a0, lds_b0, lds_a1, lds_b1);
-        k_step(kt + 1, lds_a1, lds_b1, lds_a0, lds_b0);
-    }
-    if (kt < num_k_tiles) k_step(kt, lds_a0, lds_b0, lds_a1, lds_b1);
-
-    // Epilogue: the 4 registers of atom (i, j) are n = n_slab + 16 i + 4 g + {0..3} of row m = m_slab + 16 j + col.
-    const int m_slab = m0 + wm * WTM, n_slab = n0 + wn * WTN;
+    for (int d = 0; d < NUM_COPIES; ++d) copy_pass(cur, d, 0, lds_a0, lds_b0);
+    bool stores_behind = false;
+    while (true) {
+        slot += gridDim.x;
+        const TileIo nxt = open_tile(slot);
 #pragma unroll
-    for (int j = 0; j < TM; ++j) {
-        const int mm = m_slab + j * 16 + col;
-        if (mm >= m) continue;
-        Elem* row = C + size_t(mm) * n;
+        for (int i = 0; i < TN; ++i)
 #pragma unroll
-        for (int i = 0; i < TN; ++i) {
-            const int nn = n_slab + i * 16 + 4 * g;
-            if (nn < n) *reinterpret_cast<decltype(pack4(acc[i][j], Elem{}))*>(row + nn) = pack4(acc[i][j], Elem{});
+            for (int j = 0; j < TM; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+        int kt = 0;
+        for (; kt + 2 < k_tiles_run; kt += 2) {
+            k_step(lds_a0, lds_b0, stores_behind, [&](int s) { copy_pass(cur, s, kt + 1, lds_a1, lds_b1); });
+            stores_behind = false;
+            k_step(lds_a1, lds_b1, false, [&](int s) { copy_pass(cur, s, kt + 2, lds_a0, lds_b0); });
         }
+        k_step(lds_a0, lds_b0, stores_behind, [&](int s) { copy_pass(cur, s, kt + 1, lds_a1, lds_b1); });
+        stores_behind = false;
+        // last k-tile of this tile: the copies are the first k-tile of the next tile, if there is one
+        k_step(lds_a1, lds_b1, false, [&](int s) { if (nxt.valid) copy_pass(nxt, s, 0, lds_a0, lds_b0); });
+        uint8_t* const a_last = lds_a1;
+        uint8_t* const b_last = lds_b1;
+
+        // Epilogue: the 4 registers of atom (i, j) are n = n_slab + 16 i + 4 g + {0..3} of row m = m_slab + 16 j + col.
+        // Stored straight from there a wave instruction would write 16 rows x 32 bytes; instead each wave turns its slab
+        // round through the stage that was consumed last, 16 rows at a time, and stores 4 rows x 256 consecutive bytes
+        // per instruction (16 bytes per lane). Rows are 288 bytes apart in LDS so that the 8-byte writes of 16 rows
+        // spread over the banks. The other stage is receiving the next tile meanwhile.
+        const int m_slab = cur.m0 + wm * WTM, n_slab = cur.n0 + wn * WTN;
+        static_assert(WTM == 64 && WTN == 128 && sizeof(Elem) == 2, "the staged epilogue is laid out for 128 x 64 slabs");
+        if ((n % 8) == 0) {
+            constexpr int PITCH = 288;
+            // every wave has read the last k-tile (a bare barrier: nothing here depends on the copies under way)
+            __builtin_amdgcn_s_waitcnt(waitcnt_imm(kNoWaitVm, 0));
+            asm volatile("" ::: "memory");
+            __builtin_amdgcn_s_barrier();
+            asm volatile("" ::: "memory");
+            uint8_t* region = (wave < 4 ? a_last : b_last) + (wave % 4) * (16 * PITCH);
+            const int r4 = lane / 16, c = lane % 16;
+            const int nn = n_slab + 8 * c;
+#pragma unroll
+            for (int j = 0; j < TM; ++j) {
+#pragma unroll
+                for (int i = 0; i < TN; ++i)
+                    *reinterpret_cast<decltype(pack4(acc[0][0], Elem{}))*>(region + col * PITCH + (16 * i + 4 * g) * 2) = pack4(acc[i][j], Elem{});
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const int row = 4 * q + r4, mm = m_slab + 16 * j + row;
+                    const i32x4 v = *reinterpret_cast<const i32x4*>(region + row * PITCH + c * 16);
+                    if (mm < m && nn < n) {
+                        i32x4* dst = reinterpret_cast<i32x4*>(C + size_t(mm) * n + nn);
+                        if (stream_out) __builtin_nontemporal_store(v, dst);
+                        else *dst = v;
+                    }
+                }
+            }
+            // an interior tile: every lane of every wave has just issued exactly STORES_PER_TILE stores
+            stores_behind = cur.m0 + BLOCK_M <= m && cur.n0 + BLOCK_N <= n;
+        } else {
+#pragma unroll
+            for (int j = 0; j < TM; ++j) {
+                const int mm = m_slab + j * 16 + col;
+                if (mm >= m) continue;
+                Elem* row = C + size_t(mm) * n;
+#pragma unroll
+                for (int i = 0; i < TN; ++i) {
+                    const int nn = n_slab + i * 16 + 4 * g;
+                    if (nn < n) *reinterpret_cast<decltype(pack4(acc[i][j], Elem{}))*>(row + nn) = pack4(acc[i][j], Elem{});
+                }
+            }
+        }
+        if (!nxt.valid) break;
+        cur = nxt;
     }
 }
 
@@ -349,11 +439,14 @@ inline hipError_t launch_dense(int m, int n, int k, const void* a, const void* b
     if constexpr (BLOCK_M == 256 && BLOCK_N == 256 && STAGES == 2) {
         // The largest tile runs the 8-wave kernel on 16x16x32 atoms: level with the 4-wave one where the chip's power
         // limit sets the pace (8192^3), 13 % faster at 4096^3.
+        // persistent: one workgroup per CU (a multiple of the 8 XCDs, so a workgroup's tiles stay on one XCD's range)
+        const int cus = device_cu_count() / kNumXCD * kNumXCD;
+        const int grid = sched.grid_size() < cus ? sched.grid_size() : cus;
         if constexpr (__is_same(Elem, _Float16))
-            hipLaunchKernelGGL((fp16_gemm_cute_8w<BLOCK_M, BLOCK_N>), dim3(sched.grid_size()), dim3(8 * kWaveSize), 0, stream,
+            hipLaunchKernelGGL((fp16_gemm_cute_8w<BLOCK_M, BLOCK_N>), dim3(grid), dim3(8 * kWaveSize), 0, stream,
                                static_cast<const uint8_t*>(a), static_cast<const uint8_t*>(b), static_cast<Elem*>(c), m, n, k);
         else
-            hipLaunchKernelGGL((dense_gemm_mfma_8w<MfmaBF16_16x16x32, Elem, BLOCK_M, BLOCK_N>), dim3(sched.grid_size()),
+            hipLaunchKernelGGL((dense_gemm_mfma_8w<MfmaBF16_16x16x32, Elem, BLOCK_M, BLOCK_N>), dim3(grid),
                                dim3(8 * kWaveSize), 0, stream, static_cast<const uint8_t*>(a), static_cast<const uint8_t*>(b),
                                static_cast<Elem*>(c), m, n, k);
     } else if constexpr (__is_same(Elem, _Float16))

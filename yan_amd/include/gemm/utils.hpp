@@ -37,4 +37,16 @@ __host__ __device__ constexpr int waitcnt_imm(int vmcnt, int lgkmcnt) {
 constexpr int kNoWaitVm   = 63;
 constexpr int kNoWaitLgkm = 15;
 
+// Compute units of the current device (256 on MI355X), asked once per process; 256 if the runtime will not say.
+inline int device_cu_count() {
+    static const int cus = [] {
+        int device = 0, count = 0;
+        if (hipGetDevice(&device) != hipSuccess ||
+            hipDeviceGetAttribute(&count, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || count < kNumXCD)
+            count = 256;
+        return count;
+    }();
+    return cus;
+}
+
 } // namespace yan
