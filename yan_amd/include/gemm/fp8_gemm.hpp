@@ -249,6 +249,10 @@ fp8_gemm_kernel(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_s
             }
         });
     };
+    // The staged epilogue (below) turns the slab round through the LDS stage that was consumed last.
+    constexpr bool kStagedEpilogue = STAGES == 2 && NW == 8 && Cfg::WTN == 128 && Cfg::WTM == 64;
+    [[maybe_unused]] uint8_t* epi_a = nullptr;
+    [[maybe_unused]] uint8_t* epi_b = nullptr;
     for (int pass = 0; pass < (kGemmType == GemmType::GroupedContiguous ? num_passes : 1); ++pass) {
     if constexpr (kGemmType == GemmType::GroupedContiguous) {
         rhs        = rhs_all + size_t(pass_group[pass]) * N * K;
@@ -273,6 +277,8 @@ fp8_gemm_kernel(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_s
         k_step(kb + 1, lds_a1, lds_b1, lds_a0, lds_b0);
     }
     if (NUM_K_BLOCKS % 2 == 1) k_step(NUM_K_BLOCKS - 1, lds_a0, lds_b0, lds_a1, lds_b1);
+    epi_a = (NUM_K_BLOCKS % 2 == 1) ? lds_a0 : lds_a1;
+    epi_b = (NUM_K_BLOCKS % 2 == 1) ? lds_b0 : lds_b1;
     } else {
     // Ring of STAGES stages, STAGES - 1 k-tiles in flight: what a small tile needs when the problem is bound by
     // streaming its operands and one k-tile of prefetch cannot cover the memory latency. Every wave issues the same
@@ -324,16 +330,57 @@ fp8_gemm_kernel(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_s
     }
 
     // Epilogue: the 4 registers of atom (i, j) are n = n_slab + 16i + 4g + {0..3} of row m = m_slab + 16j + col.
+    // Stored straight from there a wave instruction writes 16 rows x 32 bytes. The 256 x 256 tile instead turns each
+    // wave's slab round through the LDS stage that was consumed last, 16 rows at a time (rows 288 bytes apart, so that
+    // the 8-byte writes of 16 rows spread over the banks), and stores 4 rows x 256 consecutive bytes per instruction.
+    // An output larger than the L2s together (8 x 4 MB) is stored with the non-temporal hint: kept in L2 it pushes out
+    // the operand panels the other workgroups of the XCD are about to read.
+    bool staged = false;
+    if constexpr (kStagedEpilogue) staged = (N % 8) == 0;
+    if (staged) {
+        if constexpr (kStagedEpilogue) {
+            constexpr int PITCH = 288;
+            const bool stream_out = size_t(m) * N * 2 > (size_t(32) << 20);
+            __syncthreads();                                   // every wave has read the last k-tile
+            // Everything the epilogue derives from the lane number is derived here, behind an opaque copy of it: the
+            // main loop has no registers to spare for addresses computed ahead of time.
+            int lane_late = lane;
+            asm volatile("" : "+v"(lane_late));
+            uint8_t* region = (wave < 4 ? epi_a : epi_b) + (wave % 4) * (16 * PITCH);
+            const int r4 = lane_late / 16, c = lane_late % 16;
+            const int nn = n_slab + 8 * c;
 #pragma unroll
-    for (int j = 0; j < TM; ++j) {
-        const int mm = m_slab + j * 16 + col;
-        if (mm >= m) continue;
-        if constexpr (kTwoHalves) { if (mm < pass_lo[pass] || mm >= pass_hi[pass]) continue; }
-        __bf16* row = out + size_t(mm) * N;
+            for (int j = 0; j < TM; ++j) {
 #pragma unroll
-        for (int i = 0; i < TN; ++i) {
-            const int nn = n_slab + i * 16 + 4 * g;
-            if (nn < N) *reinterpret_cast<bf16x4*>(row + nn) = pack4(acc[i][j], __bf16{});
+                for (int i = 0; i < TN; ++i)
+                    *reinterpret_cast<bf16x4*>(region + c * PITCH + (16 * i + 4 * r4) * 2) = pack4(acc[i][j], __bf16{});
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const int row = 4 * q + r4, mm = m_slab + 16 * j + row;
+                    const i32x4 v = *reinterpret_cast<const i32x4*>(region + row * PITCH + c * 16);
+                    bool live = mm < m && nn < N;
+                    if constexpr (kTwoHalves) live = live && mm >= pass_lo[pass] && mm < pass_hi[pass];
+                    if (live) {
+                        i32x4* dst = reinterpret_cast<i32x4*>(out + size_t(mm) * N + nn);
+                        if (stream_out) __builtin_nontemporal_store(v, dst);
+                        else *dst = v;
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);      // one 16-row pass at a time: the registers are full of sums
+            }
+        }
+    } else {
+#pragma unroll
+        for (int j = 0; j < TM; ++j) {
+            const int mm = m_slab + j * 16 + col;
+            if (mm >= m) continue;
+            if constexpr (kTwoHalves) { if (mm < pass_lo[pass] || mm >= pass_hi[pass]) continue; }
+            __bf16* row = out + size_t(mm) * N;
+#pragma unroll
+            for (int i = 0; i < TN; ++i) {
+                const int nn = n_slab + i * 16 + 4 * g;
+                if (nn < N) *reinterpret_cast<bf16x4*>(row + nn) = pack4(acc[i][j], __bf16{});
+            }
         }
     }
     }   // pass
