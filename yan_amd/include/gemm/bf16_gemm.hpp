@@ -173,14 +173,17 @@ dense_gemm_body(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, El
         st = st + 1 == STAGES ? 0 : st + 1;
     }
 
-    // Epilogue: registers 4*q .. 4*q+3 of an atom are n = 8*q + 4*g + {0,1,2,3} of column m = lane % 32.
+    // Epilogue: registers 4*q .. 4*q+3 of an atom are n = 8*q + 4*g + {0,1,2,3} of column m = lane % 32. An output
+    // larger than the L2s together (8 x 4 MB) is stored with the non-temporal hint, so that it does not push the
+    // operand panels out of them.
+    const bool stream_out = size_t(m) * n * sizeof(Elem) > (size_t(32) << 20);
+    const __amdgpu_buffer_rsrc_t rsrc_c = make_out_rsrc(C + size_t(m0) * n + n0);
     const int m_lane = m0 + wm * Cfg::WTM + lane % 32;
     const int n_lane = n0 + wn * Cfg::WTN + 4 * g;
 #pragma unroll
     for (int j = 0; j < TM; ++j) {
         const int mm = m_lane + j * 32;
         if (mm >= m) continue;
-        Elem* row = C + size_t(mm) * n;
 #pragma unroll
         for (int i = 0; i < TN; ++i)
 #pragma unroll
@@ -188,7 +191,7 @@ dense_gemm_body(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, El
                 const int nn = n_lane + i * 32 + q * 8;
                 if (nn < n) {
                     const f32x4 v = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
-                    *reinterpret_cast<decltype(pack4(v, Elem{}))*>(row + nn) = pack4(v, Elem{});
+                    buffer_store_8(pack4(v, Elem{}), rsrc_c, uint32_t((mm - m0) * n + nn - n0) * 2u, stream_out);
                 }
             }
     }
@@ -355,6 +358,7 @@ dense_gemm_body_8w(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
             __builtin_amdgcn_s_barrier();
             asm volatile("" ::: "memory");
             uint8_t* region = (wave < 4 ? a_last : b_last) + (wave % 4) * (16 * PITCH);
+            const __amdgpu_buffer_rsrc_t rsrc_c = make_out_rsrc(C + size_t(cur.m0) * n + cur.n0);
             const int r4 = lane / 16, c = lane % 16;
             const int nn = n_slab + 8 * c;
 #pragma unroll
@@ -366,11 +370,8 @@ dense_gemm_body_8w(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
                 for (int q = 0; q < 4; ++q) {
                     const int row = 4 * q + r4, mm = m_slab + 16 * j + row;
                     const i32x4 v = *reinterpret_cast<const i32x4*>(region + row * PITCH + c * 16);
-                    if (mm < m && nn < n) {
-                        i32x4* dst = reinterpret_cast<i32x4*>(C + size_t(mm) * n + nn);
-                        if (stream_out) __builtin_nontemporal_store(v, dst);
-                        else *dst = v;
-                    }
+                    if (mm < m && nn < n)
+                        buffer_store_16(v, rsrc_c, uint32_t((wm * WTM + 16 * j + row) * n + wn * WTN + 8 * c) * 2u, stream_out);
                 }
             }
             // an interior tile: every lane of every wave has just issued exactly STORES_PER_TILE stores

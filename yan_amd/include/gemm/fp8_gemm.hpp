@@ -337,10 +337,11 @@ fp8_gemm_kernel(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_s
     // the operand panels the other workgroups of the XCD are about to read.
     bool staged = false;
     if constexpr (kStagedEpilogue) staged = (N % 8) == 0;
+    const bool stream_out = size_t(m) * N * 2 * (kGemmType == GemmType::GroupedMasked ? gridDim.x / sched.grid_size() : 1) > (size_t(32) << 20);
+    const __amdgpu_buffer_rsrc_t rsrc_out = make_out_rsrc(out + size_t(m0) * N + n0);
     if (staged) {
         if constexpr (kStagedEpilogue) {
             constexpr int PITCH = 288;
-            const bool stream_out = size_t(m) * N * 2 > (size_t(32) << 20);
             __syncthreads();                                   // every wave has read the last k-tile
             // Everything the epilogue derives from the lane number is derived here, behind an opaque copy of it: the
             // main loop has no registers to spare for addresses computed ahead of time.
@@ -360,11 +361,7 @@ fp8_gemm_kernel(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_s
                     const i32x4 v = *reinterpret_cast<const i32x4*>(region + row * PITCH + c * 16);
                     bool live = mm < m && nn < N;
                     if constexpr (kTwoHalves) live = live && mm >= pass_lo[pass] && mm < pass_hi[pass];
-                    if (live) {
-                        i32x4* dst = reinterpret_cast<i32x4*>(out + size_t(mm) * N + nn);
-                        if (stream_out) __builtin_nontemporal_store(v, dst);
-                        else *dst = v;
-                    }
+                    if (live) buffer_store_16(v, rsrc_out, uint32_t((mm - m0) * N + nn - n0) * 2u, stream_out);
                 }
                 __builtin_amdgcn_sched_barrier(0);      // one 16-row pass at a time: the registers are full of sums
             }
@@ -375,11 +372,10 @@ fp8_gemm_kernel(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_s
             const int mm = m_slab + j * 16 + col;
             if (mm >= m) continue;
             if constexpr (kTwoHalves) { if (mm < pass_lo[pass] || mm >= pass_hi[pass]) continue; }
-            __bf16* row = out + size_t(mm) * N;
 #pragma unroll
             for (int i = 0; i < TN; ++i) {
                 const int nn = n_slab + i * 16 + 4 * g;
-                if (nn < N) *reinterpret_cast<bf16x4*>(row + nn) = pack4(acc[i][j], __bf16{});
+                if (nn < N) buffer_store_8(pack4(acc[i][j], __bf16{}), rsrc_out, uint32_t((mm - m0) * N + nn - n0) * 2u, stream_out);
             }
         }
     }

@@ -43,6 +43,24 @@ __device__ __forceinline__ float buffer_load_f32(__amdgpu_buffer_rsrc_t rsrc, ui
     return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsrc, voffset, soffset, 0));
 }
 
+// Output stores through a descriptor, with or without the non-temporal hint (cache policy bit 1 on gfx950), chosen at
+// run time. Two intrinsic calls with different immediates on purpose: a pair of ordinary stores that differ only in
+// their non-temporal metadata is merged by the compiler into one plain store.
+__device__ __forceinline__ void buffer_store_16(i32x4 v, __amdgpu_buffer_rsrc_t rsrc, uint32_t voffset, bool streaming) {
+    if (streaming) __builtin_amdgcn_raw_buffer_store_b128(v, rsrc, voffset, 0, 2);
+    else __builtin_amdgcn_raw_buffer_store_b128(v, rsrc, voffset, 0, 0);
+}
+template <typename T8>      // any 8-byte vector
+__device__ __forceinline__ void buffer_store_8(T8 v, __amdgpu_buffer_rsrc_t rsrc, uint32_t voffset, bool streaming) {
+    typedef int i32x2 __attribute__((ext_vector_type(2)));
+    static_assert(sizeof(T8) == 8);
+    if (streaming) __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(i32x2, v), rsrc, voffset, 0, 2);
+    else __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(i32x2, v), rsrc, voffset, 0, 0);
+}
+// Descriptor over an output tile whose first element is `origin`: offsets are relative to it, bounds are the caller's
+// business (rows and columns past the matrix are skipped by predicate).
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_out_rsrc(const void* origin) { return make_rsrc(origin, 0xffffffffu); }
+
 // Per-thread state for staging a ROWS x 128-byte tile with NUM_WAVES waves: one VGPR. Everything that varies
 // per pass or per k-tile is wave-uniform and rides in the instruction's scalar offset, which the hardware adds
 // before its bounds check; a row past the end of the matrix lands at or beyond num_records and reads as zero.
