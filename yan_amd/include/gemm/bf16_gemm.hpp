@@ -346,12 +346,12 @@ dense_gemm_body_8w(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
         // Epilogue: the 4 registers of atom (i, j) are n = n_slab + 16 i + 4 g + {0..3} of row m = m_slab + 16 j + col.
         // Stored straight from there a wave instruction would write 16 rows x 32 bytes; instead each wave turns its slab
         // round through the stage that was consumed last, 16 rows at a time, and stores 4 rows x 256 consecutive bytes
-        // per instruction (16 bytes per lane). Rows are 288 bytes apart in LDS so that the 8-byte writes of 16 rows
+        // per instruction (16 bytes per lane). Rows are 272 bytes apart in LDS so that the 8-byte writes of 16 rows
         // spread over the banks. The other stage is receiving the next tile meanwhile.
         const int m_slab = cur.m0 + wm * WTM, n_slab = cur.n0 + wn * WTN;
         static_assert(WTM == 64 && WTN == 128 && sizeof(Elem) == 2, "the staged epilogue is laid out for 128 x 64 slabs");
         if ((n % 8) == 0) {
-            constexpr int PITCH = 288;
+            constexpr int PITCH = 272;
             // every wave has read the last k-tile (a bare barrier: nothing here depends on the copies under way)
             __builtin_amdgcn_s_waitcnt(waitcnt_imm(kNoWaitVm, 0));
             asm volatile("" ::: "memory");

@@ -331,7 +331,7 @@ fp8_gemm_kernel(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_s
 
     // Epilogue: the 4 registers of atom (i, j) are n = n_slab + 16i + 4g + {0..3} of row m = m_slab + 16j + col.
     // Stored straight from there a wave instruction writes 16 rows x 32 bytes. The 256 x 256 tile instead turns each
-    // wave's slab round through the LDS stage that was consumed last, 16 rows at a time (rows 288 bytes apart, so that
+    // wave's slab round through the LDS stage that was consumed last, 16 rows at a time (rows 272 bytes apart, so that
     // the 8-byte writes of 16 rows spread over the banks), and stores 4 rows x 256 consecutive bytes per instruction.
     // An output larger than the L2s together (8 x 4 MB) is stored with the non-temporal hint: kept in L2 it pushes out
     // the operand panels the other workgroups of the XCD are about to read.
@@ -341,7 +341,7 @@ fp8_gemm_kernel(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_s
     const __amdgpu_buffer_rsrc_t rsrc_out = make_out_rsrc(out + size_t(m0) * N + n0);
     if (staged) {
         if constexpr (kStagedEpilogue) {
-            constexpr int PITCH = 288;
+            constexpr int PITCH = 272;
             __syncthreads();                                   // every wave has read the last k-tile
             // Everything the epilogue derives from the lane number is derived here, behind an opaque copy of it: the
             // main loop has no registers to spare for addresses computed ahead of time.
