@@ -249,8 +249,9 @@ fp8_gemm_kernel(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_s
             }
         });
     };
-    // The staged epilogue (below) turns the slab round through the LDS stage that was consumed last.
-    constexpr bool kStagedEpilogue = STAGES == 2 && NW == 8 && Cfg::WTN == 128 && Cfg::WTM == 64;
+    // The staged epilogue (below) turns the slab round through the LDS stage that was consumed last: its operand tiles
+    // start at `epi_a` and `epi_b`.
+    constexpr bool kStagedEpilogue = Cfg::WTN >= 32;
     [[maybe_unused]] uint8_t* epi_a = nullptr;
     [[maybe_unused]] uint8_t* epi_b = nullptr;
     for (int pass = 0; pass < (kGemmType == GemmType::GroupedContiguous ? num_passes : 1); ++pass) {
@@ -327,12 +328,15 @@ fp8_gemm_kernel(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_s
         });
         st = st + 1 == STAGES ? 0 : st + 1;
     }
+    epi_a = ring + (st == 0 ? STAGES - 1 : st - 1) * STAGE_BYTES;
+    epi_b = epi_a + A_BYTES;
     }
 
     // Epilogue: the 4 registers of atom (i, j) are n = n_slab + 16i + 4g + {0..3} of row m = m_slab + 16j + col.
-    // Stored straight from there a wave instruction writes 16 rows x 32 bytes. The 256 x 256 tile instead turns each
-    // wave's slab round through the LDS stage that was consumed last, 16 rows at a time (rows 272 bytes apart, so that
-    // the 8-byte writes of 16 rows spread over the banks), and stores 4 rows x 256 consecutive bytes per instruction.
+    // Stored straight from there a wave instruction writes 16 rows x 32 bytes. Slabs of 32 columns or more instead turn
+    // round through the LDS stage that was consumed last (the only one no copy is on its way into), 16 rows at a time,
+    // and are stored 16 bytes per lane in runs of 2 * WTN consecutive bytes per row. Rows are WTN * 2 + 16 bytes apart
+    // in LDS, which spreads the 8-byte writes of 16 rows over the banks.
     // An output larger than the L2s together (8 x 4 MB) is stored with the non-temporal hint: kept in L2 it pushes out
     // the operand panels the other workgroups of the XCD are about to read.
     bool staged = false;
@@ -341,23 +345,31 @@ fp8_gemm_kernel(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_s
     const __amdgpu_buffer_rsrc_t rsrc_out = make_out_rsrc(out + size_t(m0) * N + n0);
     if (staged) {
         if constexpr (kStagedEpilogue) {
-            constexpr int PITCH = 272;
-            __syncthreads();                                   // every wave has read the last k-tile
+            constexpr int PITCH = Cfg::WTN * 2 + 16, REGION = 16 * PITCH;
+            constexpr int LANES_PER_ROW = Cfg::WTN / 8, ROWS_PER_STORE = kWaveSize / LANES_PER_ROW, STORES = 16 / ROWS_PER_STORE;
+            static_assert(STORES >= 1 && (NW / 2) * REGION <= Cfg::LDS_ROWS_A * kRowBytes && (NW / 2) * REGION <= Cfg::LDS_ROWS_B * kRowBytes);
+            // every wave has read the last k-tile (a bare barrier: __syncthreads() would also wait for the copies still
+            // on their way into the other stages, which nobody will read)
+            __builtin_amdgcn_s_waitcnt(waitcnt_imm(kNoWaitVm, 0));
+            asm volatile("" ::: "memory");
+            __builtin_amdgcn_s_barrier();
+            asm volatile("" ::: "memory");
             // Everything the epilogue derives from the lane number is derived here, behind an opaque copy of it: the
             // main loop has no registers to spare for addresses computed ahead of time.
             int lane_late = lane;
             asm volatile("" : "+v"(lane_late));
-            uint8_t* region = (wave < 4 ? epi_a : epi_b) + (wave % 4) * (16 * PITCH);
-            const int r4 = lane_late / 16, c = lane_late % 16;
+            uint8_t* region = (wave < NW / 2 ? epi_a : epi_b) + (wave % (NW / 2)) * REGION;
+            const int col_late = lane_late % 16, g_late = lane_late / 16;
+            const int r_in = lane_late / LANES_PER_ROW, c = lane_late % LANES_PER_ROW;
             const int nn = n_slab + 8 * c;
 #pragma unroll
             for (int j = 0; j < TM; ++j) {
 #pragma unroll
                 for (int i = 0; i < TN; ++i)
-                    *reinterpret_cast<bf16x4*>(region + c * PITCH + (16 * i + 4 * r4) * 2) = pack4(acc[i][j], __bf16{});
+                    *reinterpret_cast<bf16x4*>(region + col_late * PITCH + (16 * i + 4 * g_late) * 2) = pack4(acc[i][j], __bf16{});
 #pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    const int row = 4 * q + r4, mm = m_slab + 16 * j + row;
+                for (int q = 0; q < STORES; ++q) {
+                    const int row = ROWS_PER_STORE * q + r_in, mm = m_slab + 16 * j + row;
                     const i32x4 v = *reinterpret_cast<const i32x4*>(region + row * PITCH + c * 16);
                     bool live = mm < m && nn < N;
                     if constexpr (kTwoHalves) live = live && mm >= pass_lo[pass] && mm < pass_hi[pass];
