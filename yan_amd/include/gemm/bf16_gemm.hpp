@@ -173,11 +173,44 @@ dense_gemm_body(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, El
         st = st + 1 == STAGES ? 0 : st + 1;
     }
 
-    // Epilogue: registers 4*q .. 4*q+3 of an atom are n = 8*q + 4*g + {0,1,2,3} of column m = lane % 32. An output
-    // larger than the L2s together (8 x 4 MB) is stored with the non-temporal hint, so that it does not push the
-    // operand panels out of them.
+    // Epilogue: registers 4*q .. 4*q+3 of an atom are n = 8*q + 4*g + {0,1,2,3} of column m = lane % 32. Stored straight
+    // from there a wave instruction writes 32 rows x 16 bytes; instead each wave turns its slab round through the
+    // stage that was consumed last (the only one no copy is on its way into), 32 rows at a time, and stores 16 bytes
+    // per lane in runs of 2 * WTN consecutive bytes per row. An output larger than the L2s together (8 x 4 MB) is
+    // stored with the non-temporal hint, so that it does not push the operand panels out of them.
     const bool stream_out = size_t(m) * n * sizeof(Elem) > (size_t(32) << 20);
     const __amdgpu_buffer_rsrc_t rsrc_c = make_out_rsrc(C + size_t(m0) * n + n0);
+    constexpr int PITCH = Cfg::WTN * 2 + 16, REGION = 32 * PITCH;
+    constexpr int LANES_PER_ROW = Cfg::WTN / 8, ROWS_PER_STORE = kWaveSize / LANES_PER_ROW, STORES = 32 / ROWS_PER_STORE;
+    static_assert(NW * REGION <= STAGE_BYTES && STORES >= 1 && sizeof(Elem) == 2);
+    if ((n % 8) == 0) {
+        // every wave has read the last k-tile (a bare barrier: nothing here depends on the copies still under way)
+        __builtin_amdgcn_s_waitcnt(waitcnt_imm(kNoWaitVm, 0));
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        uint8_t* region = ring + (st == 0 ? STAGES - 1 : st - 1) * STAGE_BYTES + wave * REGION;
+        const int ml = lane % 32, r_in = lane / LANES_PER_ROW, c = lane % LANES_PER_ROW;
+        const int n_in_tile = wn * Cfg::WTN + 8 * c;
+#pragma unroll
+        for (int j = 0; j < TM; ++j) {
+#pragma unroll
+            for (int i = 0; i < TN; ++i)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const f32x4 v = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
+                    *reinterpret_cast<decltype(pack4(v, Elem{}))*>(region + ml * PITCH + (32 * i + 8 * q + 4 * g) * 2) = pack4(v, Elem{});
+                }
+#pragma unroll
+            for (int s = 0; s < STORES; ++s) {
+                const int row = ROWS_PER_STORE * s + r_in, m_in_tile = wm * Cfg::WTM + 32 * j + row;
+                const i32x4 v = *reinterpret_cast<const i32x4*>(region + row * PITCH + c * 16);
+                if (m0 + m_in_tile < m && n0 + n_in_tile < n)
+                    buffer_store_16(v, rsrc_c, uint32_t(m_in_tile * n + n_in_tile) * 2u, stream_out);
+            }
+        }
+        return;
+    }
     const int m_lane = m0 + wm * Cfg::WTM + lane % 32;
     const int n_lane = n0 + wn * Cfg::WTN + 4 * g;
 #pragma unroll
