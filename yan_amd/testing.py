@@ -149,6 +149,7 @@ DENSE_TEST_SHAPES = [
     (128, 4096, 7168), (512, 4096, 2048), (1024, 7168, 1024),
     (3000, 5000, 1000),          # the 256 x 256 tile (8-wave kernel) with ragged m, n and a k tail
     (2900, 5004, 520),           # same with n % 8 == 4 (narrow stores) and an odd number of k-tiles
+    (2900, 5000, 64),            # same with a single k-tile
 ]
 # (m, n, k) of the reference's own dense test (tests/test_cute.py:21-22: m in (256, 4096) x six (k, n) pairs)
 REFERENCE_DENSE_TEST_SHAPES = [(m, n, k) for m in (256, 4096)
