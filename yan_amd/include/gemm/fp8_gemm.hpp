@@ -14,6 +14,8 @@
 //     s = sA * sB. Weights feed the MFMA row operand and activations the column operand, so a lane only ever
 //     meets one activation row per atom: one sA per lane per atom per K block, and sB is wave-uniform;
 //   * the running sums stay in architectural VGPRs (the VALU cannot address AGPRs): 128 per wave;
+//   * the output leaves through LDS: each wave turns its slab round through the stage that was consumed last and stores
+//     16 bytes per lane in row runs of 2 * WTN bytes (non-temporal when the output is larger than the L2s together);
 //   * m is a run-time argument with tails predicated; N and K are compile-time;
 //   * grouped (mixture-of-experts) layouts, the reference's GemmType::GroupedContiguous / GroupedMasked hooks
 //     (yan/include/gemm/scheduler.cuh:7-11,31-48, `int* grouped_layout` of fp8_gemm.cuh:41): every output tile
