@@ -772,6 +772,51 @@ def test_entry_points_replay_correctly_from_a_captured_graph():
         assert float(replayed['fp8'].float().abs().sum()) > 0 and float(replayed['masked'][1, 40:].float().abs().sum()) == 0
 
 
+def test_capi_seeded_random_shapes_against_device_references():
+    """Breadth: 240 seeded random shapes through the C entries (every tile variant, ragged edges, k tails, leading
+    dimensions), each against an fp32 / fp64 product of the same operands on the device. The oracle-based tests above
+    pin the arithmetic; this one looks for a shape that breaks the tiling."""
+    import random
+    rng = random.Random(1234)
+    _announce('capi random shapes')
+
+    def rel_diff(x, y):
+        x, y = x.double(), y.double()
+        return float(1 - 2 * (x * y).sum() / ((x * x + y * y).sum() + 1e-300))
+
+    for it in range(90):
+        m = rng.choice([1, 7, 64, 255, 256, 257, 1000, 2048, 3000, 4100, 6000])
+        n, k = 4 * rng.randint(1, 1500), 8 * rng.randint(1, 300)
+        dtype = rng.choice([torch.bfloat16, torch.half])
+        a, b = torch.randn(m, k, device='cuda').to(dtype), torch.randn(n, k, device='cuda').to(dtype)
+        c = torch.full((m, n), 7.0, device='cuda', dtype=dtype)
+        assert (capi.gemm_bf16_tn if dtype == torch.bfloat16 else capi.gemm_fp16_tn)(a, b, c) == 0
+        assert rel_diff(c.float(), a.float() @ b.float().t()) < BF16_TOL, ('dense', m, n, k, dtype)
+    for it in range(90):
+        m = rng.choice([1, 5, 16, 17, 64, 100, 256, 300, 1024, 2050, 4096, 6000])
+        n, k = 4 * rng.randint(1, 1800), 128 * rng.randint(1, 24)
+        (a8, sa), (b8, sb), out = testing.make_fp8_case(m, n, k, seed=it, device='cuda', gen_device='cuda')
+        out.fill_(7.0)
+        if rng.random() < 0.5:
+            sa = yan.get_col_major_tensor(sa)
+        assert capi.gemm_fp8_fp8_bf16_nt((a8, sa), (b8, sb), out) == 0
+        ref = testing.dequant_lhs(a8, sa) @ testing.dequant_rhs(b8, sb).t()
+        assert rel_diff(out.float(), ref) < 1e-5, ('fp8', m, n, k)
+    lib = capi.load()
+    for it in range(60):
+        m, n, k = 4 * rng.randint(1, 600), 4 * rng.randint(1, 600), rng.randint(0, 700)
+        lda, ldb, ldc = m + 4 * rng.randint(0, 3), n + 4 * rng.randint(0, 3), n + 4 * rng.randint(0, 3)
+        a_buf, b_buf = torch.randn(max(k, 1), lda, device='cuda'), torch.randn(max(k, 1), ldb, device='cuda')
+        c_buf = torch.randn(m, ldc, device='cuda')
+        alpha, beta = rng.choice([(1.0, 0.0), (0.5, 2.0), (-1.0, 1.0)])
+        want = alpha * (a_buf[:k, :m].double().t() @ b_buf[:k, :n].double()) + (beta * c_buf[:, :n].double() if beta else 0)
+        keep = c_buf[:, n:].clone()
+        assert lib.yan_gemm_float_nt(m, n, k, alpha, a_buf.data_ptr(), lda, b_buf.data_ptr(), ldb, beta, c_buf.data_ptr(), ldc, None) == 0
+        torch.cuda.synchronize()
+        assert float((c_buf[:, :n].double() - want).abs().max()) < 1e-3, ('fp32', m, n, k, lda, ldb, ldc, alpha, beta)
+        assert torch.equal(keep, c_buf[:, n:])
+
+
 def test_capi_rejects_bad_sizes_on_device():
     from yan_amd import capi
     a = torch.zeros(64, 64, dtype=torch.bfloat16, device='cuda')
