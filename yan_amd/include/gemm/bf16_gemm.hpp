@@ -461,6 +461,8 @@ inline hipError_t check_dense_args(int m, int n, int k, const void* a, const voi
     // 32-bit descriptor offsets: every tile row, including the overhang of the last tile, must stay below 2 GiB
     const uint64_t m_pad = uint64_t(ceil_div(m, block_m)) * block_m, n_pad = uint64_t(ceil_div(n, block_n)) * block_n;
     if (m_pad * k * 2 >= kOutOfRange || n_pad * k * 2 >= kOutOfRange) return hipErrorInvalidValue;
+    // output stores address a tile with 32-bit byte offsets from its first element: block_m rows of n elements
+    if (uint64_t(block_m) * n * 2 >= kOutOfRange) return hipErrorInvalidValue;
     return hipSuccess;
 }
 

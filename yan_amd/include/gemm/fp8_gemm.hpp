@@ -433,6 +433,8 @@ public:
         if (!out || !lhs || !lhs_scales || !rhs || !rhs_scales || !grouped_layout) return hipErrorInvalidValue;
         const uint64_t m_pad = uint64_t(ceil_div<uint32_t>(m, BLOCK_M)) * BLOCK_M, n_pad = uint64_t(ceil_div<uint32_t>(n, BLOCK_N)) * BLOCK_N;
         if (m_pad * k >= kOutOfRange || n_pad * k >= kOutOfRange) return hipErrorInvalidValue;
+        // output stores address a tile with 32-bit byte offsets from its first element: BLOCK_M rows of n elements
+        if (uint64_t(BLOCK_M) * n * 2 >= kOutOfRange) return hipErrorInvalidValue;
         using Cfg = Fp8TileConfig<BLOCK_M, BLOCK_N>;
         const XcdTileScheduler<> sched(m, n, BLOCK_M, BLOCK_N);
         const uint64_t grid = uint64_t(sched.grid_size()) * (kGemmType == GemmType::GroupedMasked ? num_groups : 1);
@@ -456,6 +458,8 @@ public:
         // 32-bit descriptor offsets: every tile row, including the overhang of the last tile, must stay below 2 GiB
         const uint64_t m_pad = uint64_t(ceil_div<uint32_t>(m, BLOCK_M)) * BLOCK_M, n_pad = uint64_t(ceil_div<uint32_t>(n, BLOCK_N)) * BLOCK_N;
         if (m_pad * k >= kOutOfRange || n_pad * k >= kOutOfRange) return hipErrorInvalidValue;
+        // output stores address a tile with 32-bit byte offsets from its first element: BLOCK_M rows of n elements
+        if (uint64_t(BLOCK_M) * n * 2 >= kOutOfRange) return hipErrorInvalidValue;
         using Cfg = Fp8TileConfig<BLOCK_M, BLOCK_N>;
         const XcdTileScheduler<> sched(m, n, BLOCK_M, BLOCK_N);
         hipLaunchKernelGGL((fp8_gemm_kernel<SHAPE_N, SHAPE_K, BLOCK_M, BLOCK_N, GemmType::Normal, int(kNumStages)>), dim3(sched.grid_size()),
