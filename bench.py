@@ -4,8 +4,15 @@
 A step is one FP8 e4m3 block-scaled GEMM at M=4096, N=7168, K=7168 (per-token 1x128 activation scales, 128x128
 weight scales, bf16 output) through the JIT entry point, inputs resident in HBM before the timed region.
 Prints ONE JSON line: whole-job TFLOPS, the roofline position of the GEMM kernel (HIP-event time of the launches
-on the stream they run on) and a torch-CPU baseline on a bounded slab of the same workload.
-`--also` adds the other baseline configurations (bf16 8192^3, the M=64 decode shape) as extra fields.
+on the stream they run on), the other baseline configurations as compact legs under `extra` (bf16 8192^3 next to
+the vendor library on the same operands, the M=64 decode shape, FP8 16384^3 with outliers) and a torch-CPU baseline
+of the same workload. `--also` adds the grouped GEMMs, the quantisers and the fp32 GEMM to `extra`.
+
+Order of operations for every leg: `settle` untimed launches of the same kernel, `warmup` untimed launches, the timed
+launches, and only then the validity check. The settle phase exists because the chip's power controller reacts to the
+onset of a matrix-core load: coming from idle the first ~10 launches run at the steady rate, the next ~30 run up to a
+third slower while the clock is pulled down, and the rate is back to steady only after ~100 launches. A run that times
+25 launches after an idle period measures that transient, not the kernel. The count is printed with each leg.
 """
 import argparse
 import json
@@ -15,6 +22,7 @@ import time
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, 'tests'))
 os.environ.setdefault('YAN_CACHE_DIR', os.path.join(ROOT, '.yan_cache'))
 
 METRIC = 'TFLOPS & % of MFMA peak, fp8 block-scaled GEMM 4096x7168x7168, 1 MI355X'
@@ -23,11 +31,16 @@ PEAK_FP8_TFLOPS = 5000.0
 PEAK_BF16_TFLOPS = 2500.0
 PEAK_HBM_GBPS = 8000.0
 PEAK_FP32_TFLOPS = 157.3
+# Untimed launches of the leg's own kernel before its warm-up: about 100 ms of load each.
+SETTLE = {'cfg3': 600, 'cfg2': 150, 'cfg4': 2000, 'cfg5': 30}
 
 
-def _event_time_ms(fn, steps, warmup):
-    """Average device time of one call over `steps` back-to-back calls, from events on the current stream."""
+def _event_time_ms(fn, steps, warmup, settle=0):
+    """Average device time of one call over `steps` back-to-back calls, from events on the current stream, after
+    `settle` + `warmup` untimed calls. Returns (event ms per call, wall ms per call)."""
     import torch
+    for _ in range(settle):
+        fn()
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
@@ -47,15 +60,15 @@ def _cpu_baseline_fp8(a8, sa, b8, sb, budget_s=12.0):
     slab of rows sized for about `budget_s` seconds, scaled to the full M by the flop count."""
     import torch
     import oracle
-    from yan_amd import testing
+    import harness
     m, k = a8.shape
     n = b8.shape[0]
     b_cpu, sb_cpu = b8.cpu(), sb.cpu()
-    wd = testing.dequant_rhs(b_cpu, sb_cpu)
+    wd = harness.dequant_rhs(b_cpu, sb_cpu)
 
     def run(rows):
         t0 = time.perf_counter()
-        x = testing.dequant_lhs(a8[:rows].cpu(), sa[:rows].cpu())
+        x = harness.dequant_lhs(a8[:rows].cpu(), sa[:rows].cpu())
         out = x @ wd.t()
         return time.perf_counter() - t0, out
 
@@ -77,28 +90,53 @@ def _cpu_baseline_fp8(a8, sa, b8, sb, budget_s=12.0):
 
 
 def _measured_traffic():
-    """HBM bytes per launch of the GEMM kernel as measured with rocprofv3 hardware counters (FETCH_SIZE + WRITE_SIZE,
-    scaled by a copy of known size); the figure is kept with the profile summary it comes from. None if absent."""
+    """HBM-side bytes per launch of the GEMM kernel as measured with rocprofv3 hardware counters (FETCH_SIZE +
+    WRITE_SIZE, scaled by a copy of known size). The figure is kept with the profile summary it comes from, which also
+    records the digest of the kernel headers it was taken with: (bytes, digest) when that digest is the one of the
+    headers in this tree, (None, digest-or-None) when the profile is absent or older than the kernel."""
+    from yan_amd.jit.compiler import get_yan_version
     path = os.path.join(ROOT, 'profiles', 'fp8_gemm_4096x7168x7168_hbm_traffic.md')
+    traffic = version = None
     try:
         for line in open(path):
             if line.startswith('traffic_bytes_per_launch:'):
-                return float(line.split(':', 1)[1].split()[0])
+                traffic = float(line.split(':', 1)[1].split()[0])
+            elif line.startswith('kernel_headers_digest:'):
+                version = line.split(':', 1)[1].split()[0]
     except OSError:
         pass
-    return None
+    if traffic is None or version != get_yan_version():
+        return None, version
+    return traffic, version
+
+
+def _fp8_bytes(m, n, k):
+    return m * k + n * k + 4 * m * (k // 128) + 4 * ((n + 127) // 128) * (k // 128) + 2 * m * n
+
+
+def _sampled_fp8_diff(yan, harness, a8, sa, b8, sb, out, rows=256):
+    import torch
+    m = a8.shape[0]
+    pick = torch.randperm(m, device='cuda')[:min(rows, m)]
+    wd_t = harness.dequant_rhs(b8, sb).t() if b8.numel() <= (1 << 27) else None
+    if wd_t is not None:
+        ref = harness.dequant_lhs(a8[pick], sa[pick]) @ wd_t
+    else:       # 16384^2 weights: dequantise in column slabs
+        x = harness.dequant_lhs(a8[pick], sa[pick])
+        ref = torch.cat([x @ harness.dequant_rhs(b8[c0:c0 + 2048], sb[c0 // 128:c0 // 128 + 16]).t()
+                         for c0 in range(0, b8.shape[0], 2048)], dim=1)
+    return float(yan.calc_diff(out[pick].float(), ref))
 
 
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument('--gpus', type=int, default=1)
-    ap.add_argument('--steps', type=int, default=1000)
-    ap.add_argument('--warmup', type=int, default=100)
-    ap.add_argument('--also', action='store_true', help='also time bf16 8192^3, the decode shape, 16384^3, the grouped GEMMs, the quantisers and the fp32 GEMM (extra fields)')
+    ap.add_argument('--steps', type=int, default=200)
+    ap.add_argument('--warmup', type=int, default=20)
+    ap.add_argument('--also', action='store_true', help='also time the grouped GEMMs, the quantisers and the fp32 GEMM (more extra fields)')
     ap.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline leg')
-    ap.add_argument('--ceilings', action='store_true',
-                    help='also measure what the matrix cores sustain with register-resident operands, and what the main loop of the '
-                         'block-scaled kernel sustains on a tile that never changes (random and zero bits)')
+    ap.add_argument('--no-extra', action='store_true', help='skip the legs of the other baseline configurations')
+    ap.add_argument('--no-settle', action='store_true', help='skip the untimed settle launches (shows the power transient)')
     ap.add_argument('--calibrate-copy', action='store_true',
                     help='also run a 1 GiB device-to-device copy three times, as the known-size kernel that hardware '
                          'byte counters (FETCH_SIZE / WRITE_SIZE) are scaled by when profiling')
@@ -110,23 +148,18 @@ def main():
 
     import torch
     import yan_amd as yan
-    from yan_amd import testing
+    import harness
     from yan_amd.jit_kernels.gemm import fp8_kernel_plan
     assert torch.cuda.is_available(), 'bench.py needs a GPU'
     torch.cuda.set_device(0)
+    settle = {leg: (0 if args.no_settle else count) for leg, count in SETTLE.items()}
 
-    m, n, k = testing.BASELINE_FP8['cfg3']
-    (a8, sa), (b8, sb), out = testing.make_fp8_case(m, n, k, seed=42, device='cuda', gen_device='cuda')
+    m, n, k = harness.BASELINE_FP8['cfg3']
+    (a8, sa), (b8, sb), out = harness.make_fp8_case(m, n, k, seed=42, device='cuda', gen_device='cuda')
     sa = yan.get_col_major_tensor(sa)      # token-contiguous scales, the layout DeepGEMM-style callers hand over
     step = lambda: yan.gemm_fp8_fp8_bf16_nt((a8, sa), (b8, sb), out)
-
-    # validity of what is being timed: sampled rows against an fp32 matmul of the dequantised operands
-    step()
-    rows = torch.randperm(m, device='cuda')[:256]
-    ref = testing.dequant_lhs(a8[rows], sa[rows]) @ testing.dequant_rhs(b8, sb).t()
-    diff = float(yan.calc_diff(out[rows].float(), ref))
-    assert diff < 1e-3, f'parity lost: calc_diff={diff}'
-    del ref
+    step()                                  # loads the kernel
+    torch.cuda.synchronize()
 
     if args.calibrate_copy:
         src = torch.empty(1 << 30, dtype=torch.uint8, device='cuda').fill_(1)
@@ -136,12 +169,15 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
-    kernel_ms, wall_ms = _event_time_ms(step, args.steps, args.warmup)
+    kernel_ms, wall_ms = _event_time_ms(step, args.steps, args.warmup, settle['cfg3'])
+    # validity of what was timed: sampled rows against an fp32 matmul of the dequantised operands
+    diff = _sampled_fp8_diff(yan, harness, a8, sa, b8, sb, out)
+    assert diff < 1e-3, f'parity lost: calc_diff={diff}'
     flops = 2.0 * m * n * k
     tflops_job = flops / (wall_ms * 1e-3) / 1e12
     tflops_kernel = flops / (kernel_ms * 1e-3) / 1e12
-    bytes_alg = m * k + n * k + 4 * m * (k // 128) + 4 * ((n + 127) // 128) * (k // 128) + 2 * m * n
     _, keys, _, _, _ = fp8_kernel_plan(m, n, k, yan.get_num_sms())
+    traffic, traffic_digest = _measured_traffic()
 
     line = {
         'metric': METRIC, 'value': round(tflops_job, 1), 'unit': 'TFLOPS', 'n_gpus': 1,
@@ -150,59 +186,83 @@ def main():
         'data': 'synthetic: N(0,1) sources, seed 42, quantised per-token 1x128 / per-block 128x128',
         'config': {'workload': 'configs[2]: FP8 e4m3 block-scaled GEMM M=4096 N=7168 K=7168, bf16 out',
                    'tile': f"{keys['BLOCK_M']}x{keys['BLOCK_N']}x128", 'cache_state': 'warm (same operands every step)',
+                   'settle_launches': settle['cfg3'],
+                   'settle': 'untimed launches of the same kernel before the warm-up: the power controller takes ~100 launches '
+                             'to settle after an idle period',
                    'calc_diff_sampled_rows': diff},
         'roofline': {'bound': 'mfma', 'achieved': round(tflops_kernel, 1), 'peak': PEAK_FP8_TFLOPS, 'unit': 'TFLOP/s',
-                     'frac': round(tflops_kernel / PEAK_FP8_TFLOPS, 4), 'traffic': _measured_traffic(),
+                     'frac': round(tflops_kernel / PEAK_FP8_TFLOPS, 4), 'traffic': traffic,
+                     'traffic_source': f'profiles/fp8_gemm_4096x7168x7168_hbm_traffic.md, kernel headers {traffic_digest}'
+                                       if traffic is not None else 'no profile of the kernel headers in this tree',
                      'kernel': 'fp8_gemm_kernel', 'kernel_us': round(kernel_ms * 1e3, 2),
-                     'algorithmic_flop_per_launch': flops, 'algorithmic_bytes_per_launch': bytes_alg},
+                     'algorithmic_flop_per_launch': flops, 'algorithmic_bytes_per_launch': _fp8_bytes(m, n, k)},
     }
 
-    if args.also:
-        extra = {}
-        mm, nn, kk = testing.BASELINE_BF16['cfg2']
-        a, b, c = testing.make_bf16_case(mm, nn, kk, seed=42, scale=kk ** -0.5, device='cuda', gen_device='cuda')
-        ms, _ = _event_time_ms(lambda: yan.gemm_bf16_tn(a, b, c), 50, 10)
-        extra['bf16_8192'] = {'us': round(ms * 1e3, 1), 'tflops': round(2.0 * mm * nn * kk / ms / 1e9, 1),
-                              'frac_of_bf16_peak': round(2.0 * mm * nn * kk / ms / 1e9 / PEAK_BF16_TFLOPS, 4)}
-        ms, _ = _event_time_ms(lambda: torch.matmul(a, b.t(), out=c), 50, 10)
-        extra['bf16_8192_torch_hipblaslt'] = {'us': round(ms * 1e3, 1), 'tflops': round(2.0 * mm * nn * kk / ms / 1e9, 1)}
+    extra = {}
+    if not args.no_extra:
+        # configs[1]: bf16 8192^3, next to torch.matmul (hipBLASLt) on the same operands
+        mm, nn, kk = harness.BASELINE_BF16['cfg2']
+        a, b, c = harness.make_bf16_case(mm, nn, kk, seed=42, scale=kk ** -0.5, device='cuda', gen_device='cuda')
+        ms, _ = _event_time_ms(lambda: yan.gemm_bf16_tn(a, b, c), 20, 5, settle['cfg2'])
+        pick = torch.randperm(mm, device='cuda')[:256]
+        d = float(yan.calc_diff(c[pick].float(), a[pick].float() @ b.float().t()))
+        assert d < 1e-5, f'bf16 parity lost: calc_diff={d}'
+        fl = 2.0 * mm * nn * kk
+        extra['bf16_8192'] = {'us': round(ms * 1e3, 1), 'tflops': round(fl / ms / 1e9, 1),
+                              'frac_of_bf16_peak': round(fl / ms / 1e9 / PEAK_BF16_TFLOPS, 4), 'steps': 20, 'warmup': 5,
+                              'settle_launches': settle['cfg2'], 'calc_diff_sampled_rows': d}
+        ms, _ = _event_time_ms(lambda: torch.matmul(a, b.t(), out=c), 20, 5, settle['cfg2'])
+        extra['bf16_8192_torch_hipblaslt'] = {'us': round(ms * 1e3, 1), 'tflops': round(fl / ms / 1e9, 1)}
         del a, b, c
-        mm, nn, kk = testing.BASELINE_FP8['cfg4']
-        (x8, sx), (w8, sw), o = testing.make_fp8_case(mm, nn, kk, seed=42, device='cuda')
+        # configs[3]: the M=64 decode shape, HBM-bound. The kernel is shorter than the host side of a call, so its
+        # device time comes from the profiler; cold = a 512 MB write before every call.
+        mm, nn, kk = harness.BASELINE_FP8['cfg4']
+        (x8, sx), (w8, sw), o = harness.make_fp8_case(mm, nn, kk, seed=42, device='cuda')
         sx = yan.get_col_major_tensor(sx)
         decode = lambda: yan.gemm_fp8_fp8_bf16_nt((x8, sx), (w8, sw), o)
-        _, wall = _event_time_ms(decode, 200, 20)
-        # this kernel is shorter than the host side of a call, so its own device time comes from the profiler
-        ms = yan.bench_kineto(decode, 'fp8_gemm_kernel', suppress_kineto_output=True) * 1e3
-        ms_cold = yan.bench_kineto(decode, 'fp8_gemm_kernel', suppress_kineto_output=True, flush_l2=True) * 1e3
-        byt = mm * kk + nn * kk + 4 * mm * (kk // 128) + 4 * (nn // 128) * (kk // 128) + 2 * mm * nn
-        extra['fp8_decode_64x4096x7168'] = {'kernel_us_warm': round(ms * 1e3, 2), 'kernel_us_cold': round(ms_cold * 1e3, 2),
-                                            'call_to_call_us': round(wall * 1e3, 2),
-                                            'gb_per_s_warm': round(byt / ms / 1e6, 1), 'gb_per_s_cold': round(byt / ms_cold / 1e6, 1),
-                                            'frac_of_hbm_peak_cold': round(byt / ms_cold / 1e6 / PEAK_HBM_GBPS, 4)}
-        mm, nn, kk = testing.BASELINE_FP8['cfg5']
-        (x8, sx), (w8, sw), o = testing.make_fp8_case(mm, nn, kk, seed=42, dist='outlier', device='cuda', gen_device='cuda')
-        sx = yan.get_col_major_tensor(sx)
-        ms, _ = _event_time_ms(lambda: yan.gemm_fp8_fp8_bf16_nt((x8, sx), (w8, sw), o), 10, 2)
-        extra['fp8_16384_outliers'] = {'us': round(ms * 1e3, 1), 'tflops': round(2.0 * mm * nn * kk / ms / 1e9, 1),
-                                       'frac_of_fp8_peak': round(2.0 * mm * nn * kk / ms / 1e9 / PEAK_FP8_TFLOPS, 4)}
+        _, wall = _event_time_ms(decode, 200, 20, settle['cfg4'])
+        t_warm = yan.bench_kineto(decode, 'fp8_gemm', suppress_kineto_output=True)
+        t_cold = yan.bench_kineto(decode, 'fp8_gemm', suppress_kineto_output=True, flush_l2=True)
+        d = _sampled_fp8_diff(yan, harness, x8, sx, w8, sw, o)
+        assert d < 1e-3, f'decode parity lost: calc_diff={d}'
+        byt = _fp8_bytes(mm, nn, kk)
+        extra['fp8_decode_64x4096x7168'] = {'kernel_us_warm': round(t_warm * 1e6, 2), 'kernel_us_cold': round(t_cold * 1e6, 2),
+                                            'call_to_call_us': round(wall * 1e3, 2), 'algorithmic_bytes': byt,
+                                            'gb_per_s_warm': round(byt / t_warm / 1e9, 1), 'gb_per_s_cold': round(byt / t_cold / 1e9, 1),
+                                            'frac_of_hbm_peak_warm': round(byt / t_warm / 1e9 / PEAK_HBM_GBPS, 4),
+                                            'frac_of_hbm_peak_cold': round(byt / t_cold / 1e9 / PEAK_HBM_GBPS, 4),
+                                            'calc_diff': d}
         del x8, sx, w8, sw, o
+        # configs[4]: FP8 16384^3, uniform[-4, 4] sources with 1 % of the entries x 50
+        mm, nn, kk = harness.BASELINE_FP8['cfg5']
+        (x8, sx), (w8, sw), o = harness.make_fp8_case(mm, nn, kk, seed=42, dist='outlier', device='cuda', gen_device='cuda')
+        sx = yan.get_col_major_tensor(sx)
+        ms, _ = _event_time_ms(lambda: yan.gemm_fp8_fp8_bf16_nt((x8, sx), (w8, sw), o), 10, 2, settle['cfg5'])
+        d = _sampled_fp8_diff(yan, harness, x8, sx, w8, sw, o, rows=128)
+        assert d < 1e-3, f'16384^3 parity lost: calc_diff={d}'
+        fl = 2.0 * mm * nn * kk
+        extra['fp8_16384_outliers'] = {'us': round(ms * 1e3, 1), 'tflops': round(fl / ms / 1e9, 1),
+                                       'frac_of_fp8_peak': round(fl / ms / 1e9 / PEAK_FP8_TFLOPS, 4), 'steps': 10, 'warmup': 2,
+                                       'settle_launches': settle['cfg5'], 'calc_diff_sampled_rows': d}
+        del x8, sx, w8, sw, o
+
+    if args.also:
         # grouped (mixture-of-experts) layouts: 4 groups x 8192 rows contiguous; 4 groups x 1024 of 1024 rows masked
         rows, nn, kk = (8192,) * 4, 4096, 7168
-        (x8, sx), (w8, sw), o, idx = testing.make_grouped_contiguous_case(rows, nn, kk, seed=42, device='cuda', gen_device='cuda')
+        (x8, sx), (w8, sw), o, idx = harness.make_grouped_contiguous_case(rows, nn, kk, seed=42, device='cuda', gen_device='cuda')
         sx = yan.get_col_major_tensor(sx)
-        ms, _ = _event_time_ms(lambda: yan.m_grouped_gemm_fp8_fp8_bf16_nt_contiguous((x8, sx), (w8, sw), o, idx), 20, 3)
+        ms, _ = _event_time_ms(lambda: yan.m_grouped_gemm_fp8_fp8_bf16_nt_contiguous((x8, sx), (w8, sw), o, idx), 20, 3, 100)
         fl = 2.0 * sum(rows) * nn * kk
         extra['fp8_grouped_contiguous_4x8192x4096x7168'] = {'us': round(ms * 1e3, 1), 'tflops': round(fl / ms / 1e9, 1),
                                                             'frac_of_fp8_peak': round(fl / ms / 1e9 / PEAK_FP8_TFLOPS, 4)}
-        (x8, sx), (w8, sw), o, mm_ = testing.make_grouped_masked_case(4, 1024, nn, kk, (1024,) * 4, seed=42, device='cuda', gen_device='cuda')
-        ms, _ = _event_time_ms(lambda: yan.m_grouped_gemm_fp8_fp8_bf16_nt_masked((x8, sx), (w8, sw), o, mm_, 1024), 50, 5)
+        (x8, sx), (w8, sw), o, mm_ = harness.make_grouped_masked_case(4, 1024, nn, kk, (1024,) * 4, seed=42, device='cuda', gen_device='cuda')
+        ms, _ = _event_time_ms(lambda: yan.m_grouped_gemm_fp8_fp8_bf16_nt_masked((x8, sx), (w8, sw), o, mm_, 1024), 50, 5, 600)
         fl = 2.0 * 4 * 1024 * nn * kk
         extra['fp8_grouped_masked_4x1024x4096x7168'] = {'us': round(ms * 1e3, 1), 'tflops': round(fl / ms / 1e9, 1),
                                                         'frac_of_fp8_peak': round(fl / ms / 1e9 / PEAK_FP8_TFLOPS, 4)}
         del x8, sx, w8, sw, o
         # quantisers in front of the GEMM (HBM-bound): cfg3's activations per token, its weights per block, from bf16
-        mm, nn, kk = testing.BASELINE_FP8['cfg3']
+        mm, nn, kk = harness.BASELINE_FP8['cfg3']
         xs = torch.randn(mm, kk, device='cuda').bfloat16()
         ws = torch.randn(nn, kk, device='cuda').bfloat16()
         for name, fn, kern, elems, groups in (
@@ -218,7 +278,7 @@ def main():
         # fp32 GEMM (fp32 MFMA, 157.3 TFLOP/s peak): a large square, the largest shape of the reference's fp32 test and
         # its m = 128 shape with the fewest outputs, each next to torch.matmul (hipBLASLt) on the same operands
         for mm, nn, kk in ((8192, 8192, 8192), (4096, 7168, 16384), (128, 2112, 7168)):
-            a, b, c = testing.make_float_case(mm, nn, kk, seed=42, device='cuda', gen_device='cuda')
+            a, b, c = harness.make_float_case(mm, nn, kk, seed=42, device='cuda', gen_device='cuda')
             reps = 10 if mm > 128 else 200
             ms, _ = _event_time_ms(lambda: yan.gemm_float_nt(a, b, c), reps, 3)
             ms_t, _ = _event_time_ms(lambda: torch.matmul(a, b.t(), out=c), reps, 3)
@@ -227,16 +287,8 @@ def main():
                                              'frac_of_fp32_peak': round(fl / ms / 1e9 / PEAK_FP32_TFLOPS, 4),
                                              'torch_hipblaslt_us': round(ms_t * 1e3, 1)}
             del a, b, c
+    if extra:
         line['extra'] = extra
-
-    if args.ceilings:
-        from yan_amd import probe
-        line['ceilings_tflops'] = {kind: {data: round(probe.mfma_ceiling(kind, data), 1) for data in ('random', 'zero')}
-                                   for kind in probe.MODES}
-        line['roofline']['frac_of_mfma_only_ceiling'] = round(
-            tflops_kernel / line['ceilings_tflops']['fp8_16x16x128_zero_c_plus_fold']['random'], 4)
-        line['roofline']['frac_of_fed_loop_ceiling'] = round(
-            tflops_kernel / line['ceilings_tflops']['fp8_fold_plus_lds_reads_barrier_copies']['random'], 4)
 
     if not args.no_cpu:
         line['cpu_baseline'] = _cpu_baseline_fp8(a8, sa, b8, sb)

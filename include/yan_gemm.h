@@ -33,7 +33,8 @@ extern "C" {
 #endif
 
 /* c[m,n] = a[m,k] . b[n,k]^T, bf16 in, fp32 accumulate, bf16 out (round to nearest even).
- * Requires n % 4 == 0, k % 8 == 0, and (m rounded up to 256) * k * 2 < 2^31 bytes, same for n.
+ * Requires n % 4 == 0, k % 8 == 0, (m rounded up to the tile's rows, at most 256) * k * 2 < 2^31 bytes, same for n,
+ * and 256 * n * 2 < 2^31 bytes (output stores address one tile with 32-bit offsets).
  * Replaces gemm_fp16_tn -> gemm_tn<128,128,3> of the reference (yan/jit_kernels/cute_gemm.py:21-64,
  * yan/include/gemm/cute_gemm.cuh:262-378), with the bf16 dtype and fp32 accumulation. */
 YAN_API int yan_gemm_bf16_tn(int m, int n, int k, const void* a, const void* b, void* c, void* stream);
@@ -45,7 +46,8 @@ YAN_API int yan_gemm_fp16_tn(int m, int n, int k, const void* a, const void* b, 
  *   a  m x k with M contiguous: element (i, kk) at a[i + kk*lda];   b  n x k with N contiguous: b[j + kk*ldb];
  *   c  m x n row-major: c[i*ldc + j].  beta == 0 does not read c.
  * Requires m, n, lda, ldb, ldc multiples of 4, lda >= m, ldb >= n, ldc >= n, 16-byte aligned pointers and
- * (k + 144) * lda * 4 < 2^31 bytes, same for ldb. k == 0 scales c by beta.
+ * ((k + 1024) * lda + 256) * 4 < 2^31 bytes, same for ldb (the kernel prefetches up to 8 k-tiles of 128 k-rows past
+ * the end through a descriptor with 32-bit offsets; those rows read as zero). k == 0 scales c by beta.
  * Replaces gemm_float_nt -> gemm_nt of the reference (yan/jit_kernels/simple_gemm.py:18-57,
  * yan/include/gemm/simple_gemm.cuh:194-247), same argument order and memory convention. */
 YAN_API int yan_gemm_float_nt(int m, int n, int k, float alpha, const float* a, int lda, const float* b, int ldb,
@@ -57,9 +59,13 @@ YAN_API int yan_gemm_float_nt(int m, int n, int k, float alpha, const float* a, 
  *              (row-major: strides (k/128, 1); token-contiguous as DeepGEMM callers pass it: (1, m))
  *   rhs        e4m3 [n,k] row-major;  rhs_scales fp32 [ceil(n/128)][k/128] row-major
  *   out        bf16 [m,n] row-major
- * Requires k % 128 == 0, n % 4 == 0; m arbitrary. `num_sms` is the caller's compute-unit cap (the reference passes
- * it to its persistent kernel, yan/jit_kernels/gemm.py:26-30); this build launches one workgroup per tile and
- * accepts the argument for signature compatibility (tile choice uses it as the number of compute units when > 0).
+ * Requires k % 128 == 0, n % 4 == 0; m arbitrary; (m rounded up to the tile's rows, at most 256) * k < 2^31 bytes, same
+ * for n; 256 * n * 2 < 2^31 bytes; the last activation scale at an offset below 2^28 elements.
+ * `num_sms` is the caller's compute-unit cap, the grid size of the reference's persistent kernel
+ * (yan/include/gemm/fp8_gemm.cuh:40, yan/jit_kernels/gemm.py:26-30): 0, or a value of at least the device's compute
+ * units, starts one workgroup per output tile; a smaller value starts that many workgroups (rounded down to a
+ * multiple of 8 from 8 up), each walking several tiles, and is also the number of compute units the tile choice
+ * plans for. Results do not depend on it. The grouped entry points below take it in the same sense.
  * Nothing is allocated and no state is kept between calls.
  * Replaces the FP8 entry the reference only sketches: template yan/jit_kernels/gemm.py:9-31, kernel
  * yan/include/gemm/fp8_gemm.cuh:40-196. */
@@ -113,12 +119,15 @@ YAN_API int yan_gemm_select_tile(int op, int m, int n, int k, int num_cus, int* 
 YAN_API const char* yan_gemm_version(void);
 
 /* The JIT boundary, for reference: signatures of `launch` in the kernel.so of each op
- * (argument lists of yan/jit_kernels/cute_gemm.py:55-59 and yan/jit_kernels/gemm.py:23-30; the last two ints of
- * the FP8 form are this build's explicit activation-scale strides, in elements). */
+ * (argument lists of yan/jit_kernels/cute_gemm.py:55-59 and yan/jit_kernels/gemm.py:23-30). The FP8 form with the
+ * reference's nine arguments takes token-contiguous activation scales (element (i, kb) at kb * m + i); the strided form
+ * is this build's addition for every other layout, with the two strides in elements. */
 typedef void (*yan_jit_launch_dense_fn)(int m, int n, int k, void* A, void* B, void* C, void* stream, int* return_code);
 typedef void (*yan_jit_launch_fp8_fn)(void* lhs, void* lhs_scales, void* rhs, void* rhs_scales, void* out, int m,
-                                      void* stream, int num_sms, int smem_size, int lhs_scales_stride_m,
-                                      int lhs_scales_stride_k, int* return_code);
+                                      void* stream, int num_sms, int smem_size, int* return_code);
+typedef void (*yan_jit_launch_fp8_strided_fn)(void* lhs, void* lhs_scales, void* rhs, void* rhs_scales, void* out, int m,
+                                              void* stream, int num_sms, int smem_size, int lhs_scales_stride_m,
+                                              int lhs_scales_stride_k, int* return_code);
 
 #ifdef __cplusplus
 }

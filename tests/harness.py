@@ -1,4 +1,4 @@
-"""Harness-side helpers shared by tests, the smoke entry and the benchmark: FP8 quantisers in the DeepGEMM
+"""Harness-side helpers shared by the tests, the smoke entry and the benchmark (not part of the operator package): FP8 quantisers in the DeepGEMM
 convention and seeded constructors for the benchmark configurations. The reference defines neither (its FP8 path
 has no Python entry or test); the recipes are the ones the benchmark configurations name:
 per-token 1x128 / per-block 128x128 amax, clamp 1e-4, x * (448 / amax) -> e4m3fn, scale = amax / 448.
@@ -93,7 +93,7 @@ def make_fp8_case(m: int, n: int, k: int, seed: int = 42, dist: str = 'normal', 
     a8, sa = build(m, per_token_cast_to_fp8, 1)
     b8, sb = build(n, per_block_cast_to_fp8, 128)
     if col_major_scales:
-        from .jit_kernels.utils import get_col_major_tensor
+        from yan_amd.jit_kernels.utils import get_col_major_tensor
         sa = get_col_major_tensor(sa)
     return (a8, sa), (b8, sb), torch.zeros(m, n, dtype=torch.bfloat16, device=device)
 
@@ -101,22 +101,28 @@ def make_fp8_case(m: int, n: int, k: int, seed: int = 42, dist: str = 'normal', 
 def make_grouped_contiguous_case(group_rows, n: int, k: int, seed: int = 42, device='cpu', gen_device='cpu',
                                  padding_blocks: int = 0, alignment: int = 128):
     """((A8, sA), (B8 [G,n,k], sB [G,ceil(n/128),k/128]), out, m_indices) for the contiguous grouped layout:
-    group g contributes `group_rows[g]` real rows, padded with zero rows up to the alignment (padding rows carry
-    the group's index, as a caller that pads with zeros would do); `padding_blocks` whole blocks with index -1 follow.
+    the g-th positive entry of `group_rows` is group g and contributes that many real rows, padded with zero rows up to
+    the alignment (padding rows carry the group's index, as a caller that pads with zeros would do); a negative entry
+    is a block of that many padding rows (index -1, a multiple of the alignment) at that position; `padding_blocks`
+    whole blocks with index -1 follow at the end. Padding blocks hold random values, which the kernel must not touch.
     `out` is pre-filled with a sentinel so that rows the kernel must not write can be checked."""
-    groups = len(group_rows)
+    groups = sum(1 for r in group_rows if r > 0)
     gen = torch.Generator(device=gen_device).manual_seed(seed)
     qs, ss, idx = [], [], []
-    for g, rows in enumerate(group_rows):
-        padded = (rows + alignment - 1) // alignment * alignment
-        x = torch.zeros(padded, k, device=gen_device)
-        x[:rows] = torch.randn(rows, k, generator=gen, device=gen_device)
+    g = 0
+    for rows in tuple(group_rows) + ((-padding_blocks * alignment,) if padding_blocks else ()):
+        if rows > 0:
+            padded = (rows + alignment - 1) // alignment * alignment
+            x = torch.zeros(padded, k, device=gen_device)
+            x[:rows] = torch.randn(rows, k, generator=gen, device=gen_device)
+            label, g = g, g + 1
+        else:
+            padded = -rows
+            assert padded % alignment == 0
+            x = torch.randn(padded, k, generator=gen, device=gen_device)
+            label = -1
         q, sc = per_token_cast_to_fp8(x.to(device))
-        qs.append(q), ss.append(sc), idx.append(torch.full((padded,), g, dtype=torch.int32))
-    if padding_blocks:
-        rows = padding_blocks * alignment
-        q, sc = per_token_cast_to_fp8(torch.randn(rows, k, generator=gen, device=gen_device).to(device))
-        qs.append(q), ss.append(sc), idx.append(torch.full((rows,), -1, dtype=torch.int32))
+        qs.append(q), ss.append(sc), idx.append(torch.full((padded,), label, dtype=torch.int32))
     a8, sa = torch.cat(qs), torch.cat(ss)
     ws = [per_block_cast_to_fp8(torch.randn(n, k, generator=gen, device=gen_device).to(device)) for _ in range(groups)]
     b8, sb = torch.stack([w[0] for w in ws]), torch.stack([w[1] for w in ws])
@@ -174,7 +180,12 @@ FP8_TEST_SHAPES = [
 FP8_SIDE_SHAPES = [(1024, 4096, 7168), (8192, 4096, 7168), (200, 384, 512), (1152, 512, 512), (128, 4096, 1024), (128, 320, 384),
                    (256, 200, 128), (256, 512, 512)]
 # Grouped FP8 GEMMs: (rows per group, n, k, blocks of padding rows) and (groups, m_max, n, k, masked_m, expected_m).
+# Long groups on 256-row tiles whose two 128-row halves belong to different groups, or one of them to padding: a padding
+# block between the groups (negative entry) and one at the end; group 1 has 63 blocks, so it starts and the run ends on
+# odd multiples of 128. The test also runs the rows rotated by one block, which moves every boundary by 128 rows.
+GROUPED_TWO_PASS_CASE = ((8192, -128, 8064, 8192, 8192), 4096, 1024, 1)
 GROUPED_CONTIGUOUS_TEST_CASES = [
+    GROUPED_TWO_PASS_CASE,
     ((100, 128, 1, 300), 320, 384, 1), ((128, 128), 4096, 1024, 0), ((129,), 200, 128, 2),
     ((1024, 1024, 1024, 1024), 4096, 7168, 0), ((8192, 8192, 8192, 8192), 4096, 7168, 0),
     # long groups whose boundaries fall in the middle of 256-row tiles (two-pass tiles), with a trailing padding block
@@ -189,11 +200,19 @@ GROUPED_MASKED_TEST_CASES = [
 ]
 
 
+# Shapes run under a compute-unit cap (set_num_sms): the 256 x 256 tiles (two rounds of 64 workgroups) and ring tiles.
+NUM_SMS_CAP = 64
+CAPPED_SHAPES = [(2048, 4096, 1024), (512, 4096, 2048), (300, 2112, 640)]
+
+
+# Shapes run with empirical tile selection (YAN_TUNE_TILES=1): three candidate tiles each, for both GEMMs.
+TUNED_SHAPES = [(4096, 5120, 5120), (2048, 7168, 7168)]
+
+
 def jit_kernels_in_use(num_cus: int = 256):
-    """(name, arg_defs, code) of every distinct JIT kernel the shapes above, the quantisers and the probe select."""
-    from . import probe
-    from .jit import cpp_format, generate
-    from .jit_kernels import bf16_gemm, fp8_cast, gemm, m_grouped_gemm, simple_gemm
+    """(name, arg_defs, code) of every distinct JIT kernel the shapes above, and the quantisers select."""
+    from yan_amd.jit import cpp_format, generate
+    from yan_amd.jit_kernels import bf16_gemm, fp8_cast, gemm, m_grouped_gemm, simple_gemm
     kernels = {}
 
     def add(name, arg_defs, includes, code_template, keys):
@@ -209,18 +228,30 @@ def jit_kernels_in_use(num_cus: int = 256):
         name, keys, arg_defs = simple_gemm.float_kernel_plan(m, n, num_cus)
         add(name, arg_defs, simple_gemm.includes, simple_gemm.template, keys)
     for m, n, k in FP8_TEST_SHAPES + FP8_SIDE_SHAPES:
-        if m:
-            name, keys, arg_defs, _, code_template = gemm.fp8_kernel_plan(m, n, k, num_cus)
+        for token_contiguous in (True, False) if m else ():     # both layouts of the activation scales
+            name, keys, arg_defs, _, code_template = gemm.fp8_kernel_plan(m, n, k, num_cus, token_contiguous)
             add(name, arg_defs, gemm.includes, code_template, keys)
-    name, arg_defs, code = probe.probe_kernel()
-    kernels.setdefault((name, code), (name, arg_defs, code))
+    for m, n, k in CAPPED_SHAPES:
+        for cus, cap in ((num_cus, 0), (num_cus, NUM_SMS_CAP), (NUM_SMS_CAP, NUM_SMS_CAP)):
+            name, keys, arg_defs = bf16_gemm.dense_kernel_plan(m, n, k, torch.bfloat16, cus, cap)
+            add(name, arg_defs, bf16_gemm.includes, bf16_gemm.template, keys)
+        for cus in (num_cus, NUM_SMS_CAP):
+            name, keys, arg_defs, _, code_template = gemm.fp8_kernel_plan(m, n, k, cus, False)
+            add(name, arg_defs, gemm.includes, code_template, keys)
+    for m, n, k in TUNED_SHAPES:
+        name, keys, space, arg_defs = bf16_gemm.dense_tuning_plan(m, n, k, torch.bfloat16, num_cus)
+        for extra in space:
+            add(name, arg_defs, bf16_gemm.includes, bf16_gemm.template, {**keys, **extra})
+        name, keys, space, arg_defs, code_template = gemm.fp8_tuning_plan(m, n, k, num_cus, True)
+        for extra in space:
+            add(name, arg_defs, gemm.includes, code_template, {**keys, **extra})
     for kind in ('per_token', 'per_block'):
         for dtype in (torch.bfloat16, torch.float32):
             name, keys, arg_defs, code_template = fp8_cast.cast_kernel_plan(kind, dtype)
             add(name, arg_defs, fp8_cast.includes, code_template, keys)
     for rows, n, k, pad_blocks in GROUPED_CONTIGUOUS_TEST_CASES:
-        m = sum((r + 127) // 128 * 128 for r in rows) + 128 * pad_blocks
-        name, keys, arg_defs, _ = m_grouped_gemm.grouped_kernel_plan('GroupedContiguous', len(rows), m, n, k, num_cus)
+        m = sum((abs(r) + 127) // 128 * 128 for r in rows) + 128 * pad_blocks
+        name, keys, arg_defs, _ = m_grouped_gemm.grouped_kernel_plan('GroupedContiguous', sum(1 for r in rows if r > 0), m, n, k, num_cus)
         add(name, arg_defs, m_grouped_gemm.includes, m_grouped_gemm.template, keys)
     for groups, m_max, n, k, _, expected_m in GROUPED_MASKED_TEST_CASES:
         name, keys, arg_defs, _ = m_grouped_gemm.grouped_kernel_plan('GroupedMasked', groups, min(expected_m, m_max), n, k, num_cus)
@@ -233,7 +264,7 @@ def prebuild_jit_kernels(num_cus: int = 256, verbose: bool = False, jobs: int = 
     current kernel cache, `jobs` compilers at a time (default: one per CPU, at most 8). Returns the number of kernels."""
     import os
     from concurrent.futures import ThreadPoolExecutor
-    from .jit import build
+    from yan_amd.jit import build
     kernels = jit_kernels_in_use(num_cus)
     jobs = jobs or max(1, min(8, os.cpu_count() or 1))
 

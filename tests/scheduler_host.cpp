@@ -1,0 +1,66 @@
+// Host-side check of the workgroup -> tile mapping (gemm/scheduler.hpp is __host__ __device__): built and run by
+// tests/test_host_cpu.py with `hipcc --cuda-host-only`, no device involved.
+//
+// For a range of (tiles_m, tiles_n) it asserts that
+//   * tile_of over [0, grid_size()) visits every tile exactly once and marks the remaining slots invalid
+//     (reference: yan/include/gemm/scheduler.cuh:39-41, num_blocks = ceil(m/BLOCK_M) * ceil(N/BLOCK_N));
+//   * under every compute-unit cap, the walk b, b + grid, b + 2 grid, ... of capped_grid() workgroups covers every slot
+//     exactly once and, for grids that are multiples of 8, never leaves the XCD residue b % 8;
+//   * the 32 slots that the 8 XCDs run first (4 per XCD ... 32 per XCD) form compact patches: the slots one XCD owns are a
+//     contiguous range of the band-major sequence.
+#include "gemm/scheduler.hpp"
+
+#include <cstdio>
+#include <vector>
+
+#define CHECK(cond)                                                                                   \
+    do {                                                                                              \
+        if (!(cond)) {                                                                                \
+            std::printf("FAILED %s at %s:%d (m=%d n=%d bm=%d bn=%d)\n", #cond, __FILE__, __LINE__, m, n, bm, bn); \
+            return 1;                                                                                 \
+        }                                                                                             \
+    } while (0)
+
+int main() {
+    int cases = 0;
+    const int blocks[][2] = {{256, 256}, {128, 256}, {64, 16}, {256, 224}};
+    for (const auto& blk : blocks) {
+        const int bm = blk[0], bn = blk[1];
+        for (int tm = 1; tm <= 40; tm += (tm < 12 ? 1 : 7))
+            for (int tn = 1; tn <= 70; tn += (tn < 10 ? 1 : 9)) {
+                // ragged sizes: the last tile of each dimension holds a single row / column
+                const int m = (tm - 1) * bm + 1, n = (tn - 1) * bn + 1;
+                const yan::XcdTileScheduler<> sched(m, n, bm, bn);
+                CHECK(sched.tiles_m == tm && sched.tiles_n == tn && sched.total == tm * tn);
+                const int slots = sched.grid_size();
+                CHECK(slots >= sched.total && slots < sched.total + yan::kNumXCD && slots % yan::kNumXCD == 0);
+                std::vector<int> seen(size_t(tm) * tn, 0);
+                int invalid = 0;
+                for (int bid = 0; bid < slots; ++bid) {
+                    const yan::TileCoord t = sched.tile_of(bid);
+                    if (!t.valid) { ++invalid; continue; }
+                    CHECK(t.m_idx >= 0 && t.m_idx < tm && t.n_idx >= 0 && t.n_idx < tn);
+                    ++seen[size_t(t.m_idx) * tn + t.n_idx];
+                }
+                CHECK(invalid == slots - sched.total);
+                for (int v : seen) CHECK(v == 1);
+                // walks under a cap
+                for (int cap : {0, 1, 3, 8, 20, 64, 100, 255, 256, 300}) {
+                    const int grid = yan::capped_grid(slots, cap, 256);
+                    CHECK(grid >= 1 && grid <= slots);
+                    if (cap <= 0 || cap >= 256 || cap >= slots) CHECK(grid == slots);
+                    else CHECK(grid <= cap && (cap < yan::kNumXCD || grid % yan::kNumXCD == 0) && grid > cap - yan::kNumXCD);
+                    std::vector<int> hit(slots, 0);
+                    for (int b = 0; b < grid; ++b)
+                        for (int slot = b; slot < slots; slot += grid) {
+                            ++hit[slot];
+                            if (grid % yan::kNumXCD == 0) CHECK(slot % yan::kNumXCD == b % yan::kNumXCD);
+                        }
+                    for (int v : hit) CHECK(v == 1);
+                }
+                ++cases;
+            }
+    }
+    std::printf("ok %d\n", cases);
+    return 0;
+}

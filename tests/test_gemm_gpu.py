@@ -16,7 +16,8 @@ import torch
 
 import oracle
 import yan_amd as yan
-from yan_amd import capi, jit, testing
+import harness as testing
+from yan_amd import capi, jit
 
 pytestmark = pytest.mark.gpu
 
@@ -478,18 +479,93 @@ def test_fp8_outlier_16384_cubed():
     assert oracle.calc_diff(got, ref) < FP8_TOL
     assert oracle.calc_diff(got, ref) < 1e-5
     assert bool(torch.isfinite(out[::97].float()).all())
+    # the whole 16384 x 16384 output (4096 tiles) against a chunked fp32 matmul of the dequantised operands on the device:
+    # over everything, and slab by slab so that no band of tiles can hide behind the rest
+    wd = testing.dequant_rhs(b8, sb)
+    num = den = 0.0
+    for r0 in range(0, m, 1024):
+        ref = testing.dequant_lhs(a8[r0:r0 + 1024], sa[r0:r0 + 1024]) @ wd.t()
+        got = out[r0:r0 + 1024].float()
+        assert bool(torch.isfinite(got).all())
+        slab_num = (got.double() * ref.double()).sum().item()
+        slab_den = (got.double() ** 2 + ref.double() ** 2).sum().item()
+        assert 1 - 2 * slab_num / slab_den < 1e-4, r0
+        num, den = num + slab_num, den + slab_den
+    assert 1 - 2 * num / den < 1e-4
+
+
+# ----------------------------------------------------------------------------- the compute-unit cap (num_sms)
+def _event_ms(fn, reps):
+    fn()
+    torch.cuda.synchronize()
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(reps):
+        fn()
+    end.record()
+    end.synchronize()
+    return start.elapsed_time(end) / reps
+
+
+@pytest.mark.parametrize('m,n,k', testing.CAPPED_SHAPES)
+def test_num_sms_caps_the_workgroups_without_changing_a_bit(m, n, k):
+    """The reference's persistent kernels launch `num_sms` blocks (yan/include/gemm/fp8_gemm.cuh:40,
+    yan/jit_kernels/gemm.py:26-30, utils.py:6-29). Here a cap below the device's compute units launches that many
+    workgroups (a multiple of 8), each walking several tiles: same kernel, same tile, same bits as one workgroup per
+    tile; and through set_num_sms the public entries stay within tolerance of the oracle."""
+    from yan_amd.jit_kernels import bf16_gemm, gemm
+    _announce('num_sms cap', m, n, k)
+    cap, stream = testing.NUM_SMS_CAP, torch.cuda.current_stream()
+    full = yan.get_num_sms()
+    assert cap < full
+    (a8, sa), (b8, sb), out = testing.make_fp8_case(m, n, k, seed=21, device='cuda')
+    name, keys, defs, smem, tmpl = gemm.fp8_kernel_plan(m, n, k, full, False)
+    rt = jit.build(name, defs, jit.generate(gemm.includes, defs, jit.cpp_format(tmpl, keys)))
+    capped = torch.full_like(out, float('nan'))
+    assert rt(a8, sa, b8, sb, out, m, stream, full, smem, sa.stride(0), sa.stride(1)) == 0
+    assert rt(a8, sa, b8, sb, capped, m, stream, cap, smem, sa.stride(0), sa.stride(1)) == 0
+    assert torch.equal(capped, out)
+    assert oracle.calc_diff(_np(out), _fp8_ref(a8, sa, b8, sb)) < 1e-5
+    a, b, c = testing.make_bf16_case(m, n, k, seed=22, device='cuda')
+    results = []
+    for num_sms_cap in (0, cap):
+        name, dkeys, ddefs = bf16_gemm.dense_kernel_plan(m, n, k, torch.bfloat16, full, num_sms_cap)
+        drt = jit.build(name, ddefs, jit.generate(bf16_gemm.includes, ddefs, jit.cpp_format(bf16_gemm.template, dkeys)))
+        c = torch.full_like(c, float('nan'))
+        assert drt(m, n, k, a, b, c, stream) == 0
+        results.append(c)
+    assert torch.equal(results[0], results[1])
+    try:
+        yan.set_num_sms(cap)
+        assert yan.get_num_sms() == cap
+        out2, c2 = torch.full_like(out, float('nan')), torch.full_like(c, float('nan'))
+        yan.gemm_fp8_fp8_bf16_nt((a8, sa), (b8, sb), out2)
+        yan.gemm_bf16_tn(a, b, c2)
+        assert torch.equal(out2, out)                 # the block-scaled sum is formed in the same order by every tile
+        assert float(yan.calc_diff(c2.float(), a.float() @ b.float().t())) < BF16_TOL
+    finally:
+        yan.set_num_sms(full)
+
+
+def test_num_sms_cap_is_what_runs_at_the_headline_size():
+    """cfg3 under a cap of 64 of 256 compute units: identical bits, and two to four times the time, i.e. the cap is the
+    number of compute units that work (448 tiles: 7 rounds of 64 instead of 1.75 rounds of 256). Less than four times:
+    a quarter of the chip is not power-limited and each of its compute units runs a tile about a third faster."""
+    from yan_amd.jit_kernels import gemm
+    m, n, k = testing.BASELINE_FP8['cfg3']
+    _announce('num_sms cap at cfg3', m, n, k)
+    (a8, sa), (b8, sb), out = testing.make_fp8_case(m, n, k, seed=42, device='cuda', gen_device='cuda', col_major_scales=True)
+    full, stream = yan.get_num_sms(), torch.cuda.current_stream()
+    name, keys, defs, smem, tmpl = gemm.fp8_kernel_plan(m, n, k, full, True)
+    rt = jit.build(name, defs, jit.generate(gemm.includes, defs, jit.cpp_format(tmpl, keys)))
+    capped = torch.full_like(out, float('nan'))
+    t_full = _event_ms(lambda: rt(a8, sa, b8, sb, out, m, stream, full, smem), 20)
+    t_cap = _event_ms(lambda: rt(a8, sa, b8, sb, capped, m, stream, 64, smem), 10)
+    assert torch.equal(capped, out)
+    assert 1.7 * t_full < t_cap < 6.0 * t_full, (t_full, t_cap)
 
 
 # ----------------------------------------------------------------------------- the ahead-of-time C-ABI library
-def test_mfma_ceiling_probe_runs_and_stays_below_the_vendor_peak():
-    from yan_amd import probe
-    for kind, peak in (('bf16_32x32x16', 2520.0), ('bf16_16x16x32', 2520.0), ('fp8_16x16x128_accumulate', 5040.0),
-                       ('fp8_16x16x128_zero_c_plus_fold', 5040.0)):
-        zero = probe.mfma_ceiling(kind, 'zero', iters=1000, launches=5)
-        rand = probe.mfma_ceiling(kind, 'random', iters=1000, launches=5)
-        assert 0.3 * peak < rand <= zero * 1.05 and zero < peak * 1.02, (kind, rand, zero)
-
-
 def test_tuner_times_a_space_of_tiles_on_the_device():
     """The empirical half of compile_and_tune (yan/jit_kernels/tuner.py:24-69): every candidate of `space` is built, run
     once, timed over back-to-back launches after a cache flush, and the fastest is kept and memoised."""
@@ -499,7 +575,7 @@ def test_tuner_times_a_space_of_tiles_on_the_device():
     a, b, c = testing.make_bf16_case(m, n, k, seed=3, device='cuda')
     args = (m, n, k, a, b, c, torch.cuda.current_stream())
     from yan_amd.jit_kernels.heuristics import get_dense_num_stages
-    space = tuple({'BLOCK_M': bm, 'BLOCK_N': bn, 'NUM_STAGES': get_dense_num_stages(bm, bn)} for bm, bn in ((256, 256), (128, 128), (64, 64)))
+    space = tuple({'BLOCK_M': bm, 'BLOCK_N': bn, 'NUM_STAGES': get_dense_num_stages(bm, bn), 'NUM_SMS': 0} for bm, bn in ((256, 256), (128, 128), (64, 64)))
     tuner = JITTuner()
     kw = dict(name='gemm_bf16_tn', keys={}, space=space, includes=bf16_gemm.includes,
               arg_defs=bf16_gemm._arg_defs(torch.bfloat16), template=bf16_gemm.template, args=args)
@@ -510,6 +586,36 @@ def test_tuner_times_a_space_of_tiles_on_the_device():
     c.zero_()
     assert best(*args) == 0
     assert float(yan.calc_diff(c.float(), a.float() @ b.float().t())) < 1e-5
+
+
+@pytest.mark.parametrize('m,n,k', testing.TUNED_SHAPES)
+def test_entry_points_pick_the_fastest_of_three_tiles_when_asked(m, n, k, monkeypatch):
+    """With YAN_TUNE_TILES=1 the first call of a shape hands the cost model's three best tiles to the tuner
+    (yan/jit_kernels/cute_gemm.py:42-53, tuner.py:42-69); the winner is memoised per shape and the result is the same
+    GEMM."""
+    from yan_amd.jit_kernels import bf16_gemm, gemm
+    from yan_amd.jit_kernels.tuner import jit_tuner
+    _announce('tuned tiles', m, n, k)
+    monkeypatch.setenv('YAN_TUNE_TILES', '1')
+    a, b, c = testing.make_bf16_case(m, n, k, seed=5, scale=k ** -0.5, device='cuda', gen_device='cuda')
+    yan.gemm_bf16_tn(a, b, c)
+    name, keys, space, _ = bf16_gemm.dense_tuning_plan(m, n, k, torch.bfloat16, yan.get_num_sms(), 0)
+    chosen = jit_tuner.tuned_keys[(name, str({key: keys[key] for key in sorted(keys)}))]
+    assert chosen in list(space) and len(space) == 3
+    pick = torch.randperm(m, device='cuda')[:512]
+    assert float(yan.calc_diff(c[pick].float(), a[pick].float() @ b.float().t())) < BF16_TOL
+    (a8, sa), (b8, sb), out = testing.make_fp8_case(m, n, k, seed=6, device='cuda', gen_device='cuda', col_major_scales=True)
+    yan.gemm_fp8_fp8_bf16_nt((a8, sa), (b8, sb), out)
+    name, keys, space, _, _ = gemm.fp8_tuning_plan(m, n, k, yan.get_num_sms(), True)
+    chosen = jit_tuner.tuned_keys[(name, str({key: keys[key] for key in sorted(keys)}))]
+    assert chosen in list(space) and len(space) == 3
+    ref = testing.dequant_lhs(a8[pick], sa[pick]) @ testing.dequant_rhs(b8, sb).t()
+    assert float(yan.calc_diff(out[pick].float(), ref)) < 1e-5
+    # the tile the cost model alone would have picked gives the same bits (every tile sums the K blocks in the same order)
+    monkeypatch.setenv('YAN_TUNE_TILES', '0')
+    again = torch.zeros_like(out)
+    yan.gemm_fp8_fp8_bf16_nt((a8, sa), (b8, sb), again)
+    assert torch.equal(again, out)
 
 
 # ----------------------------------------------------------------------------- quantisers in front of the FP8 GEMM
@@ -620,6 +726,18 @@ def test_grouped_contiguous_parity(rows, n, k, pad_blocks):
     JIT kernel; a single group gives the bits of the plain GEMM."""
     (a8, sa), (b8, sb), out, idx = testing.make_grouped_contiguous_case(rows, n, k, seed=5, padding_blocks=pad_blocks)
     m = a8.size(0)
+    group_rows = [r for r in rows if r > 0]           # negative entries are padding blocks between groups
+    if rows == testing.GROUPED_TWO_PASS_CASE[0]:
+        # this case exists for the 256-row tile whose halves belong to different groups or to padding: make sure a
+        # change of the cost table cannot silently move it to another tile
+        from yan_amd.jit_kernels.m_grouped_gemm import grouped_kernel_plan
+        assert grouped_kernel_plan('GroupedContiguous', len(group_rows), m, n, k, 256)[1]['BLOCK_M'] == 256
+        blocks = idx.view(-1, 128)[:, 0]
+        # halves of the 256-row tiles, as laid out here and as rotated by one block further down
+        halves = torch.cat([b[:len(b) // 2 * 2].view(-1, 2) for b in (blocks, torch.roll(blocks, 1))])
+        assert bool(((halves[:, 0] != halves[:, 1]) & (halves >= 0).all(1)).any())      # two groups in one tile
+        assert bool(((halves[:, 0] < 0) & (halves[:, 1] >= 0)).any())                   # padding, then a group
+        assert bool(((halves[:, 0] >= 0) & (halves[:, 1] < 0)).any())                   # a group, then padding
     a8d, sad, b8d, sbd, idxd = a8.cuda(), sa.cuda(), b8.cuda(), sb.cuda(), idx.cuda()
     got = out.cuda()
     assert yan.m_grouped_gemm_fp8_fp8_bf16_nt_contiguous((a8d, sad), (b8d, sbd), got, idxd) is None
@@ -629,7 +747,7 @@ def test_grouped_contiguous_parity(rows, n, k, pad_blocks):
         ref = torch.from_numpy(ref)
     else:       # the per-group product on the device in fp32, rows of the oracle sampled below
         ref = out.float()
-        for g in range(len(rows)):
+        for g in range(len(group_rows)):
             sel = (idx == g).nonzero().flatten()
             ref[sel] = (testing.dequant_lhs(a8d[sel.cuda()], sad[sel.cuda()]) @ testing.dequant_rhs(b8d[g], sbd[g]).t()).cpu()
         pick = torch.arange(0, m, 97)
@@ -655,7 +773,7 @@ def test_grouped_contiguous_parity(rows, n, k, pad_blocks):
         yan.m_grouped_gemm_fp8_fp8_bf16_nt_contiguous((rolled[0], rolled[1]), (b8d, sbd), got2, rolled[2])
         assert torch.equal(torch.roll(got2, -128, 0), got)
     # the first group's rows through the plain entry point
-    r0 = (rows[0] + 127) // 128 * 128
+    r0 = (group_rows[0] + 127) // 128 * 128
     plain = torch.zeros(r0, n, dtype=torch.bfloat16, device='cuda')
     yan.gemm_fp8_fp8_bf16_nt((a8d[:r0], sad[:r0].contiguous()), (b8d[0], sbd[0]), plain)
     assert float(yan.calc_diff(plain.float(), got[:r0].float())) < 1e-9

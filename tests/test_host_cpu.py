@@ -1,5 +1,7 @@
 """Host-side logic that needs no device: helpers, tile heuristics, tuner selection rules, entry-point argument
 checks (reference: yan/jit_kernels/utils.py:32-85, yan/jit_kernels/tuner.py:12-78, yan/jit_kernels/cute_gemm.py:21-30)."""
+import os
+
 import pytest
 import torch
 
@@ -33,7 +35,7 @@ def test_tile_heuristics_fill_256_cus():
     assert bm == 64 and yan.ceil_div(4096, bn) >= 64
     # ... the decode shape runs the tiled kernel on 64 x 16 tiles with a deep ring of LDS stages, and up to 16 rows go
     # to the weight-streaming kernel (one workgroup per 16 weight rows) while those workgroups fit the chip at once
-    assert heuristics.get_fp8_tile(64, 4096, 7168, 256) == (64, 16) and heuristics.get_fp8_num_stages(64, 16) == 8
+    assert heuristics.get_fp8_tile(64, 4096, 7168, 256) == (64, 16) and heuristics.get_fp8_num_stages(64, 16) == 12
     assert heuristics.get_fp8_tile(1, 4096, 7168, 256) == (16, 16) and heuristics.get_fp8_tile(16, 2048, 7168, 256) == (16, 16)
     assert heuristics.get_skinny_fp8_config(17, 4096, 7168, 256) == 0 and heuristics.get_skinny_fp8_config(16, 7168, 7168, 256) == 0
     assert heuristics.get_fp8_num_stages(256, 256) == 2 and heuristics.get_dense_num_stages(256, 256) == 2
@@ -51,13 +53,20 @@ def test_tile_heuristics_fill_256_cus():
 
 def test_kernel_plans_keep_reference_keys_and_argument_order():
     name, keys, defs = bf16_gemm.dense_kernel_plan(4096, 7168, 2048, torch.bfloat16, 256)
-    assert name == 'gemm_bf16_tn' and sorted(keys) == ['BLOCK_M', 'BLOCK_N', 'NUM_STAGES']
+    assert name == 'gemm_bf16_tn' and sorted(keys) == ['BLOCK_M', 'BLOCK_N', 'NUM_SMS', 'NUM_STAGES'] and keys['NUM_SMS'] == 0
+    assert bf16_gemm.dense_kernel_plan(4096, 7168, 2048, torch.bfloat16, 64, 64)[1]['NUM_SMS'] == 64
     assert [d[0] for d in defs] == ['m', 'n', 'k', 'A', 'B', 'C', 'stream']
     assert bf16_gemm.dense_kernel_plan(4096, 7168, 2048, torch.half, 256)[0] == 'gemm_fp16_tn'
     name, keys, defs, smem, _ = gemm.fp8_kernel_plan(4096, 7168, 7168, 256)
     assert name == 'gemm_fp8_fp8_bf16_nt'
     assert sorted(keys) == ['BLOCK_M', 'BLOCK_N', 'K', 'N', 'NUM_STAGES', 'NUM_TMA_MULTICAST']
-    assert [d[0] for d in defs][:9] == ['lhs', 'lhs_scales', 'rhs', 'rhs_scales', 'out', 'm', 'stream', 'num_sms', 'smem_size']
+    # the reference's nine run-time names, exactly (yan/jit_kernels/gemm.py:23-30), for token-contiguous activation scales
+    assert [d[0] for d in defs] == ['lhs', 'lhs_scales', 'rhs', 'rhs_scales', 'out', 'm', 'stream', 'num_sms', 'smem_size']
+    assert defs is gemm.arg_defs and gemm.fp8_kernel_plan(4096, 7168, 7168, 256)[4] is gemm.template
+    # any other strided layout: the same, plus the two strides
+    strided = gemm.fp8_kernel_plan(4096, 7168, 7168, 256, False)
+    assert [d[0] for d in strided[2]] == [d[0] for d in defs] + ['lhs_scales_stride_m', 'lhs_scales_stride_k'] and strided[1] == keys
+    assert strided[0] == 'gemm_fp8_fp8_bf16_nt_strided'           # its own name: the tuner memoises per (name, keys)
     name, fkeys, defs = simple_gemm.float_kernel_plan(4096, 7168, 256)
     assert name == 'gemm_float_nt' and sorted(fkeys) == ['BLOCK_M', 'BLOCK_N']
     assert [d[0] for d in defs] == ['m', 'n', 'k', 'alpha', 'A', 'ldA', 'B', 'ldB', 'beta', 'C', 'ldC', 'stream']
@@ -145,3 +154,58 @@ def test_reference_package_name_is_an_alias():
     for name in ('gemm_fp16_tn', 'bench_kineto', 'get_col_major_tensor', 'calc_diff', 'jit', 'jit_kernels', 'gemm'):
         assert hasattr(by_reference_name, name), name
     assert callable(by_reference_name.jit_kernels.cute_gemm_accuracy_test)
+
+
+def test_tile_scheduler_visits_every_tile_once_and_walks_cover_every_slot(tmp_path, repo_root):
+    """XcdTileScheduler::tile_of and capped_grid are __host__ __device__: the checks live in tests/scheduler_host.cpp,
+    compiled for the host only."""
+    import subprocess
+    from yan_amd.jit.compiler import get_hipcc_compiler, get_jit_include_dir
+    exe = tmp_path / 'scheduler_host'
+    subprocess.check_call([get_hipcc_compiler()[0], '-x', 'hip', '--cuda-host-only', '-std=c++20', '-O1', f'-I{get_jit_include_dir()}',
+                           os.path.join(repo_root, 'tests', 'scheduler_host.cpp'), '-o', str(exe)])
+    done = subprocess.run([str(exe)], stdout=subprocess.PIPE, universal_newlines=True)
+    assert done.returncode == 0 and done.stdout.startswith('ok '), done.stdout
+    assert int(done.stdout.split()[1]) > 400
+
+
+def test_tuner_rebuilds_when_a_callers_dict_changes_between_calls(monkeypatch):
+    """A caller that reuses one mutable keys dict (the loop of the reference's tests/test_jit.py) gets the kernel of the
+    keys it passes, not of the keys it passed last time; only read-only plan keys take the same-object short cut."""
+    from yan_amd.jit_kernels import tuner as tuner_mod
+    built = []
+
+    def fake_build(name, arg_defs, code):
+        built.append(code)
+        return object()
+    monkeypatch.setattr(tuner_mod, 'build', fake_build)
+    t = tuner_mod.JITTuner()
+    kw = dict(name='k', space=(), includes=(), arg_defs=(('x', int),), template='int v = {V};', args=(1,))
+    keys = {'V': 1}
+    first = t.compile_and_tune(keys=keys, **kw)
+    assert t.compile_and_tune(keys=keys, **kw) is first and len(built) == 1
+    keys['V'] = 2
+    second = t.compile_and_tune(keys=keys, **kw)
+    assert second is not first and len(built) == 2 and 'int v = 2;' in built[1]
+    frozen = tuner_mod.FrozenKeys({'V': 1})
+    assert t.compile_and_tune(keys=frozen, **kw) is first and t.compile_and_tune(keys=frozen, **kw) is first
+    with pytest.raises(TypeError):
+        frozen['V'] = 3
+
+
+def test_compare_tensors_verdicts(capsys):
+    """yan/jit_kernels/utils.py:138-179: element-wise and similarity modes, shape mismatch, unknown mode."""
+    from yan_amd.jit_kernels import compare_tensors
+    x = torch.arange(12, dtype=torch.float32).view(3, 4)
+    assert compare_tensors(x, x.clone()) is True and compare_tensors(x, x.clone(), mode='similarity', verbose=False) is True
+    y = x.clone()
+    y[1, 2] += 0.5
+    capsys.readouterr()
+    assert compare_tensors(y, x, verbose=False) is False
+    said = capsys.readouterr().out
+    assert 'FAILED' in said and 'Max diff: 0.500000' in said and '[1, 2]' in said and 'Actual tensor' not in said
+    assert compare_tensors(y, x, atol=1.0) is True
+    assert compare_tensors(y, x, mode='similarity', diff_tolerance=1e-2) is True
+    assert compare_tensors(y, x, mode='similarity', diff_tolerance=1e-9) is False
+    assert compare_tensors(torch.zeros(3), torch.zeros(3), mode='similarity') is True
+    assert compare_tensors(x, x[:2]) is False and compare_tensors(x, x, mode='cosine') is False

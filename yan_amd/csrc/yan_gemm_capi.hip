@@ -99,7 +99,7 @@ int yan_gemm_fp8_fp8_bf16_nt(const void* lhs, const float* lhs_scales, long long
     // the kernel addresses the scale tensor with 32-bit byte offsets
     const long long last = (long long)(m - 1) * lhs_scales_stride_m + (long long)(k / 128 - 1) * lhs_scales_stride_k;
     if (lhs_scales_stride_m < 0 || lhs_scales_stride_k < 0 || last >= (1ll << 28)) return int(hipErrorInvalidValue);
-    const int cus = num_sms > 0 ? num_sms : device_cus();
+    const int cus = (num_sms > 0 && num_sms < device_cus()) ? num_sms : device_cus();
     hipStream_t s = static_cast<hipStream_t>(stream);
     __hip_bfloat16* o = static_cast<__hip_bfloat16*>(out);
     if (skinny_atoms(m, n, cus))
@@ -125,14 +125,14 @@ int yan_m_grouped_gemm_fp8_fp8_bf16_nt_contiguous(const void* lhs, const float* 
     if (m < 0 || n < 0 || k <= 0 || num_groups <= 0 || (m % 128) != 0) return int(hipErrorInvalidValue);
     const long long last = (long long)(m - 1) * lhs_scales_stride_m + (long long)(k / 128 - 1) * lhs_scales_stride_k;
     if (lhs_scales_stride_m < 0 || lhs_scales_stride_k < 0 || last >= (1ll << 28)) return int(hipErrorInvalidValue);
-    const int cus = num_sms > 0 ? num_sms : device_cus();
+    const int cus = (num_sms > 0 && num_sms < device_cus()) ? num_sms : device_cus();
     int bm = 0, bn = 0;
     pick_grouped(m, n, cus, 1, 128, num_groups, &bm, &bn);
 #define YAN_GROUPED_CASE(BM, BN)                                                                                     \
     if (bm == BM && bn == BN)                                                                                        \
         return int(yan::Gemm<0, 0, BM, BN, 128, 1, yan::Fp8TileConfig<BM, BN>::MAX_RING_STAGES, 1, yan::GemmType::GroupedContiguous>::run_grouped(             \
             static_cast<__hip_bfloat16*>(out), lhs, lhs_scales, int(lhs_scales_stride_m), int(lhs_scales_stride_k), 0, rhs, \
-            rhs_scales, m_indices, num_groups, m, n, k, static_cast<hipStream_t>(stream)));
+            rhs_scales, m_indices, num_groups, m, n, k, static_cast<hipStream_t>(stream), num_sms));
     YAN_GROUPED_CASE(256, 256) YAN_GROUPED_CASE(256, 128) YAN_GROUPED_CASE(128, 256) YAN_GROUPED_CASE(128, 128)
     YAN_GROUPED_CASE(64, 128) YAN_GROUPED_CASE(64, 64)
 #undef YAN_GROUPED_CASE
@@ -148,14 +148,14 @@ int yan_m_grouped_gemm_fp8_fp8_bf16_nt_masked(const void* lhs, const float* lhs_
     const long long last = (long long)(m_max - 1) * lhs_scales_stride_m + (long long)(k / 128 - 1) * lhs_scales_stride_k;
     if (lhs_scales_stride_m < 0 || lhs_scales_stride_k < 0 || lhs_scales_stride_g < 0 || last >= (1ll << 28) ||
         lhs_scales_stride_g >= (1ll << 31)) return int(hipErrorInvalidValue);
-    const int cus = num_sms > 0 ? num_sms : device_cus();
+    const int cus = (num_sms > 0 && num_sms < device_cus()) ? num_sms : device_cus();
     int bm = 0, bn = 0;
     pick_grouped(expected_m < m_max ? expected_m : m_max, n, cus, num_groups, 0, 1, &bm, &bn);
 #define YAN_GROUPED_CASE(BM, BN)                                                                                     \
     if (bm == BM && bn == BN)                                                                                        \
         return int(yan::Gemm<0, 0, BM, BN, 128, 1, yan::Fp8TileConfig<BM, BN>::MAX_RING_STAGES, 1, yan::GemmType::GroupedMasked>::run_grouped(                 \
             static_cast<__hip_bfloat16*>(out), lhs, lhs_scales, int(lhs_scales_stride_m), int(lhs_scales_stride_k),  \
-            int(lhs_scales_stride_g), rhs, rhs_scales, masked_m, num_groups, m_max, n, k, static_cast<hipStream_t>(stream)));
+            int(lhs_scales_stride_g), rhs, rhs_scales, masked_m, num_groups, m_max, n, k, static_cast<hipStream_t>(stream), num_sms));
     YAN_GROUPED_CASE(256, 256) YAN_GROUPED_CASE(256, 128) YAN_GROUPED_CASE(128, 256) YAN_GROUPED_CASE(128, 128)
     YAN_GROUPED_CASE(64, 128) YAN_GROUPED_CASE(64, 64)
 #undef YAN_GROUPED_CASE

@@ -50,13 +50,13 @@ struct DenseTileConfig {
 template <typename Atom, typename Elem, int BLOCK_M, int BLOCK_N, int STAGES>
 __device__ __forceinline__ void
 dense_gemm_body(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, Elem* __restrict__ C,
-                int m, int n, int k) {
+                int m, int n, int k, int bid) {
     using Cfg = DenseTileConfig<BLOCK_M, BLOCK_N>;
     constexpr int NW = Cfg::NUM_WAVES, TN = Cfg::WTN / 32, TM = Cfg::WTM / 32;
     static_assert(STAGES >= 3 && STAGES <= Cfg::MAX_STAGES, "a ring of three or more stages that fits the LDS");
 
     const XcdTileScheduler<> sched(m, n, BLOCK_M, BLOCK_N);
-    const TileCoord tile = sched.tile_of(blockIdx.x);
+    const TileCoord tile = sched.tile_of(bid);
     if (!tile.valid) return;
     const int m0 = tile.m_idx * BLOCK_M, n0 = tile.n_idx * BLOCK_N;
 
@@ -433,18 +433,30 @@ dense_gemm_mfma_8w(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
     dense_gemm_body_8w<Atom, Elem, BLOCK_M, BLOCK_N>(A, B, C, m, n, k);
 }
 
+// Workgroup b runs tiles b, b + gridDim.x, ...: exactly one when the launcher starts a workgroup per tile, several under
+// a compute-unit cap. Between two tiles every wave must have left the epilogue of the first, which reads an LDS stage
+// the second one's first copies go into.
+template <typename Atom, typename Elem, int BLOCK_M, int BLOCK_N, int STAGES>
+__device__ __forceinline__ void
+dense_gemm_walk(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, Elem* __restrict__ C, int m, int n, int k, int num_slots) {
+    for (int slot = blockIdx.x; slot < num_slots; slot += gridDim.x) {
+        dense_gemm_body<Atom, Elem, BLOCK_M, BLOCK_N, STAGES>(A, B, C, m, n, k, slot);
+        if (slot + int(gridDim.x) < num_slots) __syncthreads();
+    }
+}
+
 template <typename Atom, typename Elem, int BLOCK_M, int BLOCK_N, int STAGES>
 __global__ void __launch_bounds__(4 * kWaveSize)
-dense_gemm_mfma(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, Elem* __restrict__ C, int m, int n, int k) {
-    dense_gemm_body<Atom, Elem, BLOCK_M, BLOCK_N, STAGES>(A, B, C, m, n, k);
+dense_gemm_mfma(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, Elem* __restrict__ C, int m, int n, int k, int num_slots) {
+    dense_gemm_walk<Atom, Elem, BLOCK_M, BLOCK_N, STAGES>(A, B, C, m, n, k, num_slots);
 }
 
 // The fp16 flavour under the name of the reference's kernel (yan/include/gemm/cute_gemm.cuh:20), so that profiler
 // filters written for it (tests/test_cute.py:35 looks for 'fp16_gemm_cute') keep finding it.
 template <int BLOCK_M, int BLOCK_N, int STAGES>
 __global__ void __launch_bounds__(4 * kWaveSize)
-fp16_gemm_cute(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, _Float16* __restrict__ C, int m, int n, int k) {
-    dense_gemm_body<MfmaF16_32x32x16, _Float16, BLOCK_M, BLOCK_N, STAGES>(A, B, C, m, n, k);
+fp16_gemm_cute(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, _Float16* __restrict__ C, int m, int n, int k, int num_slots) {
+    dense_gemm_walk<MfmaF16_32x32x16, _Float16, BLOCK_M, BLOCK_N, STAGES>(A, B, C, m, n, k, num_slots);
 }
 
 template <int BLOCK_M, int BLOCK_N>
@@ -466,18 +478,21 @@ inline hipError_t check_dense_args(int m, int n, int k, const void* a, const voi
     return hipSuccess;
 }
 
+// `num_sms`: the caller's compute-unit cap (0 = none), see capped_grid in scheduler.hpp.
 template <typename Atom, typename Elem, int BLOCK_M, int BLOCK_N, int STAGES = DenseTileConfig<BLOCK_M, BLOCK_N>::MAX_STAGES>
-inline hipError_t launch_dense(int m, int n, int k, const void* a, const void* b, void* c, hipStream_t stream) {
+inline hipError_t launch_dense(int m, int n, int k, const void* a, const void* b, void* c, hipStream_t stream, int num_sms = 0) {
     if (m == 0 || n == 0) return hipSuccess;
     if (hipError_t e = check_dense_args(m, n, k, a, b, c, BLOCK_M, BLOCK_N); e != hipSuccess) return e;
     using Cfg = DenseTileConfig<BLOCK_M, BLOCK_N>;
     const XcdTileScheduler<> sched(m, n, BLOCK_M, BLOCK_N);
+    const int slots = sched.grid_size();
     if constexpr (BLOCK_M == 256 && BLOCK_N == 256 && STAGES == 2) {
         // The largest tile runs the 8-wave kernel on 16x16x32 atoms: level with the 4-wave one where the chip's power
         // limit sets the pace (8192^3), 13 % faster at 4096^3.
-        // persistent: one workgroup per CU (a multiple of the 8 XCDs, so a workgroup's tiles stay on one XCD's range)
+        // persistent: one workgroup per CU (a multiple of the 8 XCDs, so a workgroup's tiles stay on one XCD's range),
+        // or as many as the caller's cap allows
         const int cus = device_cu_count() / kNumXCD * kNumXCD;
-        const int grid = sched.grid_size() < cus ? sched.grid_size() : cus;
+        const int grid = capped_grid(slots < cus ? slots : cus, num_sms, device_cu_count());
         if constexpr (__is_same(Elem, _Float16))
             hipLaunchKernelGGL((fp16_gemm_cute_8w<BLOCK_M, BLOCK_N>), dim3(grid), dim3(8 * kWaveSize), 0, stream,
                                static_cast<const uint8_t*>(a), static_cast<const uint8_t*>(b), static_cast<Elem*>(c), m, n, k);
@@ -485,14 +500,17 @@ inline hipError_t launch_dense(int m, int n, int k, const void* a, const void* b
             hipLaunchKernelGGL((dense_gemm_mfma_8w<MfmaBF16_16x16x32, Elem, BLOCK_M, BLOCK_N>), dim3(grid),
                                dim3(8 * kWaveSize), 0, stream, static_cast<const uint8_t*>(a), static_cast<const uint8_t*>(b),
                                static_cast<Elem*>(c), m, n, k);
-    } else if constexpr (__is_same(Elem, _Float16))
-        hipLaunchKernelGGL((fp16_gemm_cute<BLOCK_M, BLOCK_N, STAGES>), dim3(sched.grid_size()),
-                           dim3(Cfg::NUM_WAVES * kWaveSize), 0, stream, static_cast<const uint8_t*>(a),
-                           static_cast<const uint8_t*>(b), static_cast<Elem*>(c), m, n, k);
-    else
-        hipLaunchKernelGGL((dense_gemm_mfma<Atom, Elem, BLOCK_M, BLOCK_N, STAGES>), dim3(sched.grid_size()),
-                           dim3(Cfg::NUM_WAVES * kWaveSize), 0, stream, static_cast<const uint8_t*>(a),
-                           static_cast<const uint8_t*>(b), static_cast<Elem*>(c), m, n, k);
+    } else {
+        const int grid = capped_grid(slots, num_sms, device_cu_count());
+        if constexpr (__is_same(Elem, _Float16))
+            hipLaunchKernelGGL((fp16_gemm_cute<BLOCK_M, BLOCK_N, STAGES>), dim3(grid),
+                               dim3(Cfg::NUM_WAVES * kWaveSize), 0, stream, static_cast<const uint8_t*>(a),
+                               static_cast<const uint8_t*>(b), static_cast<Elem*>(c), m, n, k, slots);
+        else
+            hipLaunchKernelGGL((dense_gemm_mfma<Atom, Elem, BLOCK_M, BLOCK_N, STAGES>), dim3(grid),
+                               dim3(Cfg::NUM_WAVES * kWaveSize), 0, stream, static_cast<const uint8_t*>(a),
+                               static_cast<const uint8_t*>(b), static_cast<Elem*>(c), m, n, k, slots);
+    }
     return hipGetLastError();
 }
 
@@ -502,12 +520,12 @@ inline hipError_t launch_dense(int m, int n, int k, const void* a, const void* b
 // 256x256x64 stages are 128 KB of the 160 KB, smaller tiles can hold a deeper ring).
 template <int BLOCK_M, int BLOCK_N, int NUM_STAGES>
 inline hipError_t gemm_tn(int m, int n, int k, const __hip_bfloat16* A, const __hip_bfloat16* B, __hip_bfloat16* C,
-                          hipStream_t stream) {
-    return yan::launch_dense<yan::MfmaBF16_32x32x16, __bf16, BLOCK_M, BLOCK_N, NUM_STAGES>(m, n, k, A, B, C, stream);
+                          hipStream_t stream, int num_sms = 0) {
+    return yan::launch_dense<yan::MfmaBF16_32x32x16, __bf16, BLOCK_M, BLOCK_N, NUM_STAGES>(m, n, k, A, B, C, stream, num_sms);
 }
 
 // fp16 in, fp32 accumulate, fp16 out.
 template <int BLOCK_M, int BLOCK_N, int NUM_STAGES>
-inline hipError_t gemm_tn(int m, int n, int k, const __half* A, const __half* B, __half* C, hipStream_t stream) {
-    return yan::launch_dense<yan::MfmaF16_32x32x16, _Float16, BLOCK_M, BLOCK_N, NUM_STAGES>(m, n, k, A, B, C, stream);
+inline hipError_t gemm_tn(int m, int n, int k, const __half* A, const __half* B, __half* C, hipStream_t stream, int num_sms = 0) {
+    return yan::launch_dense<yan::MfmaF16_32x32x16, _Float16, BLOCK_M, BLOCK_N, NUM_STAGES>(m, n, k, A, B, C, stream, num_sms);
 }

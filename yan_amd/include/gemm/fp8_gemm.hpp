@@ -56,7 +56,10 @@ struct Fp8TileConfig {
     static constexpr int  RING_SCALE_BYTES = ceil_div(BLOCK_M * 4, 1024) * 1024;
     static constexpr int  RING_STAGE_BYTES = (LDS_ROWS_A + LDS_ROWS_B) * kRowBytes + RING_SCALE_BYTES;
     static constexpr bool RING_CAPABLE = BLOCK_M % 64 == 0 && (BLOCK_M / 8) % NUM_WAVES == 0 && BLOCK_N % 16 == 0;
-    static constexpr int  MAX_RING_STAGES = RING_CAPABLE ? (160 * 1024 / RING_STAGE_BYTES < 8 ? 160 * 1024 / RING_STAGE_BYTES : 8) : 2;
+    // At most 8 stages, 12 for the narrow tiles of the decode shapes: those stream 16 or 32 weight rows per workgroup, are
+    // bound by the latency of their loads and gain from every k-tile more in flight (a stage is only 13 KB there).
+    static constexpr int  RING_DEPTH_CAP = BLOCK_N <= 32 ? 12 : 8;
+    static constexpr int  MAX_RING_STAGES = RING_CAPABLE ? (160 * 1024 / RING_STAGE_BYTES < RING_DEPTH_CAP ? 160 * 1024 / RING_STAGE_BYTES : RING_DEPTH_CAP) : 2;
 };
 
 // Normal:            lhs [m, K], rhs [N, K], out [m, N]; grouped_layout unused.
@@ -67,12 +70,13 @@ struct Fp8TileConfig {
 //                    are computed; lhs_scales of group g start at g * sa_stride_g floats. The grid is G times the
 //                    grid of one [m, N] problem.
 // STAGES: 2 = two LDS stages with the next k-tile's scales in registers; 3.. = a ring of that many stages.
-template <int SHAPE_N, int SHAPE_K, int BLOCK_M, int BLOCK_N, GemmType kGemmType = GemmType::Normal, int STAGES = 2>
-__global__ void __launch_bounds__((get_num_waves(BLOCK_M, BLOCK_N) * kWaveSize))
-fp8_gemm_kernel(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_scales,
-                const uint8_t* __restrict__ rhs, const float* __restrict__ rhs_scales,
-                __bf16* __restrict__ out, int m, int n_rt, int k_rt, int sa_stride_m, int sa_stride_k,
-                const int* __restrict__ grouped_layout = nullptr, int sa_stride_g = 0) {
+// One output tile (one slot of the launch: `bid` is what blockIdx.x would be with a workgroup per slot).
+template <int SHAPE_N, int SHAPE_K, int BLOCK_M, int BLOCK_N, GemmType kGemmType, int STAGES>
+__device__ __forceinline__ void
+fp8_gemm_tile(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_scales,
+              const uint8_t* __restrict__ rhs, const float* __restrict__ rhs_scales,
+              __bf16* __restrict__ out, int m, int n_rt, int k_rt, int sa_stride_m, int sa_stride_k,
+              const int* __restrict__ grouped_layout, int sa_stride_g, int bid, int num_slots) {
     using Cfg  = Fp8TileConfig<BLOCK_M, BLOCK_N>;
     using Atom = MfmaFP8_16x16x128;
     constexpr int NW = Cfg::NUM_WAVES, TN = Cfg::WTN / 16, TM = Cfg::WTM / 16;
@@ -85,7 +89,6 @@ fp8_gemm_kernel(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_s
     static_assert(STAGES == 2 || (STAGES >= 3 && STAGES <= Cfg::MAX_RING_STAGES), "no ring of this depth for this tile");
 
     const XcdTileScheduler<> sched(m, N, BLOCK_M, BLOCK_N);
-    int bid = blockIdx.x;
     if constexpr (kGemmType == GemmType::GroupedMasked) {
         const int group = bid / sched.grid_size();
         bid -= group * sched.grid_size();
@@ -343,7 +346,7 @@ fp8_gemm_kernel(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_s
     // the operand panels the other workgroups of the XCD are about to read.
     bool staged = false;
     if constexpr (kStagedEpilogue) staged = (N % 8) == 0;
-    const bool stream_out = size_t(m) * N * 2 * (kGemmType == GemmType::GroupedMasked ? gridDim.x / sched.grid_size() : 1) > (size_t(32) << 20);
+    const bool stream_out = size_t(m) * N * 2 * (kGemmType == GemmType::GroupedMasked ? num_slots / sched.grid_size() : 1) > (size_t(32) << 20);
     const __amdgpu_buffer_rsrc_t rsrc_out = make_out_rsrc(out + size_t(m0) * N + n0);
     if (staged) {
         if constexpr (kStagedEpilogue) {
@@ -396,11 +399,30 @@ fp8_gemm_kernel(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_s
     }   // pass
 }
 
+// Workgroup b runs slots b, b + gridDim.x, ...: exactly one when the launcher starts a workgroup per slot, a walk over
+// several when the caller caps the number of compute units (the reference's persistent kernel under `num_sms`,
+// yan/include/gemm/fp8_gemm.cuh:40, scheduler.cuh:39-58). Between two tiles every wave must have left the epilogue of
+// the first (which reads the LDS stage the second one's first copies go into).
+template <int SHAPE_N, int SHAPE_K, int BLOCK_M, int BLOCK_N, GemmType kGemmType = GemmType::Normal, int STAGES = 2>
+__global__ void __launch_bounds__((get_num_waves(BLOCK_M, BLOCK_N) * kWaveSize))
+fp8_gemm_kernel(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_scales,
+                const uint8_t* __restrict__ rhs, const float* __restrict__ rhs_scales,
+                __bf16* __restrict__ out, int m, int n_rt, int k_rt, int sa_stride_m, int sa_stride_k,
+                const int* __restrict__ grouped_layout, int sa_stride_g, int num_slots) {
+    for (int slot = blockIdx.x; slot < num_slots; slot += gridDim.x) {
+        fp8_gemm_tile<SHAPE_N, SHAPE_K, BLOCK_M, BLOCK_N, kGemmType, STAGES>(lhs, lhs_scales, rhs, rhs_scales, out, m, n_rt, k_rt,
+                                                                             sa_stride_m, sa_stride_k, grouped_layout, sa_stride_g,
+                                                                             slot, num_slots);
+        if (slot + int(gridDim.x) < num_slots) __syncthreads();
+    }
+}
+
 // Host side of the kernel, shaped after the class the reference's JIT template instantiates
 // (yan/jit_kernels/gemm.py:20-30: Gemm<N, K, BLOCK_M, BLOCK_N, 128, 1, kNumStages, kNumTMAMulticast, Normal>::run).
 // BLOCK_K is fixed at 128. kNumStages is the number of LDS stages: 2, or a ring of 3 .. Fp8TileConfig::MAX_RING_STAGES
 // for the small tiles that support one. kNumTMAMulticast is accepted and unused (gfx950 has no multicast copy), as
-// are `num_sms` and `smem_size` (one workgroup per tile, static LDS).
+// is `smem_size` (static LDS). `num_sms` caps the number of workgroups, as it sizes the reference's persistent grid
+// (capped_grid in scheduler.hpp).
 template <uint32_t SHAPE_N, uint32_t SHAPE_K, uint32_t BLOCK_M, uint32_t BLOCK_N, uint32_t BLOCK_K,
           uint32_t kNumGroups, uint32_t kNumStages, uint32_t kNumTMAMulticast, GemmType kGemmType>
 class Gemm {
@@ -424,7 +446,8 @@ public:
     // ints; `lhs_scales_stride_g` is used by the masked layout only. n and k as in run_sized.
     static hipError_t run_grouped(__hip_bfloat16* out, const void* lhs, const float* lhs_scales, int lhs_scales_stride_m,
                                   int lhs_scales_stride_k, int lhs_scales_stride_g, const void* rhs, const float* rhs_scales,
-                                  const int* grouped_layout, int num_groups, int m, int n, int k, hipStream_t stream) {
+                                  const int* grouped_layout, int num_groups, int m, int n, int k, hipStream_t stream,
+                                  int num_sms = 0) {
         static_assert(kGemmType != GemmType::Normal);
         if (m == 0 || n == 0 || num_groups == 0) return hipSuccess;
         if (m < 0 || n < 0 || k <= 0 || num_groups < 0 || (n % 4) != 0 || (k % 128) != 0) return hipErrorInvalidValue;
@@ -437,12 +460,13 @@ public:
         if (uint64_t(BLOCK_M) * n * 2 >= kOutOfRange) return hipErrorInvalidValue;
         using Cfg = Fp8TileConfig<BLOCK_M, BLOCK_N>;
         const XcdTileScheduler<> sched(m, n, BLOCK_M, BLOCK_N);
-        const uint64_t grid = uint64_t(sched.grid_size()) * (kGemmType == GemmType::GroupedMasked ? num_groups : 1);
-        if (grid >= kOutOfRange) return hipErrorInvalidValue;
-        hipLaunchKernelGGL((fp8_gemm_kernel<SHAPE_N, SHAPE_K, BLOCK_M, BLOCK_N, kGemmType, int(kNumStages)>), dim3(uint32_t(grid)),
+        const uint64_t slots = uint64_t(sched.grid_size()) * (kGemmType == GemmType::GroupedMasked ? num_groups : 1);
+        if (slots >= kOutOfRange) return hipErrorInvalidValue;
+        const int grid = capped_grid(int(slots), num_sms, device_cu_count());
+        hipLaunchKernelGGL((fp8_gemm_kernel<SHAPE_N, SHAPE_K, BLOCK_M, BLOCK_N, kGemmType, int(kNumStages)>), dim3(grid),
                            dim3(Cfg::NUM_WAVES * kWaveSize), 0, stream, static_cast<const uint8_t*>(lhs), lhs_scales,
                            static_cast<const uint8_t*>(rhs), rhs_scales, reinterpret_cast<__bf16*>(out), m, n, k,
-                           lhs_scales_stride_m, lhs_scales_stride_k, grouped_layout, lhs_scales_stride_g);
+                           lhs_scales_stride_m, lhs_scales_stride_k, grouped_layout, lhs_scales_stride_g, int(slots));
         return hipGetLastError();
     }
 
@@ -450,7 +474,7 @@ public:
     static hipError_t run_sized(__hip_bfloat16* out, const void* lhs, const float* lhs_scales, int lhs_scales_stride_m,
                                 int lhs_scales_stride_k, const void* rhs, const float* rhs_scales, int m, int n, int k,
                                 hipStream_t stream, int num_sms, uint32_t smem_size) {
-        (void)num_sms, (void)smem_size;
+        (void)smem_size;
         if (m == 0 || n == 0) return hipSuccess;
         if (m < 0 || n < 0 || k <= 0 || (n % 4) != 0 || (k % 128) != 0) return hipErrorInvalidValue;
         if ((SHAPE_N && n != int(SHAPE_N)) || (SHAPE_K && k != int(SHAPE_K))) return hipErrorInvalidValue;
@@ -462,10 +486,11 @@ public:
         if (uint64_t(BLOCK_M) * n * 2 >= kOutOfRange) return hipErrorInvalidValue;
         using Cfg = Fp8TileConfig<BLOCK_M, BLOCK_N>;
         const XcdTileScheduler<> sched(m, n, BLOCK_M, BLOCK_N);
-        hipLaunchKernelGGL((fp8_gemm_kernel<SHAPE_N, SHAPE_K, BLOCK_M, BLOCK_N, GemmType::Normal, int(kNumStages)>), dim3(sched.grid_size()),
+        const int slots = sched.grid_size(), grid = capped_grid(slots, num_sms, device_cu_count());
+        hipLaunchKernelGGL((fp8_gemm_kernel<SHAPE_N, SHAPE_K, BLOCK_M, BLOCK_N, GemmType::Normal, int(kNumStages)>), dim3(grid),
                            dim3(Cfg::NUM_WAVES * kWaveSize), 0, stream, static_cast<const uint8_t*>(lhs), lhs_scales,
                            static_cast<const uint8_t*>(rhs), rhs_scales, reinterpret_cast<__bf16*>(out), m, n, k,
-                           lhs_scales_stride_m, lhs_scales_stride_k);
+                           lhs_scales_stride_m, lhs_scales_stride_k, static_cast<const int*>(nullptr), 0, slots);
         return hipGetLastError();
     }
 };

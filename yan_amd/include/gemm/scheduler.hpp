@@ -44,4 +44,15 @@ struct XcdTileScheduler {
     }
 };
 
+// Workgroups to launch for `slots` units of work (tiles, or groups x tiles) under the caller's compute-unit cap, the
+// `num_sms` of the reference's persistent kernels (yan/include/gemm/fp8_gemm.cuh:40 launches num_sms blocks,
+// yan/jit_kernels/utils.py:6-29 holds the cap). No cap (0, or at least `device_cus`): one workgroup per slot, and the
+// hardware hands them to compute units as they free up. A cap below the device's compute units: that many workgroups,
+// rounded down to a multiple of the 8 XCDs so that slot b, b + grid, b + 2 grid, ... all fall to the same XCD and the
+// scheduler's per-XCD ranges keep their meaning; workgroup b then walks those slots.
+__host__ __device__ inline int capped_grid(int slots, int num_sms, int device_cus) {
+    if (num_sms <= 0 || num_sms >= device_cus || num_sms >= slots) return slots;
+    return num_sms >= kNumXCD ? num_sms / kNumXCD * kNumXCD : num_sms;
+}
+
 } // namespace yan

@@ -4,5 +4,6 @@ from .gemm import gemm_fp8_fp8_bf16_nt
 from .simple_gemm import gemm_float_nt, accuracy_test as simple_gemm_accuracy_test
 from .m_grouped_gemm import m_grouped_gemm_fp8_fp8_bf16_nt_contiguous, m_grouped_gemm_fp8_fp8_bf16_nt_masked
 from .fp8_cast import per_token_cast_to_fp8, per_block_cast_to_fp8
-from .utils import ceil_div, set_num_sms, get_num_sms, get_col_major_tensor, get_m_alignment_for_contiguous_layout
+from .utils import (ceil_div, set_num_sms, get_num_sms, get_col_major_tensor, get_m_alignment_for_contiguous_layout,
+                    compare_tensors)
 from .tuner import jit_tuner

@@ -4,15 +4,17 @@ Same contract as the reference's `gemm_fp16_tn` (`yan/jit_kernels/cute_gemm.py:2
 `[n,k]`, `c` is `[m,n]`, all row-major on the current device; the call is asynchronous on the current stream;
 `m == 0` or `n == 0` returns at once. The reference only has the fp16 flavour and accumulates in fp16; here both
 bf16 and fp16 exist and both accumulate in fp32. Keys and argument order of the JIT kernel are the reference's:
-keys `BLOCK_M, BLOCK_N, NUM_STAGES`, args `(m, n, k, A, B, C, stream)`.
+keys `BLOCK_M, BLOCK_N, NUM_STAGES`, args `(m, n, k, A, B, C, stream)`. The reference's dense kernel is not persistent and
+knows no `num_sms`; here a cap set with `set_num_sms` below the device's compute units becomes one more key, `NUM_SMS`
+(0 without a cap), so that the argument list stays the reference's.
 """
 import functools
 
 import torch
 
-from .heuristics import get_best_dense_config, get_dense_num_stages
-from .tuner import jit_tuner
-from .utils import get_num_sms
+from .heuristics import get_best_dense_config, get_dense_num_stages, get_dense_tile_space, tuning_enabled
+from .tuner import FrozenKeys, jit_tuner
+from .utils import get_num_sms, get_num_sms_cap
 
 includes = ('"gemm/bf16_gemm.hpp"', )
 template = """
@@ -20,8 +22,9 @@ template = """
 constexpr auto BLOCK_M = {BLOCK_M};
 constexpr auto BLOCK_N = {BLOCK_N};
 constexpr auto kNumStages = {NUM_STAGES};
+constexpr auto kNumSMs = {NUM_SMS};
 
-__return_code = static_cast<int>(gemm_tn<BLOCK_M, BLOCK_N, kNumStages>(m, n, k, A, B, C, stream));
+__return_code = static_cast<int>(gemm_tn<BLOCK_M, BLOCK_N, kNumStages>(m, n, k, A, B, C, stream, kNumSMs));
 """
 
 
@@ -30,11 +33,23 @@ def _arg_defs(dtype: torch.dtype):
 
 
 @functools.lru_cache(maxsize=None)
-def dense_kernel_plan(m: int, n: int, k: int, dtype: torch.dtype, num_cus: int):
-    """(name, keys, arg_defs) of the JIT kernel a call with these sizes uses; needs no GPU."""
+def dense_kernel_plan(m: int, n: int, k: int, dtype: torch.dtype, num_cus: int, num_sms_cap: int = 0):
+    """(name, keys, arg_defs) of the JIT kernel a call with these sizes uses; needs no GPU. `num_cus` steers the tile
+    choice, `num_sms_cap` (0 = none) is the number of workgroups the launch may start."""
     block_m, block_n = get_best_dense_config(m, n, k, num_cus)
     name = 'gemm_bf16_tn' if dtype == torch.bfloat16 else 'gemm_fp16_tn'
-    return name, {'BLOCK_M': block_m, 'BLOCK_N': block_n, 'NUM_STAGES': get_dense_num_stages(block_m, block_n)}, _arg_defs(dtype)
+    keys = FrozenKeys({'BLOCK_M': block_m, 'BLOCK_N': block_n, 'NUM_STAGES': get_dense_num_stages(block_m, block_n), 'NUM_SMS': num_sms_cap})
+    return name, keys, _arg_defs(dtype)
+
+
+@functools.lru_cache(maxsize=None)
+def dense_tuning_plan(m: int, n: int, k: int, dtype: torch.dtype, num_cus: int, num_sms_cap: int = 0):
+    """(name, keys, space, arg_defs) for empirical tile selection: the shape is the tuner's memo key and the cost
+    model's three best tiles are its candidates."""
+    name = 'gemm_bf16_tn' if dtype == torch.bfloat16 else 'gemm_fp16_tn'
+    space = tuple({'BLOCK_M': bm, 'BLOCK_N': bn, 'NUM_STAGES': get_dense_num_stages(bm, bn)}
+                  for bm, bn in get_dense_tile_space(m, n, k, num_cus))
+    return name, FrozenKeys({'M': m, 'N': n, 'K': k, 'NUM_SMS': num_sms_cap}), space, _arg_defs(dtype)
 
 
 def _gemm_16bit_tn(a: torch.Tensor, b: torch.Tensor, c: torch.Tensor, dtype: torch.dtype) -> None:
@@ -50,8 +65,11 @@ def _gemm_16bit_tn(a: torch.Tensor, b: torch.Tensor, c: torch.Tensor, dtype: tor
 
     stream = torch.cuda.current_stream()
     args = (m, n, k, a, b, c, stream)
-    name, keys, arg_defs = dense_kernel_plan(m, n, k, dtype, get_num_sms())
-    runtime = jit_tuner.compile_and_tune(name=name, keys=keys, space=(), includes=includes,
+    if tuning_enabled():
+        name, keys, space, arg_defs = dense_tuning_plan(m, n, k, dtype, get_num_sms(), get_num_sms_cap())
+    else:
+        (name, keys, arg_defs), space = dense_kernel_plan(m, n, k, dtype, get_num_sms(), get_num_sms_cap()), ()
+    runtime = jit_tuner.compile_and_tune(name=name, keys=keys, space=space, includes=includes,
                                          arg_defs=arg_defs, template=template, args=args)
     rc = runtime(*args)
     assert rc == 0, f'{name} failed with HIP error {rc}'

@@ -13,7 +13,7 @@ from typing import Tuple
 
 import torch
 
-from .tuner import jit_tuner
+from .tuner import FrozenKeys, jit_tuner
 from .utils import ceil_div
 
 includes = ('"gemm/fp8_cast.hpp"', )
@@ -49,7 +49,7 @@ def per_block_arg_defs(dtype: torch.dtype):
 @functools.lru_cache(maxsize=None)
 def cast_kernel_plan(kind: str, dtype: torch.dtype):
     """(name, keys, arg_defs, template) of the JIT kernel behind a quantiser; needs no GPU."""
-    keys = {'SRC': _src_name(dtype)}
+    keys = FrozenKeys({'SRC': _src_name(dtype)})
     if kind == 'per_token':
         return 'per_token_cast_to_fp8', keys, per_token_arg_defs(dtype), per_token_template
     assert kind == 'per_block'

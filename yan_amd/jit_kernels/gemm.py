@@ -2,9 +2,10 @@
 
 The reference ships only the JIT template of this op (`yan/jit_kernels/gemm.py:8-31`: keys `N, K, BLOCK_M,
 BLOCK_N, NUM_STAGES, NUM_TMA_MULTICAST`; run-time names `lhs, lhs_scales, rhs, rhs_scales, out, m, stream,
-num_sms, smem_size`) and no Python entry. The template below keeps those keys and names; TMA descriptors have no
-gfx950 counterpart, so the operands go to `Gemm::run` as plain pointers and the strides of the activation scales
-are passed explicitly, which lets the kernel read them row-major or token-contiguous without a transposing copy.
+num_sms, smem_size`) and no Python entry. `template` and `arg_defs` below keep exactly those keys and names; TMA
+descriptors have no gfx950 counterpart, so the operands go to `Gemm::run` as plain pointers. Activation scales that are
+not token-contiguous (row-major, say) run through `strided_template`, which takes their two strides as extra arguments,
+so no layout needs a transposing copy.
 
     out[i, j] = bf16( sum_kb lhs_scales[i, kb] * rhs_scales[j // 128, kb]
                               * sum_{t < 128} f32(lhs[i, 128 kb + t]) * f32(rhs[j, 128 kb + t]) )
@@ -14,13 +15,14 @@ from typing import Tuple
 
 import torch
 
-from .heuristics import get_best_fp8_config, get_fp8_num_stages, get_skinny_fp8_config
-from .tuner import jit_tuner
+from .heuristics import get_best_fp8_config, get_fp8_num_stages, get_fp8_tile_space, get_skinny_fp8_config, tuning_enabled
+from .tuner import FrozenKeys, jit_tuner
 from .utils import get_num_sms, ceil_div, get_col_major_tensor
 
 # C++ code templates
 includes = ('"gemm/fp8_gemm.hpp"', '"gemm/fp8_gemm_skinny.hpp"')
-template = """
+
+_keys_block = """
 using namespace yan;
 
 // Templated args from Python JIT call
@@ -29,7 +31,13 @@ constexpr auto BLOCK_M = {BLOCK_M};
 constexpr auto BLOCK_N = {BLOCK_N};
 constexpr auto kNumStages = {NUM_STAGES};
 constexpr auto kNumTMAMulticast = {NUM_TMA_MULTICAST};
-
+"""
+# Activation scales as DeepGEMM-style callers hand them over (`get_col_major_tensor`): element (i, kb) at kb * m + i.
+_token_contiguous_scales = """
+// Token-contiguous activation scales
+const int lhs_scales_stride_m = 1, lhs_scales_stride_k = m;
+"""
+_tiled_launch = """
 // Make a templated GEMM
 using GemmType = Gemm<N, K, BLOCK_M, BLOCK_N, 128, 1, kNumStages, kNumTMAMulticast, GemmType::Normal>;
 
@@ -37,45 +45,62 @@ using GemmType = Gemm<N, K, BLOCK_M, BLOCK_N, 128, 1, kNumStages, kNumTMAMultica
 __return_code = static_cast<int>(GemmType::run(out, lhs, lhs_scales, lhs_scales_stride_m, lhs_scales_stride_k,
                                                rhs, rhs_scales, m, stream, num_sms, smem_size));
 """
-
 # A handful of activation rows: BLOCK_M / 16 activation atoms and 16 weight rows per workgroup, the K blocks of a
 # workgroup shared out over NUM_WAVES waves; no LDS staging, NUM_STAGES is the per-wave load depth's name only.
-skinny_template = """
-using namespace yan;
-
-// Templated args from Python JIT call
-constexpr auto N = {N}, K = {K};
-constexpr auto BLOCK_M = {BLOCK_M};
-constexpr auto BLOCK_N = {BLOCK_N};
-constexpr auto kNumStages = {NUM_STAGES};
-constexpr auto kNumTMAMulticast = {NUM_TMA_MULTICAST};
-static_assert(BLOCK_N == 16 && BLOCK_M % 16 == 0);
+_skinny_launch = """static_assert(BLOCK_N == 16 && BLOCK_M % 16 == 0);
 
 // Launch kernel
 __return_code = static_cast<int>(launch_fp8_skinny<N, K, BLOCK_M / 16, {NUM_WAVES}>(
     out, lhs, lhs_scales, lhs_scales_stride_m, lhs_scales_stride_k, rhs, rhs_scales, m, N, K, stream));
 """
 
+# The reference's keys and run-time names, nothing else (yan/jit_kernels/gemm.py:9-30): code that formats this template
+# with `N, K, BLOCK_M, BLOCK_N, NUM_STAGES, NUM_TMA_MULTICAST` and builds it with `arg_defs` gets the kernel for
+# token-contiguous activation scales.
+template = _keys_block + _token_contiguous_scales + _tiled_launch
 arg_defs = (('lhs', torch.float8_e4m3fn), ('lhs_scales', torch.float),
             ('rhs', torch.float8_e4m3fn), ('rhs_scales', torch.float),
             ('out', torch.bfloat16), ('m', int),
-            ('stream', torch.cuda.Stream), ('num_sms', int), ('smem_size', int),
-            ('lhs_scales_stride_m', int), ('lhs_scales_stride_k', int))
+            ('stream', torch.cuda.Stream), ('num_sms', int), ('smem_size', int))
+# Any other strided layout of the activation scales (row-major included) runs without a transposing copy: the same
+# kernels with the two strides, in elements, as two more run-time arguments.
+strided_template = _keys_block + _tiled_launch
+strided_arg_defs = arg_defs + (('lhs_scales_stride_m', int), ('lhs_scales_stride_k', int))
+skinny_template = _keys_block + _token_contiguous_scales + _skinny_launch
+skinny_strided_template = _keys_block + _skinny_launch
 
 
 @functools.lru_cache(maxsize=None)
-def fp8_kernel_plan(m: int, n: int, k: int, num_cus: int):
+def fp8_kernel_plan(m: int, n: int, k: int, num_cus: int, token_contiguous_scales: bool = True):
     """(name, keys, arg_defs, smem_size, template) of the JIT kernel a call with these sizes uses; needs no GPU."""
+    defs = arg_defs if token_contiguous_scales else strided_arg_defs
+    # the tuner memoises per (name, keys): the two argument lists need two names
+    name = 'gemm_fp8_fp8_bf16_nt' if token_contiguous_scales else 'gemm_fp8_fp8_bf16_nt_strided'
     skinny_atoms = get_skinny_fp8_config(m, n, k, num_cus)
     if skinny_atoms:
-        keys = {'N': n, 'K': k, 'BLOCK_M': 16 * skinny_atoms, 'BLOCK_N': 16, 'NUM_STAGES': 4, 'NUM_TMA_MULTICAST': 1,
-                'NUM_WAVES': 8}
-        return 'gemm_fp8_fp8_bf16_nt', keys, arg_defs, 8 * skinny_atoms * 64 * 16, skinny_template
+        keys = FrozenKeys({'N': n, 'K': k, 'BLOCK_M': 16 * skinny_atoms, 'BLOCK_N': 16, 'NUM_STAGES': 4, 'NUM_TMA_MULTICAST': 1,
+                'NUM_WAVES': 8})
+        return (name, keys, defs, 8 * skinny_atoms * 64 * 16,
+                skinny_template if token_contiguous_scales else skinny_strided_template)
     block_m, block_n = get_best_fp8_config(m, n, k, num_cus)
-    keys = {'N': n, 'K': k, 'BLOCK_M': block_m, 'BLOCK_N': block_n, 'NUM_STAGES': get_fp8_num_stages(block_m, block_n),
-            'NUM_TMA_MULTICAST': 1}
+    keys = FrozenKeys({'N': n, 'K': k, 'BLOCK_M': block_m, 'BLOCK_N': block_n, 'NUM_STAGES': get_fp8_num_stages(block_m, block_n),
+            'NUM_TMA_MULTICAST': 1})
     smem_size = keys['NUM_STAGES'] * (block_m + block_n) * 128
-    return 'gemm_fp8_fp8_bf16_nt', keys, arg_defs, smem_size, template
+    return name, keys, defs, smem_size, template if token_contiguous_scales else strided_template
+
+
+@functools.lru_cache(maxsize=None)
+def fp8_tuning_plan(m: int, n: int, k: int, num_cus: int, token_contiguous_scales: bool = True):
+    """(name, keys, space, arg_defs, template) for empirical tile selection among the cost model's three best tiles of
+    the tiled kernel (`m` joins the keys as the tuner's memo key), or None when the weight-streaming kernel runs."""
+    if get_skinny_fp8_config(m, n, k, num_cus):
+        return None
+    space = tuple({'BLOCK_M': bm, 'BLOCK_N': bn, 'NUM_STAGES': get_fp8_num_stages(bm, bn)}
+                  for bm, bn in get_fp8_tile_space(m, n, k, num_cus))
+    keys = FrozenKeys({'M': m, 'N': n, 'K': k, 'NUM_TMA_MULTICAST': 1})
+    if token_contiguous_scales:
+        return 'gemm_fp8_fp8_bf16_nt', keys, space, arg_defs, template
+    return 'gemm_fp8_fp8_bf16_nt_strided', keys, space, strided_arg_defs, strided_template
 
 
 def gemm_fp8_fp8_bf16_nt(lhs: Tuple[torch.Tensor, torch.Tensor],
@@ -107,10 +132,18 @@ def gemm_fp8_fp8_bf16_nt(lhs: Tuple[torch.Tensor, torch.Tensor],
         return
 
     num_sms = get_num_sms()
-    name, keys, defs, smem_size, code_template = fp8_kernel_plan(m, n, k, num_sms)
-    args = (lhs, lhs_scales, rhs, rhs_scales, out, m, torch.cuda.current_stream(), num_sms, smem_size,
-            lhs_scales.stride(0), lhs_scales.stride(1))
-    runtime = jit_tuner.compile_and_tune(name=name, keys=keys, space=(), includes=includes,
+    stride_m, stride_k = lhs_scales.stride()
+    token_contiguous = (m == 1 or stride_m == 1) and (lhs_scales.size(1) == 1 or stride_k == m)
+    name, keys, defs, smem_size, code_template = fp8_kernel_plan(m, n, k, num_sms, token_contiguous)
+    space = ()
+    if tuning_enabled():
+        tuning = fp8_tuning_plan(m, n, k, num_sms, token_contiguous)
+        if tuning is not None:
+            name, keys, space, defs, code_template = tuning
+    args = (lhs, lhs_scales, rhs, rhs_scales, out, m, torch.cuda.current_stream(), num_sms, smem_size)
+    if not token_contiguous:
+        args += (stride_m, stride_k)
+    runtime = jit_tuner.compile_and_tune(name=name, keys=keys, space=space, includes=includes,
                                          arg_defs=defs, template=code_template, args=args)
     rc = runtime(*args)
     assert rc == 0, f'{name} failed with HIP error {rc}'

@@ -26,6 +26,23 @@ def rank_tiles(m: int, n: int, num_cus: int, table, groups: int = 1) -> List[Tup
     return sorted(ranked)
 
 
+def tuning_enabled() -> bool:
+    """Empirical tile selection on the first call per shape (`YAN_TUNE_TILES=1`): the entry points hand the cost model's
+    three best tiles to the tuner as its `space` and the fastest on the device wins, as the reference's tuner does with
+    its candidate list (`yan/jit_kernels/cute_gemm.py:42-53`, `tuner.py:42-69`). Off by default: the first call of a
+    shape then costs up to three compilations and sixty timed launches."""
+    import os
+    return os.getenv('YAN_TUNE_TILES', '0') not in ('', '0')
+
+
+def get_dense_tile_space(m: int, n: int, k: int, num_cus: int, count: int = 3) -> List[Tuple[int, int]]:
+    return [tile for _, tile in rank_tiles(m, n, num_cus, _DENSE_TILES)[:count]]
+
+
+def get_fp8_tile_space(m: int, n: int, k: int, num_cus: int, count: int = 3) -> List[Tuple[int, int]]:
+    return [tile for _, tile in rank_tiles(m, n, num_cus, _FP8_TILES)[:count]]
+
+
 def get_best_dense_config(m: int, n: int, k: int, num_cus: int) -> Tuple[int, int]:
     return rank_tiles(m, n, num_cus, _DENSE_TILES)[0][1]
 
@@ -41,9 +58,9 @@ def get_dense_num_stages(block_m: int, block_n: int) -> int:
 
 
 def get_fp8_num_stages(block_m: int, block_n: int) -> int:
-    """LDS stages of the tiled FP8 kernel for a tile: a ring as deep as the 160 KB LDS allows, at most 8
-    (`Fp8TileConfig::MAX_RING_STAGES` in fp8_gemm.hpp): 2 for 256 x 256, 3 for 256 x 128 and 128 x 256, up to 8 for the
-    smallest. Tiles below 256 x 256 are what the cost model picks when a problem is short on work per CU, i.e. bound by
+    """LDS stages of the tiled FP8 kernel for a tile: a ring as deep as the 160 KB LDS allows, at most 8, or 12 for the
+    tiles of 16 and 32 weight rows that run the decode shapes (`Fp8TileConfig::MAX_RING_STAGES` in fp8_gemm.hpp): 2 for
+    256 x 256, 3 for 256 x 128 and 128 x 256, 8 for 64 x 64, 12 for 64 x 16. Tiles below 256 x 256 are what the cost model picks when a problem is short on work per CU, i.e. bound by
     operand streaming, and there one k-tile of prefetch does not cover the memory latency."""
     waves = 8 if block_m * block_n >= 256 * 128 else 4
     capable = block_m % 64 == 0 and (block_m // 8) % waves == 0 and block_n % 16 == 0
@@ -51,7 +68,7 @@ def get_fp8_num_stages(block_m: int, block_n: int) -> int:
         return 2
     rows = ceil_div(block_m, 8 * waves) * 8 * waves + ceil_div(block_n, 8 * waves) * 8 * waves      # whole copy passes
     stage_bytes = rows * 128 + ceil_div(block_m * 4, 1024) * 1024
-    return max(2, min(8, 160 * 1024 // stage_bytes))
+    return max(2, min(12 if block_n <= 32 else 8, 160 * 1024 // stage_bytes))
 
 
 def get_best_grouped_fp8_config(m: int, n: int, k: int, num_cus: int, groups: int = 1, m_alignment: int = 0,

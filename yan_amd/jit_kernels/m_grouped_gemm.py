@@ -14,7 +14,7 @@ import torch
 
 from .gemm import includes
 from .heuristics import get_best_grouped_fp8_config, get_fp8_num_stages
-from .tuner import jit_tuner
+from .tuner import FrozenKeys, jit_tuner
 from .utils import ceil_div, get_m_alignment_for_contiguous_layout, get_num_sms
 
 template = """
@@ -34,7 +34,7 @@ using GemmType = Gemm<N, K, BLOCK_M, BLOCK_N, 128, kNumGroups, kNumStages, kNumT
 // Launch kernel
 __return_code = static_cast<int>(GemmType::run_grouped(out, lhs, lhs_scales, lhs_scales_stride_m, lhs_scales_stride_k,
                                                        lhs_scales_stride_g, rhs, rhs_scales, grouped_layout,
-                                                       kNumGroups, m, N, K, stream));
+                                                       kNumGroups, m, N, K, stream, num_sms));
 """
 
 arg_defs = (('lhs', torch.float8_e4m3fn), ('lhs_scales', torch.float),
@@ -55,9 +55,9 @@ def grouped_kernel_plan(gemm_type: str, num_groups: int, m: int, n: int, k: int,
     else:
         block_m, block_n = get_best_grouped_fp8_config(m, n, k, num_cus, num_groups)
         name = 'm_grouped_gemm_fp8_fp8_bf16_nt'
-    keys = {'N': n, 'K': k, 'BLOCK_M': block_m, 'BLOCK_N': block_n, 'NUM_GROUPS': num_groups,
+    keys = FrozenKeys({'N': n, 'K': k, 'BLOCK_M': block_m, 'BLOCK_N': block_n, 'NUM_GROUPS': num_groups,
             'NUM_STAGES': get_fp8_num_stages(block_m, block_n),
-            'NUM_TMA_MULTICAST': 1, 'GEMM_TYPE': gemm_type}
+            'NUM_TMA_MULTICAST': 1, 'GEMM_TYPE': gemm_type})
     return name, keys, arg_defs, keys['NUM_STAGES'] * (block_m + block_n) * 128
 
 

@@ -12,7 +12,7 @@ import functools
 import torch
 
 from .heuristics import get_best_float_config
-from .tuner import jit_tuner
+from .tuner import FrozenKeys, jit_tuner
 from .utils import get_num_sms
 
 includes = ('"gemm/simple_gemm.hpp"', )
@@ -43,7 +43,7 @@ arg_defs = (('m', int), ('n', int), ('k', int),
 def float_kernel_plan(m: int, n: int, num_cus: int):
     """(name, keys, arg_defs) of the JIT kernel a call with these sizes uses; needs no GPU."""
     block_m, block_n = get_best_float_config(m, n, num_cus)
-    return 'gemm_float_nt', {'BLOCK_M': block_m, 'BLOCK_N': block_n}, arg_defs
+    return 'gemm_float_nt', FrozenKeys({'BLOCK_M': block_m, 'BLOCK_N': block_n}), arg_defs
 
 
 def _leading_dim(x: torch.Tensor) -> int:

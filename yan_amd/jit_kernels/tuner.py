@@ -34,14 +34,29 @@ def _time_candidate(runtime: Runtime, args: tuple) -> float:
     return start.elapsed_time(end)
 
 
+class FrozenKeys(dict):
+    """Keys of a kernel plan that its owner promises never to change (the entry points memoise their plans and hand
+    the same object over on every call): any attempt to modify one raises."""
+
+    def _frozen(self, *_, **__):
+        raise TypeError('the keys of a memoised kernel plan are read-only')
+
+    __setitem__ = __delitem__ = clear = pop = popitem = setdefault = update = __ior__ = _frozen
+
+
 class JITTuner:
     def __init__(self) -> None:
         self.tuned: Dict[Tuple[str, str], Runtime] = {}
         self.tuned_keys: Dict[Tuple[str, str], Dict[str, Any]] = {}
-        # Callers that pass the very same `keys` object again (the entry points memoise their plans) skip building the
-        # textual signature: (name, id(keys)) -> (keys, runtime); the stored reference both keeps the id from being
-        # reused and is compared on lookup.
+        # Callers that pass the very same FrozenKeys object again skip building the textual signature:
+        # (name, id(keys)) -> (keys, runtime); the stored reference both keeps the id from being reused and is compared
+        # on lookup. An ordinary dict, which its owner may change between calls, always takes the signature path, as
+        # in the reference.
         self._same_object: Dict[Tuple[str, int], Tuple[Dict[str, Any], Runtime]] = {}
+
+    def _remember(self, name: str, keys: Dict[str, Any], runtime: Runtime) -> None:
+        if isinstance(keys, FrozenKeys):
+            self._same_object[(name, id(keys))] = (keys, runtime)
 
     def compile_and_tune(self, name: str, keys: Dict[str, Any], space: tuple,
                          includes: tuple, arg_defs: tuple, template: str, args: tuple) -> Runtime:
@@ -56,7 +71,7 @@ class JITTuner:
         if hit is not None:
             if debug:
                 print(f'Using cached JIT kernel {name} with keys {keys}')
-            self._same_object[(name, id(caller_keys))] = (caller_keys, hit)
+            self._remember(name, caller_keys, hit)
             return hit
         if debug:
             print(f'Auto-tuning JIT kernel {name} with keys {keys}')
@@ -89,7 +104,7 @@ class JITTuner:
             print(f'Best JIT kernel {name} with keys {keys} has tuned keys {best[2]} and time {best[0]}')
         self.tuned[signature] = best[1]
         self.tuned_keys[signature] = dict(best[2])
-        self._same_object[(name, id(caller_keys))] = (caller_keys, best[1])
+        self._remember(name, caller_keys, best[1])
         return best[1]
 
 

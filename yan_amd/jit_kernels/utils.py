@@ -26,6 +26,13 @@ def get_num_sms() -> int:
     return _num_sms
 
 
+def get_num_sms_cap() -> int:
+    """The cap as the kernels' launchers take it: 0 when every compute unit may be used (never capped, or capped at the
+    device's count), else the cap."""
+    cap = get_num_sms()
+    return 0 if cap >= _device_cu_count() else cap
+
+
 def ceil_div(x: int, y: int) -> int:
     return (x + y - 1) // y
 
@@ -45,3 +52,43 @@ def get_col_major_tensor(x: torch.Tensor) -> torch.Tensor:
     if not (batched.stride(1) == 1 and batched.stride(2) == rows):
         batched = batched.transpose(1, 2).contiguous().transpose(1, 2)
     return batched if x.dim() == 3 else batched.squeeze(0)
+
+
+def compare_tensors(actual: torch.Tensor, expected: torch.Tensor, mode: str = 'element-wise', rtol: float = 1e-5,
+                    atol: float = 1e-8, diff_tolerance: float = 1e-6, verbose: bool = True) -> bool:
+    """Compare a result with its expectation, print a one-line verdict and return it (reference:
+    `yan/jit_kernels/utils.py:138-179`, used by its accuracy tests). `mode='element-wise'` is `torch.allclose` with
+    `rtol` / `atol` and, on failure, reports the mean and the largest difference and where it sits;
+    `mode='similarity'` is `calc_diff(actual, expected) <= diff_tolerance` (0 when both are all zero). A shape mismatch
+    or an unknown mode fails. Passing verdicts carry their figures only when `verbose`; failures always do, and with
+    `verbose` also show the first ten elements of both tensors."""
+    lines = []
+    if actual.shape != expected.shape:
+        passed = False
+        lines.append(f'Shape mismatch: {tuple(actual.shape)} vs {tuple(expected.shape)}')
+    elif mode == 'element-wise':
+        passed = bool(torch.allclose(actual, expected, rtol=rtol, atol=atol))
+        if passed:
+            lines.append(f'(Tensors are element-wise close within rtol={rtol}, atol={atol})')
+        else:
+            gap = (actual - expected).abs()
+            worst = int(gap.argmax())
+            where = [int(i) for i in torch.unravel_index(torch.tensor(worst), gap.shape)] if gap.dim() else []
+            lines.append(f'Mean diff: {gap.mean().item():.6f}, Max diff: {gap.max().item():.6f}')
+            lines.append(f'Max diff at {where}: {actual.flatten()[worst].item():.6f} vs {expected.flatten()[worst].item():.6f}')
+    elif mode == 'similarity':
+        x, y = actual.double(), expected.double()
+        norm = (x * x + y * y).sum()
+        diff = 0.0 if norm == 0 else float(1 - 2 * (x * y).sum() / norm)
+        passed = diff <= diff_tolerance
+        lines.append(f'(Difference: {diff:.6f} {"<=" if passed else ">"} Tolerance: {diff_tolerance})')
+    else:
+        passed = False
+        lines.append(f"Invalid mode '{mode}'. Choose 'element-wise' or 'similarity'.")
+    print('Verification: PASSED' if passed else 'Verification: FAILED')
+    if lines and (verbose or not passed):
+        print('\n'.join(lines))
+    if not passed and verbose:
+        print(f'Actual tensor:\n{actual.flatten()[:10]}\n')
+        print(f'Expected tensor:\n{expected.flatten()[:10]}\n')
+    return passed
