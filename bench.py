@@ -55,6 +55,55 @@ def _event_time_ms(fn, steps, warmup, settle=0):
     return start.elapsed_time(end) / steps, wall_ms / steps
 
 
+def _clock_and_power(fn, seconds=0.4):
+    """Shader clock (MHz) and board power (W) while `fn` is launched back to back for about `seconds`, read from the
+    amdgpu driver's sysfs files (pp_dpm_sclk, hwmon power1_input / power1_average) every few milliseconds; None where
+    the files are absent or unreadable. Outside every timed region: the sampling thread shares the interpreter with
+    the launch loop."""
+    import glob
+    import threading
+    import torch
+    sclk = (glob.glob('/sys/class/drm/card*/device/pp_dpm_sclk') + [None])[0]
+    power = (glob.glob('/sys/class/drm/card*/device/hwmon/hwmon*/power1_input') +
+             glob.glob('/sys/class/drm/card*/device/hwmon/hwmon*/power1_average') + [None])[0]
+    if sclk is None and power is None:
+        return None
+    clocks, watts, stop = [], [], threading.Event()
+
+    def sample():
+        while not stop.is_set():
+            try:
+                if sclk:
+                    active = [line for line in open(sclk).read().splitlines() if line.rstrip().endswith('*')]
+                    if active:
+                        clocks.append(float(active[0].split(':')[1].lower().replace('mhz', '').replace('*', '').strip()))
+                if power:
+                    watts.append(float(open(power).read()) * 1e-6)
+            except (OSError, ValueError, IndexError):
+                pass
+            time.sleep(0.004)
+
+    fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(20):
+        fn()
+    torch.cuda.synchronize()
+    per_call = (time.perf_counter() - t0) / 20
+    calls = max(20, int(seconds / max(per_call, 1e-6)))
+    for _ in range(calls // 2):         # back under load before sampling starts
+        fn()
+    thread = threading.Thread(target=sample, daemon=True)
+    thread.start()
+    for _ in range(calls):
+        fn()
+    torch.cuda.synchronize()
+    stop.set()
+    thread.join()
+    mean = lambda xs: round(sum(xs) / len(xs), 1) if xs else None
+    return {'shader_clock_mhz': mean(clocks), 'board_power_w': mean(watts), 'samples': max(len(clocks), len(watts))}
+
+
 def _cpu_baseline_fp8(a8, sa, b8, sb, budget_s=12.0):
     """The reference's CPU path for this metric: torch CPU matmul of the dequantised operands (fp32), timed on a
     slab of rows sized for about `budget_s` seconds, scaled to the full M by the flop count."""
@@ -173,6 +222,7 @@ def main():
     # validity of what was timed: sampled rows against an fp32 matmul of the dequantised operands
     diff = _sampled_fp8_diff(yan, harness, a8, sa, b8, sb, out)
     assert diff < 1e-3, f'parity lost: calc_diff={diff}'
+    under_load = _clock_and_power(step)
     flops = 2.0 * m * n * k
     tflops_job = flops / (wall_ms * 1e-3) / 1e12
     tflops_kernel = flops / (kernel_ms * 1e-3) / 1e12
@@ -197,6 +247,12 @@ def main():
                      'kernel': 'fp8_gemm_kernel', 'kernel_us': round(kernel_ms * 1e3, 2),
                      'algorithmic_flop_per_launch': flops, 'algorithmic_bytes_per_launch': _fp8_bytes(m, n, k)},
     }
+    if under_load and under_load['shader_clock_mhz']:
+        # the chip is power-limited under this load: the same kernel time as a fraction of the matrix-core cycles that
+        # passed at the clock the chip actually ran at (256 CUs x 8192 flop per cycle)
+        line['roofline']['under_load'] = under_load
+        line['roofline']['frac_of_mfma_cycles_at_measured_clock'] = round(
+            tflops_kernel * 1e12 / (yan.get_num_sms() * 8192 * under_load['shader_clock_mhz'] * 1e6), 4)
 
     extra = {}
     if not args.no_extra:
@@ -211,8 +267,16 @@ def main():
         extra['bf16_8192'] = {'us': round(ms * 1e3, 1), 'tflops': round(fl / ms / 1e9, 1),
                               'frac_of_bf16_peak': round(fl / ms / 1e9 / PEAK_BF16_TFLOPS, 4), 'steps': 20, 'warmup': 5,
                               'settle_launches': settle['cfg2'], 'calc_diff_sampled_rows': d}
+        load = _clock_and_power(lambda: yan.gemm_bf16_tn(a, b, c))
+        if load and load['shader_clock_mhz']:
+            extra['bf16_8192']['under_load'] = load
+            extra['bf16_8192']['frac_of_mfma_cycles_at_measured_clock'] = round(
+                fl / ms / 1e9 * 1e12 / (yan.get_num_sms() * 4096 * load['shader_clock_mhz'] * 1e6), 4)
         ms, _ = _event_time_ms(lambda: torch.matmul(a, b.t(), out=c), 20, 5, settle['cfg2'])
         extra['bf16_8192_torch_hipblaslt'] = {'us': round(ms * 1e3, 1), 'tflops': round(fl / ms / 1e9, 1)}
+        load = _clock_and_power(lambda: torch.matmul(a, b.t(), out=c))
+        if load and load['shader_clock_mhz']:
+            extra['bf16_8192_torch_hipblaslt']['under_load'] = load
         del a, b, c
         # configs[3]: the M=64 decode shape, HBM-bound. The kernel is shorter than the host side of a call, so its
         # device time comes from the profiler; cold = a 512 MB write before every call.

@@ -7,8 +7,9 @@
 // accumulation and no bounds handling. Here:
 //   * macro tile BLOCK_M x BLOCK_N x 64 (128-byte rows), staged HBM -> LDS with buffer_load ... lds (tile_io.hpp);
 //   * the 256 x 256 tile: two LDS stages, 8 waves (two per SIMD), each with a 128 x 64 slab of 16x16x32 MFMAs (128
-//     accumulator registers); while one wave of a SIMD waits at the barrier or issues copies the other keeps the
-//     matrix core busy (dense_gemm_body_8w);
+//     accumulator registers); while one wave of a SIMD issues copies or waits for a fragment the other keeps the
+//     matrix core busy, and the barrier between two k-tiles sits two steps before the end of the first, so that
+//     every wave still holds work when it has passed it (dense_gemm_body_8w);
 //   * the smaller tiles, which run problems bound by operand streaming: a ring of three to eight LDS stages, 4 waves,
 //     one per SIMD, each with a (BLOCK_N/WAVES_N) x (BLOCK_M/WAVES_M) slab of 32x32x16 MFMAs, up to 128 x 128 (256
 //     accumulator registers, which the compiler keeps in AGPRs) (dense_gemm_body);
@@ -231,12 +232,12 @@ dense_gemm_body(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, El
 }
 
 // The same contraction with 8 waves (two per SIMD) and 16x16x32 atoms: each wave owns a (BLOCK_N/2) x (BLOCK_M/4) slab,
-// 128 accumulator registers for the 256 x 256 tile. Two LDS stages; while one wave of a SIMD waits at the barrier or
-// issues its copies, the other keeps the matrix core busy. The kernel is persistent: a workgroup walks the tiles
-// blockIdx.x, blockIdx.x + gridDim.x, ... (the launcher starts one workgroup per CU), starts the copies of the next
-// tile's first k-tile during the last k-tile of the current one, and its output stores drain while the next tile is
-// already computing. With one workgroup per tile the drain and the first loads of every tile were exposed: 11 % of the
-// time at 8192^3.
+// 128 accumulator registers for the 256 x 256 tile. Two LDS stages. The kernel is persistent: a workgroup walks the tiles
+// blockIdx.x, blockIdx.x + gridDim.x, ... (the launcher starts one workgroup per CU, or as many as the caller's cap
+// allows), starts the copies of the next tile's first k-tile during the last k-tile of the current one, fetches that
+// k-tile's first fragments before it turns to the epilogue, and its output stores drain while the next tile is already
+// computing. With one workgroup per tile the drain and the first loads of every tile were exposed: 11 % of the time at
+// 8192^3.
 template <typename Atom, typename Elem, int BLOCK_M, int BLOCK_N>
 __device__ __forceinline__ void
 dense_gemm_body_8w(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, Elem* __restrict__ C, int m, int n, int k) {
@@ -267,12 +268,18 @@ dense_gemm_body_8w(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
     // out the operand panels the other workgroups of the XCD are about to read (8192^3: 805 -> 754 us).
     const bool stream_out = size_t(m) * n * sizeof(Elem) > (size_t(32) << 20);
 
+    // Every tile runs an even number of k-tiles, so that it starts in stage 0 and the stage of every k-step is known
+    // at compile time (the compiler then sees that the copies into one stage cannot touch the fragments it reads from
+    // the other, and does not wait for them): an odd count gets one more k-tile whose copies are sent out of range
+    // and move zeros.
+    const int k_tiles_run = (num_k_tiles + 1) & ~1;
     // What a wave needs to know of a tile to copy its k-tiles.
     struct TileIo {
         StA a;
         StB b;
         uint32_t tail_a, tail_b;
         int m0, n0;
+        int k_rot;          // the k-tile this tile's walk over K starts at
         bool valid;
     };
     auto open_tile = [&](int slot) {
@@ -285,21 +292,25 @@ dense_gemm_body_8w(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
         t.b.init(t.n0, ld_bytes, wave, lane);
         t.tail_a = t.a.tail_voff(k_bytes % kRowBytes);
         t.tail_b = t.b.tail_voff(k_bytes % kRowBytes);
+        t.k_rot = (slot % kNumXCD) * (k_tiles_run / kNumXCD);
         return t;
     };
-    // Every tile runs an even number of k-tiles, so that it starts in stage 0 and the stage of every k-step is known
-    // at compile time (the compiler then sees that the copies into one stage cannot touch the fragments it reads from
-    // the other, and does not wait for them): an odd count gets one more k-tile whose copies are sent out of range
-    // and move zeros.
-    const int k_tiles_run = (num_k_tiles + 1) & ~1;
-    auto copy_pass = [&](const TileIo& t, int d, int kt, uint8_t* la, uint8_t* lb) {
+    // The tiles of different XCDs (slot % 8: a property of the tile, not of the workgroup that happens to run it) start their
+    // walk over K at different k-tiles and wrap around: the whole chip asking the memory side for the same columns of
+    // every row at the same moment queues on the channels that hold them (8192 x 8192 x 9216: 954 -> 890 us; nothing
+    // changes at K = 8192). The order of summation over K therefore depends on the tile, not on the launch.
+    auto copy_pass = [&](const TileIo& t, int d, int kt_run, uint8_t* la, uint8_t* lb) {
+        const int kt = kt_run + t.k_rot >= k_tiles_run ? kt_run + t.k_rot - k_tiles_run : kt_run + t.k_rot;
         const bool tail = kt == tail_tile, past = kt >= num_k_tiles;
         if (d < StA::PASSES) t.a.issue_pass_from(rsrc_a, la, kt * kRowBytes, wave, d, past ? kOutOfRange : (tail ? t.tail_a : t.a.voff));
         else t.b.issue_pass_from(rsrc_b, lb, kt * kRowBytes, wave, d - StA::PASSES, past ? kOutOfRange : (tail ? t.tail_b : t.b.voff));
     };
 
-    // The two 32-deep halves of a 64-deep k-tile: chunk 4 * half + g of the lane's row.
-    const int koff[2] = {frag_offset<16>(lane, g), frag_offset<16>(lane, 4 + g)};
+    // The two MFMAs that cover a 64-deep k-tile: lane group g takes chunks 2g and 2g + 1 of its row, so the first MFMA
+    // contracts over chunks {0, 2, 4, 6} and the second over {1, 3, 5, 7}; both operands use the same assignment, which
+    // is all the contraction needs. With chunks g and 4 + g instead (K in natural order) every ds_read_b128 takes twice
+    // as long: the counters show 8 LDS cycles per instruction, half of them bank conflicts, against 4 with this order.
+    const int koff[2] = {frag_offset<16>(lane, 2 * g), frag_offset<16>(lane, 2 * g + 1)};
 
     // One array for both stages: with a separate array per stage the compiler knows which copies feed which fragment
     // reads and guards the reads with a wait for every outstanding vector-memory operation, the output stores of the
@@ -314,39 +325,68 @@ dense_gemm_body_8w(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
     f32x4 acc[TN][TM];
 
     // One k-tile: STEPS = 2 * TN steps of TM MFMAs (one row of atoms, one half of K); the fragments of the next step are
-    // fetched before the MFMAs of this one issue (fetching two steps ahead measured no faster); `copy(s)` runs once per
-    // step from the start of the tile and is where the copies of whatever comes next are started, one per step.
-    // `stores_behind`: the last STORES_PER_TILE vector-memory operations of this wave are the previous tile's output
-    // stores, issued after the copies this k-tile needs; the in-order counter then only has to drop to that many,
-    // and the stores drain while the new tile computes.
-    constexpr int STORES_PER_TILE = TM * 4;
-    auto k_step = [&](const uint8_t* a_cur, const uint8_t* b_cur, bool stores_behind, auto&& copy) {
-        if (stores_behind) __builtin_amdgcn_s_waitcnt(waitcnt_imm(STORES_PER_TILE, kNoWaitLgkm));
-        else wait_for_copies();
-        // a bare barrier: __syncthreads() carries a fence that would wait for the stores after all
+    // fetched before the MFMAs of this one issue (fetching two steps ahead measured no faster).
+    // The MFMAs are written as instructions whose destination is their own addend. Left to the compiler, the sums
+    // wander through the register file (every MFMA writes its result somewhere new), the kernel sits at the 256-register
+    // limit, spills, and pays wait states wherever a fragment read lands in registers a sum has just left: 4 % of the
+    // time at 8192^3. Tied, the kernel needs 220 registers.
+    // Fragments live across k-tiles: the barrier that opens k-tile t + 1 sits TAIL steps before the end of k-tile t, where
+    // every fragment of k-tile t is in registers; behind it the first fragments of k-tile t + 1 are fetched and the TAIL
+    // steps still held are multiplied while those fetches are under way.
+    constexpr int TAIL = 2, NS = 4;
+    static_assert(STEPS % NS == 0 && TAIL + 1 < NS && NUM_COPIES <= STEPS - TAIL);
+    Frag nf[NS], mf[2][TM];           // weight fragments, step s in slot s % NS; activation fragments of the two K halves
+    auto mma = [&](int s) {
+        const int half = s / TN, i = s % TN;
+#pragma unroll
+        for (int j = 0; j < TM; ++j) {
+            if constexpr (__is_same(Elem, __bf16))
+                asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+v"(acc[i][j]) : "v"(nf[s % NS]), "v"(mf[half][j]));
+            else
+                asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+v"(acc[i][j]) : "v"(nf[s % NS]), "v"(mf[half][j]));
+        }
+    };
+    // What the first step of the k-tile staged in (a, b) needs.
+    auto fetch_first = [&](const uint8_t* a, const uint8_t* b) {
+        nf[0] = *reinterpret_cast<const Frag*>(b + wn * WTN * kRowBytes + koff[0]);
+#pragma unroll
+        for (int j = 0; j < TM; ++j) mf[0][j] = *reinterpret_cast<const Frag*>(a + (wm * WTM + j * 16) * kRowBytes + koff[0]);
+    };
+    // every copy, store and fragment read of mine is done; then: every wave's
+    auto open_next = [&] {
+        __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 0));
         asm volatile("" ::: "memory");
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
+    };
+    // One k-tile, staged in (a_cur, b_cur), whose first fragments are in registers or on their way. `copy(s)` runs once per
+    // step for the first NUM_COPIES steps and starts the copies of the k-tile that comes next, staged in (a_nxt, b_nxt).
+    auto k_step = [&](const uint8_t* a_cur, const uint8_t* b_cur, const uint8_t* a_nxt, const uint8_t* b_nxt, auto&& copy) {
         const uint8_t* pa = a_cur + wm * WTM * kRowBytes;
         const uint8_t* pb = b_cur + wn * WTN * kRowBytes;
-        Frag nf[2], mf[2][TM];
-        auto fetch_n = [&](int s) { nf[s & 1] = *reinterpret_cast<const Frag*>(pb + (s % TN) * 16 * kRowBytes + koff[s / TN]); };
-        auto fetch_m = [&](int h) {
+        auto fetch_n = [&](int s) { nf[s % NS] = *reinterpret_cast<const Frag*>(pb + (s % TN) * 16 * kRowBytes + koff[s / TN]); };
 #pragma unroll
-            for (int j = 0; j < TM; ++j) mf[h][j] = *reinterpret_cast<const Frag*>(pa + j * 16 * kRowBytes + koff[h]);
-        };
-        fetch_n(0);
-        fetch_m(0);
+        for (int s = 0; s < STEPS - TAIL; ++s) {
+            if (s < NUM_COPIES) copy(s);
+            fetch_n(s + 1);
+            if (s == STEPS - TAIL - 1) {
+#pragma unroll
+                for (int x = s + 2; x < STEPS; ++x) fetch_n(x);
+            }
+            if (s + 1 == TN) {
+#pragma unroll
+                for (int j = 0; j < TM; ++j) mf[1][j] = *reinterpret_cast<const Frag*>(pa + j * 16 * kRowBytes + koff[1]);
+            }
+            mma(s);
+            __builtin_amdgcn_sched_barrier(0);        // without it the compiler hoists the reads and copies of the whole k-tile
+        }
+        open_next();
+        fetch_first(a_nxt, b_nxt);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int s = 0; s < STEPS; ++s) {
-            const int half = s / TN, i = s % TN;
-            if (s < NUM_COPIES) copy(s);
-            if (s + 1 < STEPS) fetch_n(s + 1);
-            if (s + 1 == TN) fetch_m(1);
-#pragma unroll
-            for (int j = 0; j < TM; ++j) acc[i][j] = Atom::mma(nf[s & 1], mf[half][j], acc[i][j]);
-            __builtin_amdgcn_sched_barrier(0);        // without it the compiler hoists the reads and copies of the whole k-tile
+        for (int s = STEPS - TAIL; s < STEPS; ++s) {
+            mma(s);
+            __builtin_amdgcn_sched_barrier(0);
         }
     };
 
@@ -355,7 +395,8 @@ dense_gemm_body_8w(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
     if (!cur.valid) return;
 #pragma unroll
     for (int d = 0; d < NUM_COPIES; ++d) copy_pass(cur, d, 0, lds_a0, lds_b0);
-    bool stores_behind = false;
+    open_next();
+    fetch_first(lds_a0, lds_b0);
     while (true) {
         slot += gridDim.x;
         const TileIo nxt = open_tile(slot);
@@ -365,16 +406,16 @@ dense_gemm_body_8w(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
             for (int j = 0; j < TM; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
         int kt = 0;
         for (; kt + 2 < k_tiles_run; kt += 2) {
-            k_step(lds_a0, lds_b0, stores_behind, [&](int s) { copy_pass(cur, s, kt + 1, lds_a1, lds_b1); });
-            stores_behind = false;
-            k_step(lds_a1, lds_b1, false, [&](int s) { copy_pass(cur, s, kt + 2, lds_a0, lds_b0); });
+            k_step(lds_a0, lds_b0, lds_a1, lds_b1, [&](int s) { copy_pass(cur, s, kt + 1, lds_a1, lds_b1); });
+            k_step(lds_a1, lds_b1, lds_a0, lds_b0, [&](int s) { copy_pass(cur, s, kt + 2, lds_a0, lds_b0); });
         }
-        k_step(lds_a0, lds_b0, stores_behind, [&](int s) { copy_pass(cur, s, kt + 1, lds_a1, lds_b1); });
-        stores_behind = false;
-        // last k-tile of this tile: the copies are the first k-tile of the next tile, if there is one
-        k_step(lds_a1, lds_b1, false, [&](int s) { if (nxt.valid) copy_pass(nxt, s, 0, lds_a0, lds_b0); });
+        k_step(lds_a0, lds_b0, lds_a1, lds_b1, [&](int s) { copy_pass(cur, s, kt + 1, lds_a1, lds_b1); });
+        // last k-tile of this tile: the copies are the first k-tile of the next tile, if there is one, and what is fetched
+        // behind the barrier are its first fragments (bytes nobody uses when there is none)
+        k_step(lds_a1, lds_b1, lds_a0, lds_b0, [&](int s) { if (nxt.valid) copy_pass(nxt, s, 0, lds_a0, lds_b0); });
         uint8_t* const a_last = lds_a1;
         uint8_t* const b_last = lds_b1;
+        asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");      // the last MFMAs retire before the epilogue reads the sums
 
         // Epilogue: the 4 registers of atom (i, j) are n = n_slab + 16 i + 4 g + {0..3} of row m = m_slab + 16 j + col.
         // Stored straight from there a wave instruction would write 16 rows x 32 bytes; instead each wave turns its slab
@@ -385,11 +426,7 @@ dense_gemm_body_8w(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
         static_assert(WTM == 64 && WTN == 128 && sizeof(Elem) == 2, "the staged epilogue is laid out for 128 x 64 slabs");
         if ((n % 8) == 0) {
             constexpr int PITCH = 272;
-            // every wave has read the last k-tile (a bare barrier: nothing here depends on the copies under way)
-            __builtin_amdgcn_s_waitcnt(waitcnt_imm(kNoWaitVm, 0));
-            asm volatile("" ::: "memory");
-            __builtin_amdgcn_s_barrier();
-            asm volatile("" ::: "memory");
+            // every wave has read the last k-tile: they all passed the barrier inside its k_step with its fragments in registers
             uint8_t* region = (wave < 4 ? a_last : b_last) + (wave % 4) * (16 * PITCH);
             const __amdgpu_buffer_rsrc_t rsrc_c = make_out_rsrc(C + size_t(cur.m0) * n + cur.n0);
             const int r4 = lane / 16, c = lane % 16;
@@ -407,8 +444,6 @@ dense_gemm_body_8w(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
                         buffer_store_16(v, rsrc_c, uint32_t((wm * WTM + 16 * j + row) * n + wn * WTN + 8 * c) * 2u, stream_out);
                 }
             }
-            // an interior tile: every lane of every wave has just issued exactly STORES_PER_TILE stores
-            stores_behind = cur.m0 + BLOCK_M <= m && cur.n0 + BLOCK_N <= n;
         } else {
 #pragma unroll
             for (int j = 0; j < TM; ++j) {
@@ -424,6 +459,11 @@ dense_gemm_body_8w(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
         }
         if (!nxt.valid) break;
         cur = nxt;
+        // the next tile's second k-tile is copied into the stage the epilogue went through: every wave has to be out of it
+        __builtin_amdgcn_s_waitcnt(waitcnt_imm(kNoWaitVm, 0));
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
     }
 }
 

@@ -306,6 +306,70 @@ fp8_gemm_tile(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_sca
                                                      scale_voff, (kb * sa_stride_k + part * 64 * sa_stride_m) * 4, 0, 0);
         }
     };
+    // Tiles of one or two atoms per wave (the decode shapes: 16 or 32 weight rows per workgroup) have almost nothing to
+    // compute per k-tile, and a loop that meets at a barrier for every k-tile is bound by that chain of waits: barrier,
+    // fragment reads, one MFMA, its fold, 56 times over. They consume the ring G k-tiles at a time instead: one
+    // barrier, the fragments of G k-tiles, G independent MFMAs, G folds; the copies of the G k-tiles that go where the
+    // previous group was start right after the barrier, so STAGES - 2G to STAGES - G k-tiles are in flight.
+    constexpr int G = (TN * TM <= 2 && STAGES >= 12 && STAGES % 4 == 0) ? 4 : 1;
+    if constexpr (G > 1) {
+    static_assert(Cfg::UNIFORM_SCALE_B && NB == 1 && (STAGES - 2 * G) * OPS <= 63);
+#pragma unroll
+    for (int t = 0; t < STAGES - G; ++t)
+#pragma unroll
+        for (int d = 0; d < OPS; ++d) issue_op(d, t, ring + t * STAGE_BYTES);
+    int base = 0;          // ring position of the group's first k-tile; STAGES is a multiple of G, groups never wrap
+    for (int kb0 = 0; kb0 < NUM_K_BLOCKS; kb0 += G) {
+        float sb_grp[G];
+#pragma unroll
+        for (int t = 0; t < G; ++t)
+            sb_grp[t] = rhs_scales[min(base_blk, NUM_N_BLOCKS - 1) * NUM_K_BLOCKS + min(kb0 + t, NUM_K_BLOCKS - 1)];
+        __builtin_amdgcn_s_waitcnt(waitcnt_imm((STAGES - 2 * G) * OPS, kNoWaitLgkm));
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        // every wave has left the previous group: its stages take k-tiles kb0 + STAGES - G .. kb0 + STAGES - 1 (past the
+        // last k-tile these move bytes nobody reads; they are issued all the same, the waits count instructions)
+        const int prev = base == 0 ? STAGES - G : base - G;
+#pragma unroll
+        for (int t = 0; t < G; ++t)
+#pragma unroll
+            for (int d = 0; d < OPS; ++d) issue_op(d, kb0 + STAGES - G + t, ring + (prev + t) * STAGE_BYTES);
+        f32x4 part[G][TN][TM];
+        float s_grp[G][TM];
+#pragma unroll
+        for (int t = 0; t < G; ++t) {
+            const uint8_t* cur = ring + (base + t) * STAGE_BYTES;
+            const uint8_t* pa = cur + wm * Cfg::WTM * kRowBytes;
+            const uint8_t* pb = cur + A_BYTES + wn * Cfg::WTN * kRowBytes;
+            const float* my_scales = reinterpret_cast<const float*>(cur + TILE_BYTES) + wm * Cfg::WTM + col;
+            i32x8 mf[TM], nf[TN];
+#pragma unroll
+            for (int j = 0; j < TM; ++j) { mf[j] = read_frag(pa + j * 16 * kRowBytes); s_grp[t][j] = my_scales[j * 16] * sb_grp[t]; }
+#pragma unroll
+            for (int i = 0; i < TN; ++i) nf[i] = read_frag(pb + i * 16 * kRowBytes);
+#pragma unroll
+            for (int i = 0; i < TN; ++i)
+#pragma unroll
+                for (int j = 0; j < TM; ++j) part[t][i][j] = Atom::mma(nf[i], mf[j], f32x4{0.f, 0.f, 0.f, 0.f});
+        }
+#pragma unroll
+        for (int t = 0; t < G; ++t) {
+            if (kb0 + t < NUM_K_BLOCKS) {          // wave-uniform; k-tiles past the end hold bytes of other rows
+#pragma unroll
+                for (int i = 0; i < TN; ++i)
+#pragma unroll
+                    for (int j = 0; j < TM; ++j)
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) acc[i][j][r] = __builtin_fmaf(part[t][i][j][r], s_grp[t][j], acc[i][j][r]);
+            }
+        }
+        base = base + G == STAGES ? 0 : base + G;
+    }
+    // the first stage of the group that was consumed last: no copy is on its way into it
+    epi_a = ring + (base == 0 ? STAGES - G : base - G) * STAGE_BYTES;
+    epi_b = epi_a + A_BYTES;
+    } else {
 #pragma unroll
     for (int t = 0; t < STAGES - 1; ++t)
 #pragma unroll
@@ -335,6 +399,7 @@ fp8_gemm_tile(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_sca
     }
     epi_a = ring + (st == 0 ? STAGES - 1 : st - 1) * STAGE_BYTES;
     epi_b = epi_a + A_BYTES;
+    }
     }
 
     // Epilogue: the 4 registers of atom (i, j) are n = n_slab + 16i + 4g + {0..3} of row m = m_slab + 16j + col.
