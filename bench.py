@@ -199,6 +199,7 @@ def main():
     import yan_amd as yan
     import harness
     from yan_amd.jit_kernels.gemm import fp8_kernel_plan
+    from yan_amd.jit_kernels.heuristics import get_best_dense_config
     assert torch.cuda.is_available(), 'bench.py needs a GPU'
     torch.cuda.set_device(0)
     settle = {leg: (0 if args.no_settle else count) for leg, count in SETTLE.items()}
@@ -311,6 +312,17 @@ def main():
         del x8, sx, w8, sw, o
 
     if args.also:
+        # bf16 shapes whose tiles do not fill whole rounds of 256 compute units at 256 x 256, next to torch.matmul (hipBLASLt)
+        for mm, nn, kk in ((4096, 5120, 5120), (2048, 7168, 7168), (4096, 7168, 16384), (8192, 8192, 9216)):
+            a, b, c = harness.make_bf16_case(mm, nn, kk, seed=42, scale=kk ** -0.5, device='cuda', gen_device='cuda')
+            ms, _ = _event_time_ms(lambda: yan.gemm_bf16_tn(a, b, c), 30, 5, 200)
+            ms_t, _ = _event_time_ms(lambda: torch.matmul(a, b.t(), out=c), 30, 5, 200)
+            fl = 2.0 * mm * nn * kk
+            extra[f'bf16_{mm}x{nn}x{kk}'] = {'us': round(ms * 1e3, 1), 'tflops': round(fl / ms / 1e9, 1),
+                                             'frac_of_bf16_peak': round(fl / ms / 1e9 / PEAK_BF16_TFLOPS, 4),
+                                             'tile': 'x'.join(map(str, get_best_dense_config(mm, nn, kk, yan.get_num_sms()))),
+                                             'torch_hipblaslt_us': round(ms_t * 1e3, 1), 'hipblaslt_over_this': round(ms_t / ms, 3)}
+            del a, b, c
         # grouped (mixture-of-experts) layouts: 4 groups x 8192 rows contiguous; 4 groups x 1024 of 1024 rows masked
         rows, nn, kk = (8192,) * 4, 4096, 7168
         (x8, sx), (w8, sw), o, idx = harness.make_grouped_contiguous_case(rows, nn, kk, seed=42, device='cuda', gen_device='cuda')

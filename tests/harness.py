@@ -156,7 +156,13 @@ DENSE_TEST_SHAPES = [
     (3000, 5000, 1000),          # the 256 x 256 tile (8-wave kernel) with ragged m, n and a k tail
     (2900, 5004, 520),           # same with n % 8 == 4 (narrow stores) and an odd number of k-tiles
     (2900, 5000, 64),            # same with a single k-tile
+    # the narrower tiles of the 8-wave kernel: 256 x 160, 256 x 224, 256 x 192, each once whole and once ragged in m, n and k
+    (4096, 5120, 512), (4000, 5000, 520), (2048, 7168, 256), (2047, 7100, 264), (4096, 6144, 256), (4090, 6100, 72),
 ]
+# (shape, tile the cost model must pick): the shapes above exist for these tiles
+DENSE_TILE_OF_SHAPE = {(4096, 5120, 512): (256, 160), (4000, 5000, 520): (256, 160), (2048, 7168, 256): (256, 224),
+                       (2047, 7100, 264): (256, 224), (4096, 6144, 256): (256, 192), (4090, 6100, 72): (256, 192),
+                       (3000, 5000, 1000): (256, 256), (8192, 8192, 8192): (256, 256)}
 # (m, n, k) of the reference's own dense test (tests/test_cute.py:21-22: m in (256, 4096) x six (k, n) pairs)
 REFERENCE_DENSE_TEST_SHAPES = [(m, n, k) for m in (256, 4096)
                                for k, n in ((5120, 5120), (1536, 24576), (512, 32768), (16384, 7168), (7168, 2048), (2048, 7168))]
@@ -219,7 +225,8 @@ def jit_kernels_in_use(num_cus: int = 256):
         code = generate(includes, arg_defs, cpp_format(code_template, keys))
         kernels.setdefault((name, code), (name, arg_defs, code))
 
-    for m, n, k in DENSE_TEST_SHAPES + REFERENCE_DENSE_TEST_SHAPES + [(256, 512, 512)]:
+    # the last four: shapes only the benchmark's --also legs run
+    for m, n, k in DENSE_TEST_SHAPES + REFERENCE_DENSE_TEST_SHAPES + [(256, 512, 512), (4096, 5120, 5120), (2048, 7168, 7168), (4096, 7168, 16384), (8192, 8192, 9216)]:
         for dtype in (torch.bfloat16, torch.half):
             if m and n:
                 name, keys, arg_defs = bf16_gemm.dense_kernel_plan(m, n, k, dtype, num_cus)

@@ -51,6 +51,15 @@ def test_tile_heuristics_fill_256_cus():
     assert ranked == sorted(ranked) and len(ranked) == len(heuristics._FP8_TILES)
 
 
+def test_dense_shapes_of_the_gpu_suite_reach_every_tile_of_the_8_wave_kernel():
+    """A change of the cost table must not silently take the 256 x {160, 192, 224} tiles out of the parity tests."""
+    import harness
+    for shape, tile in harness.DENSE_TILE_OF_SHAPE.items():
+        assert heuristics.get_best_dense_config(*shape, 256) == tile, shape
+        assert heuristics.get_dense_num_stages(*tile) == 2
+    assert {t for t in harness.DENSE_TILE_OF_SHAPE.values()} == {(256, 160), (256, 192), (256, 224), (256, 256)}
+
+
 def test_kernel_plans_keep_reference_keys_and_argument_order():
     name, keys, defs = bf16_gemm.dense_kernel_plan(4096, 7168, 2048, torch.bfloat16, 256)
     assert name == 'gemm_bf16_tn' and sorted(keys) == ['BLOCK_M', 'BLOCK_N', 'NUM_SMS', 'NUM_STAGES'] and keys['NUM_SMS'] == 0

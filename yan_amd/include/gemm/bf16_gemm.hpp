@@ -243,13 +243,15 @@ __device__ __forceinline__ void
 dense_gemm_body_8w(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, Elem* __restrict__ C, int m, int n, int k) {
     constexpr int NW = 8, WAVES_N = 2, WAVES_M = 4, WTN = BLOCK_N / WAVES_N, WTM = BLOCK_M / WAVES_M;
     constexpr int TN = WTN / 16, TM = WTM / 16, STEPS = 2 * TN;
-    static_assert(WTN % 16 == 0 && WTM % 16 == 0 && TN * TM * 4 <= 128);
+    static_assert(WTN % 16 == 0 && WTM % 16 == 0 && TN * TM * 4 <= 128 && TN >= 4);
     using Frag = typename Atom::Frag;
     using StA = TileStager<BLOCK_M, NW>;
     using StB = TileStager<BLOCK_N, NW>;
-    static_assert(StA::PADDED_ROWS == BLOCK_M && StB::PADDED_ROWS == BLOCK_N, "tiles are whole copy passes");
+    // BLOCK_N is any multiple of 32 from 128 to 256 (a problem whose tiles do not fill whole rounds of compute units with
+    // one width often does with another); the weight tile in LDS is rounded up to whole copy passes of 64 rows.
+    static_assert(StA::PADDED_ROWS == BLOCK_M, "the activation tile is whole copy passes");
+    constexpr int LDS_ROWS_B = StB::PADDED_ROWS;
     constexpr int NUM_COPIES = StA::PASSES + StB::PASSES;
-    static_assert(NUM_COPIES <= STEPS);
 
     const XcdTileScheduler<> sched(m, n, BLOCK_M, BLOCK_N);
     const int num_slots = sched.grid_size();
@@ -315,7 +317,7 @@ dense_gemm_body_8w(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
     // One array for both stages: with a separate array per stage the compiler knows which copies feed which fragment
     // reads and guards the reads with a wait for every outstanding vector-memory operation, the output stores of the
     // previous tile included; the waits below are exact instead.
-    constexpr int A_BYTES = BLOCK_M * kRowBytes, STAGE_BYTES = (BLOCK_M + BLOCK_N) * kRowBytes;
+    constexpr int A_BYTES = BLOCK_M * kRowBytes, STAGE_BYTES = (BLOCK_M + LDS_ROWS_B) * kRowBytes;
     __shared__ __attribute__((aligned(1024))) uint8_t stages[2 * STAGE_BYTES];
     uint8_t* const lds_a0 = stages;
     uint8_t* const lds_b0 = stages + A_BYTES;
@@ -333,7 +335,8 @@ dense_gemm_body_8w(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
     // Fragments live across k-tiles: the barrier that opens k-tile t + 1 sits TAIL steps before the end of k-tile t, where
     // every fragment of k-tile t is in registers; behind it the first fragments of k-tile t + 1 are fetched and the TAIL
     // steps still held are multiplied while those fetches are under way.
-    constexpr int TAIL = 2, NS = 4;
+    // NS slots for weight fragments, step s in slot s % NS: a divisor of STEPS, so that a step's slot is the same in every k-tile
+    constexpr int TAIL = 2, NS = STEPS % 4 == 0 ? 4 : (STEPS % 5 == 0 ? 5 : (STEPS % 7 == 0 ? 7 : STEPS));
     static_assert(STEPS % NS == 0 && TAIL + 1 < NS && NUM_COPIES <= STEPS - TAIL);
     Frag nf[NS], mf[2][TM];           // weight fragments, step s in slot s % NS; activation fragments of the two K halves
     auto mma = [&](int s) {
@@ -419,17 +422,22 @@ dense_gemm_body_8w(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
 
         // Epilogue: the 4 registers of atom (i, j) are n = n_slab + 16 i + 4 g + {0..3} of row m = m_slab + 16 j + col.
         // Stored straight from there a wave instruction would write 16 rows x 32 bytes; instead each wave turns its slab
-        // round through the stage that was consumed last, 16 rows at a time, and stores 4 rows x 256 consecutive bytes
-        // per instruction (16 bytes per lane). Rows are 272 bytes apart in LDS so that the 8-byte writes of 16 rows
-        // spread over the banks. The other stage is receiving the next tile meanwhile.
+        // round through the stage that was consumed last, 16 rows at a time, and stores whole row segments of 2 * WTN
+        // consecutive bytes, 16 bytes per lane: 4 rows x 256 bytes per instruction for the 256-wide tile. Rows are
+        // 2 * WTN + 16 bytes apart in LDS so that the 8-byte writes of 16 rows spread over the banks. The other stage is
+        // receiving the next tile meanwhile.
         const int m_slab = cur.m0 + wm * WTM, n_slab = cur.n0 + wn * WTN;
-        static_assert(WTM == 64 && WTN == 128 && sizeof(Elem) == 2, "the staged epilogue is laid out for 128 x 64 slabs");
+        static_assert(sizeof(Elem) == 2);
         if ((n % 8) == 0) {
-            constexpr int PITCH = 272;
+            constexpr int PITCH = 2 * WTN + 16;
+            // lanes per row segment; rows one store instruction covers (lanes beyond the last whole row sit idle when the
+            // segment length does not divide the wave); store instructions per 16 rows
+            constexpr int LANES_PER_ROW = WTN / 8, ROWS_PER_STORE = kWaveSize / LANES_PER_ROW, STORES = ceil_div(16, ROWS_PER_STORE);
+            static_assert((NW / 2) * 16 * PITCH <= A_BYTES && (NW / 2) * 16 * PITCH <= LDS_ROWS_B * kRowBytes);
             // every wave has read the last k-tile: they all passed the barrier inside its k_step with its fragments in registers
-            uint8_t* region = (wave < 4 ? a_last : b_last) + (wave % 4) * (16 * PITCH);
+            uint8_t* region = (wave < NW / 2 ? a_last : b_last) + (wave % (NW / 2)) * (16 * PITCH);
             const __amdgpu_buffer_rsrc_t rsrc_c = make_out_rsrc(C + size_t(cur.m0) * n + cur.n0);
-            const int r4 = lane / 16, c = lane % 16;
+            const int r_in = lane / LANES_PER_ROW, c = lane % LANES_PER_ROW;
             const int nn = n_slab + 8 * c;
 #pragma unroll
             for (int j = 0; j < TM; ++j) {
@@ -437,11 +445,13 @@ dense_gemm_body_8w(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
                 for (int i = 0; i < TN; ++i)
                     *reinterpret_cast<decltype(pack4(acc[0][0], Elem{}))*>(region + col * PITCH + (16 * i + 4 * g) * 2) = pack4(acc[i][j], Elem{});
 #pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    const int row = 4 * q + r4, mm = m_slab + 16 * j + row;
-                    const i32x4 v = *reinterpret_cast<const i32x4*>(region + row * PITCH + c * 16);
-                    if (mm < m && nn < n)
-                        buffer_store_16(v, rsrc_c, uint32_t((wm * WTM + 16 * j + row) * n + wn * WTN + 8 * c) * 2u, stream_out);
+                for (int q = 0; q < STORES; ++q) {
+                    const int row = ROWS_PER_STORE * q + r_in, mm = m_slab + 16 * j + row;
+                    if (r_in < ROWS_PER_STORE && row < 16) {
+                        const i32x4 v = *reinterpret_cast<const i32x4*>(region + row * PITCH + c * 16);
+                        if (mm < m && nn < n)
+                            buffer_store_16(v, rsrc_c, uint32_t((wm * WTM + 16 * j + row) * n + wn * WTN + 8 * c) * 2u, stream_out);
+                    }
                 }
             }
         } else {
@@ -523,10 +533,9 @@ template <typename Atom, typename Elem, int BLOCK_M, int BLOCK_N, int STAGES = D
 inline hipError_t launch_dense(int m, int n, int k, const void* a, const void* b, void* c, hipStream_t stream, int num_sms = 0) {
     if (m == 0 || n == 0) return hipSuccess;
     if (hipError_t e = check_dense_args(m, n, k, a, b, c, BLOCK_M, BLOCK_N); e != hipSuccess) return e;
-    using Cfg = DenseTileConfig<BLOCK_M, BLOCK_N>;
     const XcdTileScheduler<> sched(m, n, BLOCK_M, BLOCK_N);
     const int slots = sched.grid_size();
-    if constexpr (BLOCK_M == 256 && BLOCK_N == 256 && STAGES == 2) {
+    if constexpr (BLOCK_M == 256 && STAGES == 2) {
         // The largest tile runs the 8-wave kernel on 16x16x32 atoms: level with the 4-wave one where the chip's power
         // limit sets the pace (8192^3), 13 % faster at 4096^3.
         // persistent: one workgroup per CU (a multiple of the 8 XCDs, so a workgroup's tiles stay on one XCD's range),
@@ -541,6 +550,7 @@ inline hipError_t launch_dense(int m, int n, int k, const void* a, const void* b
                                dim3(8 * kWaveSize), 0, stream, static_cast<const uint8_t*>(a), static_cast<const uint8_t*>(b),
                                static_cast<Elem*>(c), m, n, k);
     } else {
+        using Cfg = DenseTileConfig<BLOCK_M, BLOCK_N>;
         const int grid = capped_grid(slots, num_sms, device_cu_count());
         if constexpr (__is_same(Elem, _Float16))
             hipLaunchKernelGGL((fp16_gemm_cute<BLOCK_M, BLOCK_N, STAGES>), dim3(grid),

@@ -12,7 +12,11 @@ from typing import List, Tuple
 from .utils import ceil_div
 
 # (BLOCK_M, BLOCK_N): relative time per unit of tile area. Bigger tiles reuse operands better.
-_DENSE_TILES = {(256, 256): 1.00, (256, 128): 1.12, (128, 256): 1.12, (128, 128): 1.30, (64, 128): 1.7, (64, 64): 2.4}
+# Dense tiles: 256 rows x {256, 224, 192, 160} columns run the 8-wave kernel (two LDS stages), the others the 4-wave kernel
+# with a ring of stages. Costs of the tiles from 128 x 128 up are measured: time per output of a problem that fills four
+# whole rounds of 256 compute units with the tile (8192 x 32 BLOCK_N x 8192), relative to 256 x 256.
+_DENSE_TILES = {(256, 256): 1.00, (256, 224): 1.05, (256, 192): 1.10, (256, 160): 1.19, (256, 128): 1.29, (128, 256): 1.28,
+                (128, 128): 1.46, (64, 128): 1.94, (64, 64): 2.7}
 _FP8_TILES = {(256, 256): 1.00, (256, 128): 1.12, (128, 256): 1.12, (128, 128): 1.30, (64, 128): 1.7, (64, 64): 2.2,
               (64, 32): 3.0, (64, 16): 4.5}
 
@@ -52,8 +56,11 @@ def get_best_fp8_config(m: int, n: int, k: int, num_cus: int) -> Tuple[int, int]
 
 
 def get_dense_num_stages(block_m: int, block_n: int) -> int:
-    """LDS stages of the dense kernel for a tile: as many as the 160 KB LDS holds, at most 8
-    (`DenseTileConfig::MAX_STAGES` in bf16_gemm.hpp): 2 for 256 x 256, 3 for 128 x 256, ... 8 for 64 x 64."""
+    """LDS stages of the dense kernel for a tile: 2 for the tiles of the 8-wave kernel (256 rows, more than 128 columns),
+    else as many as the 160 KB LDS holds, at most 8 (`DenseTileConfig::MAX_STAGES` in bf16_gemm.hpp): 3 for 128 x 256,
+    ... 8 for 64 x 64."""
+    if block_m == 256 and block_n > 128:
+        return 2            # the 8-wave kernel, whatever the width
     return min(8, 160 * 1024 // ((block_m + block_n) * 128))
 
 
