@@ -16,7 +16,7 @@ struct TileCost { int bm, bn; double per_area; };
 constexpr TileCost kDenseTiles[] = {{256, 256, 1.00}, {256, 224, 1.05}, {256, 192, 1.10}, {256, 160, 1.19}, {256, 128, 1.29}, {128, 256, 1.28},
                                     {128, 128, 1.46}, {64, 128, 1.94}, {64, 64, 2.7}};
 constexpr TileCost kFp8Tiles[]   = {{256, 256, 1.00}, {256, 128, 1.12}, {128, 256, 1.12}, {128, 128, 1.30}, {64, 128, 1.7}, {64, 64, 2.2},
-                                    {64, 32, 3.0}, {64, 16, 4.5}};
+                                    {64, 32, 3.0}, {32, 32, 4.0}};
 
 template <int COUNT>
 void pick(const TileCost (&tiles)[COUNT], int m, int n, int num_cus, int* bm, int* bn) {
@@ -116,7 +116,7 @@ int yan_gemm_fp8_fp8_bf16_nt(const void* lhs, const float* lhs_scales, long long
         return int(yan::Gemm<0, 0, BM, BN, 128, 1, yan::Fp8TileConfig<BM, BN>::MAX_RING_STAGES, 1, yan::GemmType::Normal>::run_sized(                          \
             o, lhs, lhs_scales, int(lhs_scales_stride_m), int(lhs_scales_stride_k), rhs, rhs_scales, m, n, k, s, num_sms, 0));
     YAN_FP8_CASE(256, 256) YAN_FP8_CASE(256, 128) YAN_FP8_CASE(128, 256) YAN_FP8_CASE(128, 128) YAN_FP8_CASE(64, 128) YAN_FP8_CASE(64, 64)
-    YAN_FP8_CASE(64, 32) YAN_FP8_CASE(64, 16)
+    YAN_FP8_CASE(64, 32) YAN_FP8_CASE(32, 32)
 #undef YAN_FP8_CASE
     return int(hipErrorInvalidValue);
 }

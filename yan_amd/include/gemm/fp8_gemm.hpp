@@ -52,12 +52,15 @@ struct Fp8TileConfig {
     static constexpr int  LDS_BYTES = 2 * (LDS_ROWS_A + LDS_ROWS_B) * kRowBytes;
     static_assert(LDS_BYTES <= 160 * 1024, "two stages must fit the 160 KB LDS");
     // Ring of more than two stages (tiles below 256 x 256, where one k-tile in flight does not cover the memory
-    // latency of an operand-streaming problem): a stage also carries the k-tile's BLOCK_M activation scales.
+    // latency of an operand-streaming problem): a stage also carries the k-tile's activation scales (one copy
+    // instruction moves 64 of them; a 32-row tile uses the first 32).
     static constexpr int  RING_SCALE_BYTES = ceil_div(BLOCK_M * 4, 1024) * 1024;
     static constexpr int  RING_STAGE_BYTES = (LDS_ROWS_A + LDS_ROWS_B) * kRowBytes + RING_SCALE_BYTES;
-    static constexpr bool RING_CAPABLE = BLOCK_M % 64 == 0 && (BLOCK_M / 8) % NUM_WAVES == 0 && BLOCK_N % 16 == 0;
-    // At most 8 stages, 12 for the narrow tiles of the decode shapes: those stream 16 or 32 weight rows per workgroup, are
-    // bound by the latency of their loads and gain from every k-tile more in flight (a stage is only 13 KB there).
+    static constexpr bool RING_CAPABLE = BLOCK_M % 32 == 0 && (BLOCK_M / 8) % NUM_WAVES == 0 && BLOCK_N % 16 == 0;
+    // At most 8 stages, 12 for the narrow tiles of the decode shapes (16 or 32 weight rows per workgroup): those have next
+    // to nothing to compute per k-tile and run at the rate their compute unit takes bytes in, which needs many k-tiles in
+    // flight (a stage is only 9 to 13 KB there). Measured with every unit pulling: about 60 GB/s per unit whatever the
+    // tile, so the tile to prefer is the one that moves the fewest bytes per output, 32 x 32 for a 64-row problem.
     static constexpr int  RING_DEPTH_CAP = BLOCK_N <= 32 ? 12 : 8;
     static constexpr int  MAX_RING_STAGES = RING_CAPABLE ? (160 * 1024 / RING_STAGE_BYTES < RING_DEPTH_CAP ? 160 * 1024 / RING_STAGE_BYTES : RING_DEPTH_CAP) : 2;
 };
@@ -293,7 +296,7 @@ fp8_gemm_tile(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_sca
     // copies would make the in-order counter wait for every older copy): every wave copies one 64-row part of them
     // with one full-width instruction; waves that share a part write the same bytes twice.
     constexpr int STAGE_BYTES = Cfg::RING_STAGE_BYTES, A_BYTES = Cfg::LDS_ROWS_A * kRowBytes, TILE_BYTES = A_BYTES + Cfg::LDS_ROWS_B * kRowBytes;
-    constexpr int OPS = StA::PASSES + StB::PASSES + 1, SCALE_PARTS = BLOCK_M / 64;
+    constexpr int OPS = StA::PASSES + StB::PASSES + 1, SCALE_PARTS = BLOCK_M >= 64 ? BLOCK_M / 64 : 1;
     static_assert(Cfg::RING_CAPABLE && (STAGES - 2) * OPS <= 63 && STAGES * STAGE_BYTES <= 160 * 1024);
     __shared__ __attribute__((aligned(1024))) uint8_t ring[STAGES * STAGE_BYTES];
     const uint32_t scale_voff = uint32_t(m0 + lane) * sa_stride_m * 4;

@@ -18,7 +18,7 @@ from .utils import ceil_div
 _DENSE_TILES = {(256, 256): 1.00, (256, 224): 1.05, (256, 192): 1.10, (256, 160): 1.19, (256, 128): 1.29, (128, 256): 1.28,
                 (128, 128): 1.46, (64, 128): 1.94, (64, 64): 2.7}
 _FP8_TILES = {(256, 256): 1.00, (256, 128): 1.12, (128, 256): 1.12, (128, 128): 1.30, (64, 128): 1.7, (64, 64): 2.2,
-              (64, 32): 3.0, (64, 16): 4.5}
+              (64, 32): 3.0, (32, 32): 4.0}
 
 
 def rank_tiles(m: int, n: int, num_cus: int, table, groups: int = 1) -> List[Tuple[float, Tuple[int, int]]]:
@@ -66,11 +66,11 @@ def get_dense_num_stages(block_m: int, block_n: int) -> int:
 
 def get_fp8_num_stages(block_m: int, block_n: int) -> int:
     """LDS stages of the tiled FP8 kernel for a tile: a ring as deep as the 160 KB LDS allows, at most 8, or 12 for the
-    tiles of 16 and 32 weight rows that run the decode shapes (`Fp8TileConfig::MAX_RING_STAGES` in fp8_gemm.hpp): 2 for
-    256 x 256, 3 for 256 x 128 and 128 x 256, 8 for 64 x 64, 12 for 64 x 16. Tiles below 256 x 256 are what the cost model picks when a problem is short on work per CU, i.e. bound by
+    tiles of 32 weight rows that run the decode shapes (`Fp8TileConfig::MAX_RING_STAGES` in fp8_gemm.hpp): 2 for
+    256 x 256, 3 for 256 x 128 and 128 x 256, 8 for 64 x 64, 12 for 64 x 32 and 32 x 32. Tiles below 256 x 256 are what the cost model picks when a problem is short on work per CU, i.e. bound by
     operand streaming, and there one k-tile of prefetch does not cover the memory latency."""
     waves = 8 if block_m * block_n >= 256 * 128 else 4
-    capable = block_m % 64 == 0 and (block_m // 8) % waves == 0 and block_n % 16 == 0
+    capable = block_m % 32 == 0 and (block_m // 8) % waves == 0 and block_n % 16 == 0
     if not capable:
         return 2
     rows = ceil_div(block_m, 8 * waves) * 8 * waves + ceil_div(block_n, 8 * waves) * 8 * waves      # whole copy passes
