@@ -419,7 +419,7 @@ fp8_gemm_tile(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_sca
     if (staged) {
         if constexpr (kStagedEpilogue) {
             constexpr int PITCH = Cfg::WTN * 2 + 16, REGION = 16 * PITCH;
-            constexpr int LANES_PER_ROW = Cfg::WTN / 8, ROWS_PER_STORE = kWaveSize / LANES_PER_ROW, STORES = 16 / ROWS_PER_STORE;
+            constexpr int LANES_PER_ROW = Cfg::WTN / 8, ROWS_PER_STORE = kWaveSize / LANES_PER_ROW, STORES = ceil_div(16, ROWS_PER_STORE);
             static_assert(STORES >= 1 && (NW / 2) * REGION <= Cfg::LDS_ROWS_A * kRowBytes && (NW / 2) * REGION <= Cfg::LDS_ROWS_B * kRowBytes);
             // every wave has read the last k-tile (a bare barrier: __syncthreads() would also wait for the copies still
             // on their way into the other stages, which nobody will read)
@@ -444,7 +444,8 @@ fp8_gemm_tile(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_sca
                 for (int q = 0; q < STORES; ++q) {
                     const int row = ROWS_PER_STORE * q + r_in, mm = m_slab + 16 * j + row;
                     const i32x4 v = *reinterpret_cast<const i32x4*>(region + row * PITCH + c * 16);
-                    bool live = mm < m && nn < N;
+                    // a slab width that does not divide 64 lanes leaves the last lanes, and rows past 16, without work
+                    bool live = mm < m && nn < N && r_in < ROWS_PER_STORE && row < 16;
                     if constexpr (kTwoHalves) live = live && mm >= pass_lo[pass] && mm < pass_hi[pass];
                     if (live) buffer_store_16(v, rsrc_out, uint32_t((mm - m0) * N + nn - n0) * 2u, stream_out);
                 }
