@@ -215,6 +215,21 @@ CAPPED_SHAPES = [(2048, 4096, 1024), (512, 4096, 2048), (300, 2112, 640)]
 TUNED_SHAPES = [(4096, 5120, 5120), (2048, 7168, 7168)]
 
 
+# FP8 tiles the cost model does not offer but the kernel supports, built through explicit keys: their wave slabs are
+# 112 and 96 columns wide, which straddle the 128-wide weight-scale blocks (two scale products per k-tile and a select per
+# row of atoms) and do not divide the 64 lanes of the staged epilogue's row stores. (BLOCK_M, BLOCK_N, (m, n, k)).
+FP8_EXPLICIT_TILE_CASES = [(256, 224, (600, 1344, 640)), (256, 224, (300, 1000, 384)), (256, 192, (520, 1156, 512))]
+
+
+def fp8_explicit_tile_plan(block_m: int, block_n: int, n: int, k: int):
+    """(name, keys, arg_defs, template) of the FP8 JIT kernel with this tile and token-contiguous scales."""
+    from yan_amd.jit_kernels import gemm
+    from yan_amd.jit_kernels.heuristics import get_fp8_num_stages
+    keys = {'N': n, 'K': k, 'BLOCK_M': block_m, 'BLOCK_N': block_n, 'NUM_STAGES': get_fp8_num_stages(block_m, block_n),
+            'NUM_TMA_MULTICAST': 1}
+    return 'gemm_fp8_fp8_bf16_nt', keys, gemm.arg_defs, gemm.template
+
+
 def jit_kernels_in_use(num_cus: int = 256):
     """(name, arg_defs, code) of every distinct JIT kernel the shapes above, and the quantisers select."""
     from yan_amd.jit import cpp_format, generate
@@ -245,6 +260,11 @@ def jit_kernels_in_use(num_cus: int = 256):
         for cus in (num_cus, NUM_SMS_CAP):
             name, keys, arg_defs, _, code_template = gemm.fp8_kernel_plan(m, n, k, cus, False)
             add(name, arg_defs, gemm.includes, code_template, keys)
+    for block_m, block_n, (m, n, k) in FP8_EXPLICIT_TILE_CASES:
+        name, keys, arg_defs, code_template = fp8_explicit_tile_plan(block_m, block_n, n, k)
+        add(name, arg_defs, gemm.includes, code_template, keys)
+        name, keys, arg_defs, _, code_template = gemm.fp8_kernel_plan(m, n, k, num_cus, True)
+        add(name, arg_defs, gemm.includes, code_template, keys)
     for m, n, k in TUNED_SHAPES:
         name, keys, space, arg_defs = bf16_gemm.dense_tuning_plan(m, n, k, torch.bfloat16, num_cus)
         for extra in space:

@@ -618,6 +618,27 @@ def test_entry_points_pick_the_fastest_of_three_tiles_when_asked(m, n, k, monkey
     assert torch.equal(again, out)
 
 
+@pytest.mark.parametrize('block_m,block_n,shape', testing.FP8_EXPLICIT_TILE_CASES)
+def test_fp8_tiles_whose_slabs_straddle_weight_scale_blocks(block_m, block_n, shape):
+    """256 x 224 and 256 x 192 tiles, built through the reference's keys (yan/jit_kernels/gemm.py:9-16): wave slabs of 112
+    and 96 columns cross the boundaries of the 128-wide weight-scale blocks and do not divide the 64 lanes of the row
+    stores. Same bits as the tile the cost model picks (every tile sums the K blocks in the same order), parity against
+    the oracle, ragged edges left alone."""
+    from yan_amd import jit
+    m, n, k = shape
+    _announce('explicit fp8 tile', block_m, block_n, m, n, k)
+    (a8, sa), (b8, sb), out = testing.make_fp8_case(m, n, k, seed=11, device='cuda', col_major_scales=True)
+    yan.gemm_fp8_fp8_bf16_nt((a8, sa), (b8, sb), out)
+    name, keys, arg_defs, code_template = testing.fp8_explicit_tile_plan(block_m, block_n, n, k)
+    runtime = jit.build(name, arg_defs, jit.generate(yan.gemm.includes, arg_defs, jit.cpp_format(code_template, keys)))
+    padded = torch.full((m + 3, n), 7.0, dtype=torch.bfloat16, device='cuda')
+    rc = runtime(a8, sa, b8, sb, padded, m, torch.cuda.current_stream(), yan.get_num_sms(), 0)
+    assert rc == 0
+    torch.cuda.synchronize()
+    assert torch.equal(padded[:m], out) and bool((padded[m:] == 7.0).all())
+    assert oracle.calc_diff(_np(out), _fp8_ref(a8, sa, b8, sb)) < 1e-5
+
+
 # ----------------------------------------------------------------------------- quantisers in front of the FP8 GEMM
 def _oracle_per_token(x):
     q, s_ = oracle.per_token_cast_to_fp8(x.float().numpy())
