@@ -178,6 +178,78 @@ def test_tile_scheduler_visits_every_tile_once_and_walks_cover_every_slot(tmp_pa
     assert int(done.stdout.split()[1]) > 400
 
 
+@pytest.mark.parametrize('shape,dtype_name', [((8192, 8192, 8192), 'bfloat16'), ((4096, 5120, 5120), 'bfloat16'), ((8192, 8192, 8192), 'half')])
+def test_tied_accumulators_of_the_8_wave_kernel_stay_where_the_mfmas_left_them(tmp_path, shape, dtype_name):
+    """The 8-wave dense kernel writes its MFMAs as asm statements whose destination is their own addend. The compiler does
+    not know how long such an instruction takes, so nothing but MFMAs may touch an accumulator register between the first
+    and the last MFMA of the main loop (a compiler-made copy right behind an MFMA would read a sum that is not there yet),
+    and what reads them first afterwards must sit behind the wait states written in the source. Checked on the generated
+    code: compiled for the device only, no GPU needed."""
+    import re
+    import subprocess
+    from yan_amd.jit import cpp_format, generate
+    from yan_amd.jit.compiler import get_hipcc_compiler, get_jit_include_dir, get_offload_arch
+    from yan_amd.jit_kernels import bf16_gemm
+    dtype = getattr(torch, dtype_name)
+    _, keys, arg_defs = bf16_gemm.dense_kernel_plan(*shape, dtype, 256, 0)
+    assert keys['BLOCK_M'] == 256 and keys['NUM_STAGES'] == 2             # the 8-wave kernel
+    src, asm = tmp_path / 'kernel.cu', tmp_path / 'kernel.s'
+    src.write_text(generate(bf16_gemm.includes, arg_defs, cpp_format(bf16_gemm.template, keys)))
+    subprocess.check_call([get_hipcc_compiler()[0], '-x', 'hip', '--cuda-device-only', '-S', '-std=c++20', '-O3',
+                           f'--offload-arch={get_offload_arch()}', '-Xclang', '-target-feature', '-Xclang', '-packed-fp32-ops',
+                           f'-I{get_jit_include_dir()}', str(src), '-o', str(asm)])
+    text = asm.read_text()
+    assert re.search(r'\.private_segment_fixed_size:\s+0\b', text), 'the kernel spills'
+    # instructions and labels of the kernel, in text order
+    lines = [line.split(';')[0].strip() for line in text.split('\n')]
+    lines = [line for line in lines if line and (line.endswith(':') or not line.startswith(('.', '//')))]
+
+    def regs(operand_text):
+        found = set()
+        for lo, hi in re.findall(r'\bv\[(\d+):(\d+)\]', operand_text):
+            found.update(range(int(lo), int(hi) + 1))
+        found.update(int(r) for r in re.findall(r'\bv(\d+)\b', operand_text))
+        return found
+
+    mfma = re.compile(r'^v_mfma_f32_16x16x32_(?:bf16|f16) (v\[\d+:\d+\]), (v\[\d+:\d+\]), (v\[\d+:\d+\]), (v\[\d+:\d+\])')
+    where = [i for i, line in enumerate(lines) if mfma.match(line)]
+    assert len(where) >= 2 * 2 * keys['BLOCK_N'] // 32 * 4          # at least the steps of two k-tiles
+    acc = set()
+    for i in where:
+        dst, a, b, c = mfma.match(lines[i]).groups()
+        assert dst == c, lines[i]                                    # accumulates in place
+        acc |= regs(dst)
+    assert len(acc) == 256 * keys['BLOCK_N'] // 512                  # one register per output of the wave's slab
+    for i in where:
+        _, a, b, _ = mfma.match(lines[i]).groups()
+        assert not (regs(a) | regs(b)) & acc, lines[i]
+
+    def mfma_in_flight_before(i):
+        """An MFMA less than 20 instructions up the straight-line path that ends at instruction i, with no `s_nop 15`
+        pair between; a path stops at a label whose predecessor in the text ends with an unconditional branch."""
+        nops = 0
+        for back in range(1, 21):
+            line = lines[i - back]
+            if line.endswith(':'):
+                if lines[i - back - 1].startswith('s_branch'):
+                    return False
+                continue
+            if line == 's_nop 15':
+                nops += 1
+            if mfma.match(line):
+                return nops < 2
+        return False
+    for i in range(where[0], len(lines)):
+        line = lines[i]
+        if mfma.match(line) or line.endswith(':') or line.startswith('s_') or not regs(line) & acc:
+            continue
+        assert not mfma_in_flight_before(i), f'{line} touches an accumulator right behind an MFMA'
+    # and the epilogue's first read of a sum sits behind the wait states written in the source
+    after = lines[where[-1] + 1:]
+    first_use = next(i for i, line in enumerate(after) if not line.endswith(':') and not line.startswith('s_') and regs(line) & acc)
+    assert sum(1 for line in after[:first_use] if line == 's_nop 15') >= 2, 'the sums are read before the last MFMAs have retired'
+
+
 def test_tuner_rebuilds_when_a_callers_dict_changes_between_calls(monkeypatch):
     """A caller that reuses one mutable keys dict (the loop of the reference's tests/test_jit.py) gets the kernel of the
     keys it passes, not of the keys it passed last time; only read-only plan keys take the same-object short cut."""
