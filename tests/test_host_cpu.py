@@ -51,6 +51,18 @@ def test_tile_heuristics_fill_256_cus():
     assert ranked == sorted(ranked) and len(ranked) == len(heuristics._FP8_TILES)
 
 
+def test_fp8_shapes_of_the_gpu_suite_reach_every_tile_of_the_cost_table():
+    import harness
+    for shape, tile in harness.FP8_TILE_OF_SHAPE.items():
+        assert shape in harness.FP8_TEST_SHAPES + harness.FP8_SIDE_SHAPES
+        assert heuristics.get_fp8_tile(*shape, 256) == tile, shape
+    assert set(harness.FP8_TILE_OF_SHAPE.values()) == set(heuristics._FP8_TILES)
+    # two full rounds of 256 x 160 tiles beat 1.25 rounds of 256 x 256 tiles
+    assert heuristics.get_best_fp8_config(4096, 5120, 5120, 256) == (256, 160)
+    # the grouped layouts keep to widths of 64, 128 and 256
+    assert heuristics.get_best_grouped_fp8_config(4096, 5120, 5120, 256, 1, 128, 4)[1] in (64, 128, 256)
+
+
 def test_dense_shapes_of_the_gpu_suite_reach_every_tile_of_the_8_wave_kernel():
     """A change of the cost table must not silently take the 256 x {160, 192, 224} tiles out of the parity tests."""
     import harness
