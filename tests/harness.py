@@ -158,11 +158,14 @@ DENSE_TEST_SHAPES = [
     (2900, 5000, 64),            # same with a single k-tile
     # the narrower tiles of the 8-wave kernel: 256 x 160, 256 x 224, 256 x 192, each once whole and once ragged in m, n and k
     (4096, 5120, 512), (4000, 5000, 520), (2048, 7168, 256), (2047, 7100, 264), (4096, 6144, 256), (4090, 6100, 72),
+    # the 192-wide tiles of the ring kernel (wave slabs of 96 columns), whole and ragged
+    (2048, 2112, 264), (2000, 2100, 136), (1024, 2112, 264), (1000, 2100, 72),
 ]
 # (shape, tile the cost model must pick): the shapes above exist for these tiles
 DENSE_TILE_OF_SHAPE = {(4096, 5120, 512): (256, 160), (4000, 5000, 520): (256, 160), (2048, 7168, 256): (256, 224),
                        (2047, 7100, 264): (256, 224), (4096, 6144, 256): (256, 192), (4090, 6100, 72): (256, 192),
-                       (3000, 5000, 1000): (256, 256), (8192, 8192, 8192): (256, 256)}
+                       (3000, 5000, 1000): (256, 256), (8192, 8192, 8192): (256, 256),
+                       (2048, 2112, 264): (128, 192), (2000, 2100, 136): (128, 192), (1024, 2112, 264): (64, 192), (1000, 2100, 72): (64, 192)}
 # (m, n, k) of the reference's own dense test (tests/test_cute.py:21-22: m in (256, 4096) x six (k, n) pairs)
 REFERENCE_DENSE_TEST_SHAPES = [(m, n, k) for m in (256, 4096)
                                for k, n in ((5120, 5120), (1536, 24576), (512, 32768), (16384, 7168), (7168, 2048), (2048, 7168))]

@@ -64,12 +64,14 @@ def test_fp8_shapes_of_the_gpu_suite_reach_every_tile_of_the_cost_table():
 
 
 def test_dense_shapes_of_the_gpu_suite_reach_every_tile_of_the_8_wave_kernel():
-    """A change of the cost table must not silently take the 256 x {160, 192, 224} tiles out of the parity tests."""
+    """A change of the cost table must not silently take the 256 x {160, 192, 224} tiles, or the 192-wide ring tiles, out of the
+    parity tests."""
     import harness
     for shape, tile in harness.DENSE_TILE_OF_SHAPE.items():
+        assert shape in harness.DENSE_TEST_SHAPES
         assert heuristics.get_best_dense_config(*shape, 256) == tile, shape
-        assert heuristics.get_dense_num_stages(*tile) == 2
-    assert {t for t in harness.DENSE_TILE_OF_SHAPE.values()} == {(256, 160), (256, 192), (256, 224), (256, 256)}
+        assert heuristics.get_dense_num_stages(*tile) == (2 if tile[0] == 256 else {(128, 192): 4, (64, 192): 5}[tile])
+    assert {t for t in harness.DENSE_TILE_OF_SHAPE.values()} == {(256, 160), (256, 192), (256, 224), (256, 256), (128, 192), (64, 192)}
 
 
 def test_kernel_plans_keep_reference_keys_and_argument_order():

@@ -14,7 +14,7 @@ struct TileCost { int bm, bn; double per_area; };
 
 // Same tables and cost model as yan_amd/jit_kernels/heuristics.py (a CPU test keeps the two in step).
 constexpr TileCost kDenseTiles[] = {{256, 256, 1.00}, {256, 224, 1.05}, {256, 192, 1.10}, {256, 160, 1.19}, {256, 128, 1.29}, {128, 256, 1.28},
-                                    {128, 128, 1.46}, {64, 128, 1.94}, {64, 64, 2.7}};
+                                    {128, 192, 1.39}, {128, 128, 1.46}, {64, 192, 1.9}, {64, 128, 1.94}, {64, 64, 2.7}};
 constexpr TileCost kFp8Tiles[]   = {{256, 256, 1.00}, {256, 192, 1.12}, {256, 160, 1.28}, {256, 128, 1.34}, {128, 256, 1.34}, {128, 128, 1.79},
                                     {64, 128, 2.4}, {64, 64, 3.8}, {64, 32, 4.8}, {32, 32, 7.0}};
 
@@ -72,7 +72,8 @@ int dense(int m, int n, int k, const void* a, const void* b, void* c, void* stre
 #define YAN_DENSE_CASE(BM, BN) if (bm == BM && bn == BN) return int(yan::launch_dense<Atom, Elem, BM, BN>(m, n, k, a, b, c, s));
 #define YAN_DENSE_CASE_8W(BM, BN) if (bm == BM && bn == BN) return int(yan::launch_dense<Atom, Elem, BM, BN, 2>(m, n, k, a, b, c, s));
     YAN_DENSE_CASE_8W(256, 256) YAN_DENSE_CASE_8W(256, 224) YAN_DENSE_CASE_8W(256, 192) YAN_DENSE_CASE_8W(256, 160)
-    YAN_DENSE_CASE(256, 128) YAN_DENSE_CASE(128, 256) YAN_DENSE_CASE(128, 128) YAN_DENSE_CASE(64, 128) YAN_DENSE_CASE(64, 64)
+    YAN_DENSE_CASE(256, 128) YAN_DENSE_CASE(128, 256) YAN_DENSE_CASE(128, 192) YAN_DENSE_CASE(128, 128) YAN_DENSE_CASE(64, 192)
+    YAN_DENSE_CASE(64, 128) YAN_DENSE_CASE(64, 64)
 #undef YAN_DENSE_CASE
 #undef YAN_DENSE_CASE_8W
     return int(hipErrorInvalidValue);
@@ -193,6 +194,6 @@ int yan_gemm_select_tile(int op, int m, int n, int k, int num_cus, int* block_m,
     return 0;
 }
 
-const char* yan_gemm_version(void) { return "yan-gemm gfx950 9 dense + 7 fp32 + 10 fp8 tile variants + 1 weight-streaming fp8 variant + 12 grouped fp8 variants + 4 quantiser kernels"; }
+const char* yan_gemm_version(void) { return "yan-gemm gfx950 11 dense + 7 fp32 + 10 fp8 tile variants + 1 weight-streaming fp8 variant + 12 grouped fp8 variants + 4 quantiser kernels"; }
 
 } // extern "C"

@@ -182,7 +182,9 @@ dense_gemm_body(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, El
     const bool stream_out = size_t(m) * n * sizeof(Elem) > (size_t(32) << 20);
     const __amdgpu_buffer_rsrc_t rsrc_c = make_out_rsrc(C + size_t(m0) * n + n0);
     constexpr int PITCH = Cfg::WTN * 2 + 16, REGION = 32 * PITCH;
-    constexpr int LANES_PER_ROW = Cfg::WTN / 8, ROWS_PER_STORE = kWaveSize / LANES_PER_ROW, STORES = 32 / ROWS_PER_STORE;
+    // lanes per row segment; rows one store instruction covers (a slab width that does not divide the wave leaves the last
+    // lanes idle); store instructions per 32 rows
+    constexpr int LANES_PER_ROW = Cfg::WTN / 8, ROWS_PER_STORE = kWaveSize / LANES_PER_ROW, STORES = ceil_div(32, ROWS_PER_STORE);
     static_assert(NW * REGION <= STAGE_BYTES && STORES >= 1 && sizeof(Elem) == 2);
     if ((n % 8) == 0) {
         // every wave has read the last k-tile (a bare barrier: nothing here depends on the copies still under way)
@@ -206,7 +208,7 @@ dense_gemm_body(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, El
             for (int s = 0; s < STORES; ++s) {
                 const int row = ROWS_PER_STORE * s + r_in, m_in_tile = wm * Cfg::WTM + 32 * j + row;
                 const i32x4 v = *reinterpret_cast<const i32x4*>(region + row * PITCH + c * 16);
-                if (m0 + m_in_tile < m && n0 + n_in_tile < n)
+                if (r_in < ROWS_PER_STORE && row < 32 && m0 + m_in_tile < m && n0 + n_in_tile < n)
                     buffer_store_16(v, rsrc_c, uint32_t(m_in_tile * n + n_in_tile) * 2u, stream_out);
             }
         }

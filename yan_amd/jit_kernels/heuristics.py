@@ -15,8 +15,11 @@ from .utils import ceil_div
 # Dense tiles: 256 rows x {256, 224, 192, 160} columns run the 8-wave kernel (two LDS stages), the others the 4-wave kernel
 # with a ring of stages. Costs of the tiles from 128 x 128 up are measured: time per output of a problem that fills four
 # whole rounds of 256 compute units with the tile (8192 x 32 BLOCK_N x 8192), relative to 256 x 256.
+# 128 x 192 and 64 x 192 (ring kernel, wave slabs 96 columns wide) are for problems that leave most compute units idle with
+# 256-wide tiles and need two rounds with 128-wide ones (2048 x 2112 x 7168: 144 tiles of 128 x 256 run 85 us, 176 of 128 x 192 68 us).
+# With this table the pick is within 2 % of the fastest tile on 67 shapes swept with every tile forced in turn.
 _DENSE_TILES = {(256, 256): 1.00, (256, 224): 1.05, (256, 192): 1.10, (256, 160): 1.19, (256, 128): 1.29, (128, 256): 1.28,
-                (128, 128): 1.46, (64, 128): 1.94, (64, 64): 2.7}
+                (128, 192): 1.39, (128, 128): 1.46, (64, 192): 1.9, (64, 128): 1.94, (64, 64): 2.7}
 # FP8 tiles: measured over 74 shapes (m = 17 ... 8192, n = 2048 ... 32768, k = 512 ... 16384) with every tile forced in turn;
 # with these costs the model's pick is within 1 % of the fastest tile on all of them. 256 x 192 and 256 x 160 are there for
 # problems whose 256 x 256 tiles leave a round of compute units partly empty (4096 x 5120 x 5120: 320 tiles, against 512
