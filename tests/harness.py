@@ -185,10 +185,11 @@ FP8_TEST_SHAPES = [
     (128, 4096, 7168), (512, 4096, 2048), (1024, 7168, 1024),
     # the 256-row tiles narrower than 256 columns, whole and ragged (FP8_TILE_OF_SHAPE below)
     (4096, 5120, 256), (4000, 5100, 384), (512, 24576, 256), (500, 24500, 384), (768, 10880, 256),
+    (1024, 2112, 256), (1000, 2100, 384),
 ]
 # Which tile the cost model picks for some of the shapes above on 256 compute units: a CPU test keeps this true, so that a
 # change of the cost table cannot silently take a tile out of the parity tests.
-FP8_TILE_OF_SHAPE = {(4096, 5120, 256): (256, 160), (4000, 5100, 384): (256, 160), (512, 24576, 256): (256, 192), (500, 24500, 384): (256, 192),
+FP8_TILE_OF_SHAPE = {(1024, 2112, 256): (64, 160), (1000, 2100, 384): (64, 160), (4096, 5120, 256): (256, 160), (4000, 5100, 384): (256, 160), (512, 24576, 256): (256, 192), (500, 24500, 384): (256, 192),
                      (768, 10880, 256): (256, 128), (4096, 7168, 7168): (256, 256), (4096, 2048, 7168): (128, 256), (1024, 4096, 7168): (128, 128),
                      (512, 4096, 2048): (64, 128), (257, 2112, 1024): (64, 64), (64, 7168, 2048): (64, 32), (64, 4096, 7168): (32, 32)}
 # Plain FP8 calls the grouped and quantiser tests make on the side (first group through the plain entry, quantise-then-

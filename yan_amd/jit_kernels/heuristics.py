@@ -23,9 +23,10 @@ _DENSE_TILES = {(256, 256): 1.00, (256, 224): 1.05, (256, 192): 1.10, (256, 160)
 # FP8 tiles: measured over 74 shapes (m = 17 ... 8192, n = 2048 ... 32768, k = 512 ... 16384) with every tile forced in turn;
 # with these costs the model's pick is within 1 % of the fastest tile on all of them. 256 x 192 and 256 x 160 are there for
 # problems whose 256 x 256 tiles leave a round of compute units partly empty (4096 x 5120 x 5120: 320 tiles, against 512
-# tiles of 256 x 160 = two full rounds, 13 % faster); 256 x 224 is supported by the kernel and never the cheapest.
+# tiles of 256 x 160 = two full rounds, 13 % faster), 64 x 160 likewise among the small tiles (1024 x 2112 x 7168: 224 tiles in one
+# round, 15 % faster than 136 tiles of 128 x 128); 256 x 224 is supported by the kernel and never the cheapest.
 _FP8_TILES = {(256, 256): 1.00, (256, 192): 1.12, (256, 160): 1.28, (256, 128): 1.34, (128, 256): 1.34, (128, 128): 1.79,
-              (64, 128): 2.4, (64, 64): 3.8, (64, 32): 4.8, (32, 32): 7.0}
+              (64, 160): 2.47, (64, 128): 2.4, (64, 64): 3.8, (64, 32): 4.8, (32, 32): 7.0}
 
 
 def rank_tiles(m: int, n: int, num_cus: int, table, groups: int = 1) -> List[Tuple[float, Tuple[int, int]]]:
