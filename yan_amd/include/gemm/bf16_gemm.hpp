@@ -6,13 +6,15 @@
 // the reference kernel (cute_gemm.cuh:14-260) is a 128x128x32 cp.async/ldmatrix/mma.sync pipeline with fp16
 // accumulation and no bounds handling. Here:
 //   * macro tile BLOCK_M x BLOCK_N x 64 (128-byte rows), staged HBM -> LDS with buffer_load ... lds (tile_io.hpp);
-//   * the 256 x 256 tile: two LDS stages, 8 waves (two per SIMD), each with a 128 x 64 slab of 16x16x32 MFMAs (128
-//     accumulator registers); while one wave of a SIMD issues copies or waits for a fragment the other keeps the
-//     matrix core busy, and the barrier between two k-tiles sits two steps before the end of the first, so that
-//     every wave still holds work when it has passed it (dense_gemm_body_8w);
-//   * the smaller tiles, which run problems bound by operand streaming: a ring of three to eight LDS stages, 4 waves,
-//     one per SIMD, each with a (BLOCK_N/WAVES_N) x (BLOCK_M/WAVES_M) slab of 32x32x16 MFMAs, up to 128 x 128 (256
-//     accumulator registers, which the compiler keeps in AGPRs) (dense_gemm_body);
+//   * tiles of 256 rows and 160 to 256 columns: two LDS stages, 8 waves (two per SIMD), each with a (BLOCK_N/2) x 64 slab
+//     of 16x16x32 MFMAs (128 accumulator registers for the 256-wide tile, tied to their instructions so that they stay
+//     where they are); while one wave of a SIMD issues copies or waits for a fragment the other keeps the matrix core
+//     busy, and the barrier between two k-tiles sits two steps before the end of the first, so that every wave still
+//     holds work when it has passed it; one workgroup per compute unit walks the tiles (dense_gemm_body_8w);
+//   * the smaller tiles (256 x 128 down to 64 x 64, widths of 64, 128, 192 and 256), which run problems bound by operand
+//     streaming: a ring of three to eight LDS stages, 4 waves, one per SIMD, each with a (BLOCK_N/WAVES_N) x
+//     (BLOCK_M/WAVES_M) slab of 32x32x16 MFMAs, up to 128 x 128 (256 accumulator registers, which the compiler keeps in
+//     AGPRs) (dense_gemm_body);
 //   * B rows feed the MFMA row operand and A rows the column operand, so a lane's four consecutive accumulator
 //     registers are four consecutive n of one m: contiguous in C;
 //   * fp32 accumulators, round-to-nearest-even on the way out;

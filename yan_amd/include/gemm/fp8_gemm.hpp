@@ -7,8 +7,9 @@
 //   * macro tile BLOCK_M x BLOCK_N x 128 (one scale block per k-tile, 128-byte rows); 8 waves, two per SIMD, for
 //     the tiles from 256 x 128 up, so one wave's scale arithmetic and LDS traffic hide under the other's MFMAs;
 //     4 waves below that;
-//   * HBM -> LDS with buffer_load ... lds (tile_io.hpp) into two LDS stages for the 256 x 256 tile and into a ring of
-//     3 to 8 stages for the smaller tiles, which run problems bound by operand streaming;
+//   * HBM -> LDS with buffer_load ... lds (tile_io.hpp) into two LDS stages for the 256-row tiles (160 to 256 columns) and
+//     into a ring of 3 to 12 stages for the smaller tiles, which run problems bound by operand streaming; the tiles of the
+//     decode shapes (32 x 32, 64 x 32) consume their ring four k-tiles per barrier;
 //   * 16x16x128 e4m3 MFMAs: one instruction covers a whole scale block, starts from a zero accumulator and
 //     yields 4 partial sums per lane, which the VALU folds into the running fp32 sums as acc += partial * s,
 //     s = sA * sB. Weights feed the MFMA row operand and activations the column operand, so a lane only ever
