@@ -189,7 +189,7 @@ FP8_TEST_SHAPES = [
 ]
 # Which tile the cost model picks for some of the shapes above on 256 compute units: a CPU test keeps this true, so that a
 # change of the cost table cannot silently take a tile out of the parity tests.
-FP8_TILE_OF_SHAPE = {(1024, 2112, 256): (64, 160), (1000, 2100, 384): (64, 160), (4096, 5120, 256): (256, 160), (4000, 5100, 384): (256, 160), (512, 24576, 256): (256, 192), (500, 24500, 384): (256, 192),
+FP8_TILE_OF_SHAPE = {(1024, 2112, 256): (128, 128), (1000, 2100, 384): (128, 128), (4096, 5120, 256): (256, 160), (4000, 5100, 384): (256, 160), (512, 24576, 256): (256, 192), (500, 24500, 384): (256, 192),
                      (768, 10880, 256): (256, 128), (4096, 7168, 7168): (256, 256), (4096, 2048, 7168): (128, 256), (1024, 4096, 7168): (128, 128),
                      (512, 4096, 2048): (64, 128), (257, 2112, 1024): (64, 64), (64, 7168, 2048): (64, 32), (64, 4096, 7168): (32, 32)}
 # Plain FP8 calls the grouped and quantiser tests make on the side (first group through the plain entry, quantise-then-
@@ -227,9 +227,10 @@ TUNED_SHAPES = [(4096, 5120, 5120), (2048, 7168, 7168)]
 
 
 # FP8 tiles the cost model does not offer but the kernel supports, built through explicit keys: their wave slabs are
-# 112 and 96 columns wide, which straddle the 128-wide weight-scale blocks (two scale products per k-tile and a select per
-# row of atoms) and do not divide the 64 lanes of the staged epilogue's row stores. (BLOCK_M, BLOCK_N, (m, n, k)).
-FP8_EXPLICIT_TILE_CASES = [(256, 224, (600, 1344, 640)), (256, 224, (300, 1000, 384)), (256, 192, (520, 1156, 512))]
+# 112, 96 and 80 columns wide, which straddle the 128-wide weight-scale blocks (two scale products per k-tile and a select
+# per row of atoms) and do not divide the 64 lanes of the staged epilogue's row stores. (BLOCK_M, BLOCK_N, (m, n, k)).
+FP8_EXPLICIT_TILE_CASES = [(256, 224, (600, 1344, 640)), (256, 224, (300, 1000, 384)), (256, 192, (520, 1156, 512)),
+                           (64, 160, (1000, 2100, 384)), (64, 160, (200, 1156, 1024))]
 
 
 def fp8_explicit_tile_plan(block_m: int, block_n: int, n: int, k: int):

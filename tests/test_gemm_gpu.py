@@ -620,9 +620,9 @@ def test_entry_points_pick_the_fastest_of_three_tiles_when_asked(m, n, k, monkey
 
 @pytest.mark.parametrize('block_m,block_n,shape', testing.FP8_EXPLICIT_TILE_CASES)
 def test_fp8_tiles_whose_slabs_straddle_weight_scale_blocks(block_m, block_n, shape):
-    """256 x 224 and 256 x 192 tiles, built through the reference's keys (yan/jit_kernels/gemm.py:9-16): wave slabs of 112
-    and 96 columns cross the boundaries of the 128-wide weight-scale blocks and do not divide the 64 lanes of the row
-    stores. Same bits as the tile the cost model picks (every tile sums the K blocks in the same order), parity against
+    """256 x 224, 256 x 192 and 64 x 160 tiles, built through the reference's keys (yan/jit_kernels/gemm.py:9-16): wave
+    slabs of 112, 96 and 80 columns cross the boundaries of the 128-wide weight-scale blocks and do not divide the 64
+    lanes of the row stores. Same bits as the tile the cost model picks (every tile sums the K blocks in the same order), parity against
     the oracle, ragged edges left alone."""
     from yan_amd import jit
     m, n, k = shape

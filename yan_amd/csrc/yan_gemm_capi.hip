@@ -15,8 +15,8 @@ struct TileCost { int bm, bn; double per_area; };
 // Same tables and cost model as yan_amd/jit_kernels/heuristics.py (a CPU test keeps the two in step).
 constexpr TileCost kDenseTiles[] = {{256, 256, 1.00}, {256, 224, 1.05}, {256, 192, 1.10}, {256, 160, 1.19}, {256, 128, 1.29}, {128, 256, 1.28},
                                     {128, 192, 1.39}, {128, 128, 1.46}, {64, 192, 1.9}, {64, 128, 1.94}, {64, 64, 2.7}};
-constexpr TileCost kFp8Tiles[]   = {{256, 256, 1.00}, {256, 192, 1.12}, {256, 160, 1.28}, {256, 128, 1.34}, {128, 256, 1.34}, {128, 128, 1.79},
-                                    {64, 160, 2.47}, {64, 128, 2.4}, {64, 64, 3.8}, {64, 32, 4.8}, {32, 32, 7.0}};
+constexpr TileCost kFp8Tiles[]   = {{256, 256, 1.00}, {256, 192, 1.12}, {256, 160, 1.28}, {256, 128, 1.34}, {128, 256, 1.34}, {128, 128, 1.5},
+                                    {64, 128, 2.3}, {64, 64, 3.55}, {64, 32, 4.8}, {32, 32, 7.0}};
 
 template <int COUNT>
 void pick(const TileCost (&tiles)[COUNT], int m, int n, int num_cus, int* bm, int* bn) {
@@ -116,7 +116,7 @@ int yan_gemm_fp8_fp8_bf16_nt(const void* lhs, const float* lhs_scales, long long
     if (bm == BM && bn == BN)                                                                                        \
         return int(yan::Gemm<0, 0, BM, BN, 128, 1, yan::Fp8TileConfig<BM, BN>::MAX_RING_STAGES, 1, yan::GemmType::Normal>::run_sized(                          \
             o, lhs, lhs_scales, int(lhs_scales_stride_m), int(lhs_scales_stride_k), rhs, rhs_scales, m, n, k, s, num_sms, 0));
-    YAN_FP8_CASE(256, 256) YAN_FP8_CASE(256, 192) YAN_FP8_CASE(256, 160) YAN_FP8_CASE(256, 128) YAN_FP8_CASE(128, 256) YAN_FP8_CASE(128, 128) YAN_FP8_CASE(64, 160) YAN_FP8_CASE(64, 128) YAN_FP8_CASE(64, 64)
+    YAN_FP8_CASE(256, 256) YAN_FP8_CASE(256, 192) YAN_FP8_CASE(256, 160) YAN_FP8_CASE(256, 128) YAN_FP8_CASE(128, 256) YAN_FP8_CASE(128, 128) YAN_FP8_CASE(64, 128) YAN_FP8_CASE(64, 64)
     YAN_FP8_CASE(64, 32) YAN_FP8_CASE(32, 32)
 #undef YAN_FP8_CASE
     return int(hipErrorInvalidValue);
@@ -194,6 +194,6 @@ int yan_gemm_select_tile(int op, int m, int n, int k, int num_cus, int* block_m,
     return 0;
 }
 
-const char* yan_gemm_version(void) { return "yan-gemm gfx950 11 dense + 7 fp32 + 11 fp8 tile variants + 1 weight-streaming fp8 variant + 12 grouped fp8 variants + 4 quantiser kernels"; }
+const char* yan_gemm_version(void) { return "yan-gemm gfx950 11 dense + 7 fp32 + 10 fp8 tile variants + 1 weight-streaming fp8 variant + 12 grouped fp8 variants + 4 quantiser kernels"; }
 
 } // extern "C"

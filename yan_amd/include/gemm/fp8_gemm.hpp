@@ -5,11 +5,11 @@
 // and K block :55-61), which in the reference is an unfinished Hopper kernel built on TMA descriptors, cluster
 // barriers and warpgroup MMAs. This is a different kernel for gfx950:
 //   * macro tile BLOCK_M x BLOCK_N x 128 (one scale block per k-tile, 128-byte rows); 8 waves, two per SIMD, for
-//     the tiles from 256 x 128 up, so one wave's scale arithmetic and LDS traffic hide under the other's MFMAs;
-//     4 waves below that;
+//     the tiles from 64 x 64 up (get_num_waves in mfma_utils.hpp), so one wave's scale arithmetic and LDS traffic hide
+//     under the other's MFMAs and eight waves issue the copies; 4 waves below that;
 //   * HBM -> LDS with buffer_load ... lds (tile_io.hpp) into two LDS stages for the 256-row tiles (160 to 256 columns) and
 //     into a ring of 3 to 12 stages for the smaller tiles, which run problems bound by operand streaming; the tiles of the
-//     decode shapes (32 x 32, 64 x 32) consume their ring four k-tiles per barrier;
+//     decode shapes (32 x 32, 64 x 32) consume their ring four k-tiles per barrier, with four more waves that only copy;
 //   * 16x16x128 e4m3 MFMAs: one instruction covers a whole scale block, starts from a zero accumulator and
 //     yields 4 partial sums per lane, which the VALU folds into the running fp32 sums as acc += partial * s,
 //     s = sA * sB. Weights feed the MFMA row operand and activations the column operand, so a lane only ever
@@ -34,6 +34,17 @@
 #include "tile_io.hpp"
 
 namespace yan {
+
+// K-tiles a tile's ring is consumed by per barrier (1: one at a time) and the waves its workgroup is launched with.
+// Tiles of one or two atoms per wave (the decode shapes) with a ring of 12 stages take four k-tiles per barrier, and
+// four more waves that only copy: a wave gets one copy instruction through per ~50 ns, and three per k-tile on each
+// of four waves (activations, weights, scales) was what bounded these tiles.
+__host__ __device__ constexpr int fp8_ring_group(int block_m, int block_n, int stages) {
+    return ((block_m == 32 || block_m == 64) && block_n == 32 && stages >= 12 && stages % 4 == 0) ? 4 : 1;
+}
+__host__ __device__ constexpr int fp8_launch_waves(int block_m, int block_n, int stages) {
+    return fp8_ring_group(block_m, block_n, stages) > 1 ? 8 : get_num_waves(block_m, block_n);
+}
 
 template <int BLOCK_M, int BLOCK_N>
 struct Fp8TileConfig {
@@ -83,7 +94,8 @@ fp8_gemm_tile(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_sca
               const int* __restrict__ grouped_layout, int sa_stride_g, int bid, int num_slots) {
     using Cfg  = Fp8TileConfig<BLOCK_M, BLOCK_N>;
     using Atom = MfmaFP8_16x16x128;
-    constexpr int NW = Cfg::NUM_WAVES, TN = Cfg::WTN / 16, TM = Cfg::WTM / 16;
+    // NW waves compute (and copy); LW are launched: the extra ones of the decode tiles only copy.
+    constexpr int NW = Cfg::NUM_WAVES, LW = fp8_launch_waves(BLOCK_M, BLOCK_N, STAGES), TN = Cfg::WTN / 16, TM = Cfg::WTM / 16;
     constexpr int NB = Cfg::SCALE_B_PER_SLAB;
     static_assert(SHAPE_K % 128 == 0 && SHAPE_N % 4 == 0);
     // SHAPE_N / SHAPE_K == 0 selects the run-time sizes (ahead-of-time library); the JIT bakes them in.
@@ -298,7 +310,7 @@ fp8_gemm_tile(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_sca
     // with one full-width instruction; waves that share a part write the same bytes twice.
     constexpr int STAGE_BYTES = Cfg::RING_STAGE_BYTES, A_BYTES = Cfg::LDS_ROWS_A * kRowBytes, TILE_BYTES = A_BYTES + Cfg::LDS_ROWS_B * kRowBytes;
     constexpr int OPS = StA::PASSES + StB::PASSES + 1, SCALE_PARTS = BLOCK_M >= 64 ? BLOCK_M / 64 : 1;
-    static_assert(Cfg::RING_CAPABLE && (STAGES - 2) * OPS <= 63 && STAGES * STAGE_BYTES <= 160 * 1024);
+    static_assert(Cfg::RING_CAPABLE && (fp8_ring_group(BLOCK_M, BLOCK_N, STAGES) > 1 || (STAGES - 2) * OPS <= 63) && STAGES * STAGE_BYTES <= 160 * 1024);
     __shared__ __attribute__((aligned(1024))) uint8_t ring[STAGES * STAGE_BYTES];
     const uint32_t scale_voff = uint32_t(m0 + lane) * sa_stride_m * 4;
     auto issue_op = [&](int d, int kb, uint8_t* stage) {
@@ -315,20 +327,40 @@ fp8_gemm_tile(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_sca
     // fragment reads, one MFMA, its fold, 56 times over. They consume the ring G k-tiles at a time instead: one
     // barrier, the fragments of G k-tiles, G independent MFMAs, G folds; the copies of the G k-tiles that go where the
     // previous group was start right after the barrier, so STAGES - 2G to STAGES - G k-tiles are in flight.
-    constexpr int G = (TN * TM <= 2 && STAGES >= 12 && STAGES % 4 == 0) ? 4 : 1;
+    constexpr int G = fp8_ring_group(BLOCK_M, BLOCK_N, STAGES);
     if constexpr (G > 1) {
-    static_assert(Cfg::UNIFORM_SCALE_B && NB == 1 && (STAGES - 2 * G) * OPS <= 63);
+    // Eight waves share the copies of a k-tile: operation o = slot * 8 + wave is the o-th 8-row group of the stage
+    // (activation rows first, then weight rows: the two tiles lie back to back) or, past the last group, the copy of
+    // the activation scales (which several waves may repeat: same bytes).
+    constexpr int GA = BLOCK_M / 8, GROUPS_AB = (BLOCK_M + BLOCK_N) / 8, SLOTS = ceil_div(GROUPS_AB + 1, LW);
+    static_assert(LW == 8 && NW == 4 && A_BYTES == GA * 8 * kRowBytes && TILE_BYTES == GROUPS_AB * 8 * kRowBytes && SCALE_PARTS == 1);
+    static_assert(Cfg::UNIFORM_SCALE_B && NB == 1 && (STAGES - 2 * G) * SLOTS <= 63);
+    uint32_t slot_voff[SLOTS];
+#pragma unroll
+    for (int sl = 0; sl < SLOTS; ++sl) {
+        const int o = sl * LW + wave, sub = lane >> 3, chunk = (lane & 7) ^ sub ^ (o & 1);      // GA is even: o and its group in B have the same parity
+        const int row = (o < GA ? m0 + o * 8 : n0 + (o - GA) * 8) + sub;
+        slot_voff[sl] = uint32_t(row) * K + chunk * kChunk;
+    }
+    auto issue_slot = [&](int sl, int kb, uint8_t* stage) {
+        const int o = sl * LW + wave;
+        // which kind of operation a slot holds is known at compile time unless the slot straddles two kinds
+        const bool data = sl * LW + LW - 1 < GROUPS_AB || (sl * LW < GROUPS_AB && o < GROUPS_AB);
+        const bool in_a = sl * LW + LW - 1 < GA || (sl * LW < GA && o < GA);
+        if (data) {
+            if (in_a) __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, YAN_LDS_PTR(stage + o * 8 * kRowBytes), kChunk, slot_voff[sl], kb * kRowBytes, 0, 0);
+            else __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, YAN_LDS_PTR(stage + o * 8 * kRowBytes), kChunk, slot_voff[sl], kb * kRowBytes, 0, 0);
+        } else {
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_sa, YAN_LDS_PTR(stage + TILE_BYTES), 4, scale_voff, kb * sa_stride_k * 4, 0, 0);
+        }
+    };
 #pragma unroll
     for (int t = 0; t < STAGES - G; ++t)
 #pragma unroll
-        for (int d = 0; d < OPS; ++d) issue_op(d, t, ring + t * STAGE_BYTES);
+        for (int sl = 0; sl < SLOTS; ++sl) issue_slot(sl, t, ring + t * STAGE_BYTES);
     int base = 0;          // ring position of the group's first k-tile; STAGES is a multiple of G, groups never wrap
     for (int kb0 = 0; kb0 < NUM_K_BLOCKS; kb0 += G) {
-        float sb_grp[G];
-#pragma unroll
-        for (int t = 0; t < G; ++t)
-            sb_grp[t] = rhs_scales[min(base_blk, NUM_N_BLOCKS - 1) * NUM_K_BLOCKS + min(kb0 + t, NUM_K_BLOCKS - 1)];
-        __builtin_amdgcn_s_waitcnt(waitcnt_imm((STAGES - 2 * G) * OPS, kNoWaitLgkm));
+        __builtin_amdgcn_s_waitcnt(waitcnt_imm((STAGES - 2 * G) * SLOTS, kNoWaitLgkm));
         asm volatile("" ::: "memory");
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
@@ -338,7 +370,12 @@ fp8_gemm_tile(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_sca
 #pragma unroll
         for (int t = 0; t < G; ++t)
 #pragma unroll
-            for (int d = 0; d < OPS; ++d) issue_op(d, kb0 + STAGES - G + t, ring + (prev + t) * STAGE_BYTES);
+            for (int sl = 0; sl < SLOTS; ++sl) issue_slot(sl, kb0 + STAGES - G + t, ring + (prev + t) * STAGE_BYTES);
+        if (wave < NW) {
+        float sb_grp[G];
+#pragma unroll
+        for (int t = 0; t < G; ++t)
+            sb_grp[t] = rhs_scales[min(base_blk, NUM_N_BLOCKS - 1) * NUM_K_BLOCKS + min(kb0 + t, NUM_K_BLOCKS - 1)];
         f32x4 part[G][TN][TM];
         float s_grp[G][TM];
 #pragma unroll
@@ -367,6 +404,7 @@ fp8_gemm_tile(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_sca
 #pragma unroll
                         for (int r = 0; r < 4; ++r) acc[i][j][r] = __builtin_fmaf(part[t][i][j][r], s_grp[t][j], acc[i][j][r]);
             }
+        }
         }
         base = base + G == STAGES ? 0 : base + G;
     }
@@ -432,6 +470,7 @@ fp8_gemm_tile(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_sca
             // main loop has no registers to spare for addresses computed ahead of time.
             int lane_late = lane;
             asm volatile("" : "+v"(lane_late));
+            if (LW > NW && wave >= NW) return;          // waves that only copy
             uint8_t* region = (wave < NW / 2 ? epi_a : epi_b) + (wave % (NW / 2)) * REGION;
             const int col_late = lane_late % 16, g_late = lane_late / 16;
             const int r_in = lane_late / LANES_PER_ROW, c = lane_late % LANES_PER_ROW;
@@ -454,6 +493,7 @@ fp8_gemm_tile(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_sca
             }
         }
     } else {
+        if (LW > NW && wave >= NW) return;              // waves that only copy
 #pragma unroll
         for (int j = 0; j < TM; ++j) {
             const int mm = m_slab + j * 16 + col;
@@ -474,7 +514,7 @@ fp8_gemm_tile(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_sca
 // yan/include/gemm/fp8_gemm.cuh:40, scheduler.cuh:39-58). Between two tiles every wave must have left the epilogue of
 // the first (which reads the LDS stage the second one's first copies go into).
 template <int SHAPE_N, int SHAPE_K, int BLOCK_M, int BLOCK_N, GemmType kGemmType = GemmType::Normal, int STAGES = 2>
-__global__ void __launch_bounds__((get_num_waves(BLOCK_M, BLOCK_N) * kWaveSize))
+__global__ void __launch_bounds__((fp8_launch_waves(BLOCK_M, BLOCK_N, STAGES) * kWaveSize))
 fp8_gemm_kernel(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_scales,
                 const uint8_t* __restrict__ rhs, const float* __restrict__ rhs_scales,
                 __bf16* __restrict__ out, int m, int n_rt, int k_rt, int sa_stride_m, int sa_stride_k,
@@ -534,7 +574,7 @@ public:
         if (slots >= kOutOfRange) return hipErrorInvalidValue;
         const int grid = capped_grid(int(slots), num_sms, device_cu_count());
         hipLaunchKernelGGL((fp8_gemm_kernel<SHAPE_N, SHAPE_K, BLOCK_M, BLOCK_N, kGemmType, int(kNumStages)>), dim3(grid),
-                           dim3(Cfg::NUM_WAVES * kWaveSize), 0, stream, static_cast<const uint8_t*>(lhs), lhs_scales,
+                           dim3(fp8_launch_waves(BLOCK_M, BLOCK_N, int(kNumStages)) * kWaveSize), 0, stream, static_cast<const uint8_t*>(lhs), lhs_scales,
                            static_cast<const uint8_t*>(rhs), rhs_scales, reinterpret_cast<__bf16*>(out), m, n, k,
                            lhs_scales_stride_m, lhs_scales_stride_k, grouped_layout, lhs_scales_stride_g, int(slots));
         return hipGetLastError();
@@ -558,7 +598,7 @@ public:
         const XcdTileScheduler<> sched(m, n, BLOCK_M, BLOCK_N);
         const int slots = sched.grid_size(), grid = capped_grid(slots, num_sms, device_cu_count());
         hipLaunchKernelGGL((fp8_gemm_kernel<SHAPE_N, SHAPE_K, BLOCK_M, BLOCK_N, GemmType::Normal, int(kNumStages)>), dim3(grid),
-                           dim3(Cfg::NUM_WAVES * kWaveSize), 0, stream, static_cast<const uint8_t*>(lhs), lhs_scales,
+                           dim3(fp8_launch_waves(BLOCK_M, BLOCK_N, int(kNumStages)) * kWaveSize), 0, stream, static_cast<const uint8_t*>(lhs), lhs_scales,
                            static_cast<const uint8_t*>(rhs), rhs_scales, reinterpret_cast<__bf16*>(out), m, n, k,
                            lhs_scales_stride_m, lhs_scales_stride_k, static_cast<const int*>(nullptr), 0, slots);
         return hipGetLastError();

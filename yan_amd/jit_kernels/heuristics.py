@@ -23,10 +23,10 @@ _DENSE_TILES = {(256, 256): 1.00, (256, 224): 1.05, (256, 192): 1.10, (256, 160)
 # FP8 tiles: measured over 74 shapes (m = 17 ... 8192, n = 2048 ... 32768, k = 512 ... 16384) with every tile forced in turn;
 # with these costs the model's pick is within 1 % of the fastest tile on all of them. 256 x 192 and 256 x 160 are there for
 # problems whose 256 x 256 tiles leave a round of compute units partly empty (4096 x 5120 x 5120: 320 tiles, against 512
-# tiles of 256 x 160 = two full rounds, 13 % faster), 64 x 160 likewise among the small tiles (1024 x 2112 x 7168: 224 tiles in one
-# round, 15 % faster than 136 tiles of 128 x 128); 256 x 224 is supported by the kernel and never the cheapest.
-_FP8_TILES = {(256, 256): 1.00, (256, 192): 1.12, (256, 160): 1.28, (256, 128): 1.34, (128, 256): 1.34, (128, 128): 1.79,
-              (64, 160): 2.47, (64, 128): 2.4, (64, 64): 3.8, (64, 32): 4.8, (32, 32): 7.0}
+# tiles of 256 x 160 = two full rounds, 13 % faster); 256 x 224 and 64 x 160 are supported by the kernel and never the
+# cheapest (a round of 64 x 160 tiles takes longer than a round of 128 x 128 tiles, which run eight waves).
+_FP8_TILES = {(256, 256): 1.00, (256, 192): 1.12, (256, 160): 1.28, (256, 128): 1.34, (128, 256): 1.34, (128, 128): 1.5,
+              (64, 128): 2.3, (64, 64): 3.55, (64, 32): 4.8, (32, 32): 7.0}
 
 
 def rank_tiles(m: int, n: int, num_cus: int, table, groups: int = 1) -> List[Tuple[float, Tuple[int, int]]]:
@@ -77,7 +77,9 @@ def get_fp8_num_stages(block_m: int, block_n: int) -> int:
     tiles of 32 weight rows that run the decode shapes (`Fp8TileConfig::MAX_RING_STAGES` in fp8_gemm.hpp): 2 for
     256 x 256, 3 for 256 x 128 and 128 x 256, 8 for 64 x 64, 12 for 64 x 32 and 32 x 32. Tiles below 256 x 256 are what the cost model picks when a problem is short on work per CU, i.e. bound by
     operand streaming, and there one k-tile of prefetch does not cover the memory latency."""
-    waves = 8 if block_m * block_n >= 256 * 128 else 4
+    waves = 4               # get_num_waves in mfma_utils.hpp
+    if block_m * block_n >= 256 * 128 or (block_m * block_n >= 64 * 64 and block_m % 64 == 0 and block_n % 64 == 0):
+        waves = 8
     capable = block_m % 32 == 0 and (block_m // 8) % waves == 0 and block_n % 16 == 0
     if not capable:
         return 2
