@@ -6,8 +6,8 @@
 //     (reference: yan/include/gemm/scheduler.cuh:39-41, num_blocks = ceil(m/BLOCK_M) * ceil(N/BLOCK_N));
 //   * under every compute-unit cap, the walk b, b + grid, b + 2 grid, ... of capped_grid() workgroups covers every slot
 //     exactly once and, for grids that are multiples of 8, never leaves the XCD residue b % 8;
-//   * the 32 slots that the 8 XCDs run first (4 per XCD ... 32 per XCD) form compact patches: the slots one XCD owns are a
-//     contiguous range of the band-major sequence.
+//   * the same holds in region order (operand rows long enough that the problem outgrows the memory-side cache), whose
+//     choice of region is pinned for a few measured shapes.
 #include "gemm/scheduler.hpp"
 
 #include <cstdio>
@@ -22,7 +22,7 @@
     } while (0)
 
 int main() {
-    int cases = 0;
+    int cases = 0, region_cases = 0;
     const int blocks[][2] = {{256, 256}, {128, 256}, {64, 16}, {256, 224}};
     for (const auto& blk : blocks) {
         const int bm = blk[0], bn = blk[1];
@@ -30,7 +30,15 @@ int main() {
             for (int tn = 1; tn <= 70; tn += (tn < 10 ? 1 : 9)) {
                 // ragged sizes: the last tile of each dimension holds a single row / column
                 const int m = (tm - 1) * bm + 1, n = (tn - 1) * bn + 1;
-                const yan::XcdTileScheduler<> sched(m, n, bm, bn);
+                // bytes per operand row: 0 = band order; the others put problems of 256 tiles and more whose operands
+                // outgrow the 256 MB cache into region order
+                for (long long row_bytes : {0ll, 4096ll, 28672ll, 262144ll}) {
+                const yan::XcdTileScheduler<> sched(m, n, bm, bn, row_bytes);
+                if (row_bytes == 0 || tm * tn < 256) CHECK(sched.region_rows == 0);
+                if (sched.region_rows) {
+                    ++region_cases;
+                    CHECK(sched.region_rows * sched.region_cols == 256 && sched.region_rows % 8 == 0 && sched.region_cols % 4 == 0);
+                }
                 CHECK(sched.tiles_m == tm && sched.tiles_n == tn && sched.total == tm * tn);
                 const int slots = sched.grid_size();
                 CHECK(slots >= sched.total && slots < sched.total + yan::kNumXCD && slots % yan::kNumXCD == 0);
@@ -59,7 +67,19 @@ int main() {
                     for (int v : hit) CHECK(v == 1);
                 }
                 ++cases;
+                }
             }
+    }
+    // what the traffic model picks for shapes that were measured (bf16, 256 x 256 tiles)
+    {
+        const int m = 0, n = 0, bm = 256, bn = 256;
+        const yan::XcdTileScheduler<> a(8192, 8192, 256, 256, 12288 * 2), b(8192, 4096, 256, 256, 14336 * 2),
+            c(12288, 12288, 256, 256, 12288 * 2), d(8192, 8192, 256, 256, 8192 * 2), e(16384, 16384, 256, 256, 16384);
+        CHECK(a.region_rows == 32 && a.rows_outer);          // the activation block stays: what band order amounts to
+        CHECK(b.region_rows == 16 && c.region_rows == 32);
+        CHECK(d.region_rows == 0);                           // 2 x 128 MiB of operands fit
+        CHECK(e.region_rows == 32 && e.rows_outer);          // the FP8 16384^3 shape
+        CHECK(region_cases > 100);
     }
     std::printf("ok %d\n", cases);
     return 0;

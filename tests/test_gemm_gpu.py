@@ -147,6 +147,25 @@ def test_dense_baseline_8192_cubed():
     assert 1 - 2 * num / den < BF16_TOL
 
 
+@pytest.mark.parametrize('m,n,k', [(8192, 4096, 14336), (12100, 12200, 12288)])
+def test_dense_beyond_the_memory_side_cache_walks_regions(m, n, k):
+    """Operands of more than 256 MB put the 256 x 256 kernel's tile walk into region order (16 x 16 tiles per round for the
+    first shape, 32 x 8 with ragged edges for the second): every 512-row block of the output against a chunked fp32
+    matmul on the device, so that a tile written to the wrong place, twice or not at all fails its block."""
+    _announce('dense beyond the cache', m, n, k)
+    from yan_amd.jit_kernels import bf16_gemm
+    assert bf16_gemm.dense_kernel_plan(m, n, k, torch.bfloat16, yan.get_num_sms(), 0)[1]['BLOCK_M'] == 256
+    a, b, c = testing.make_bf16_case(m, n, k, seed=9, scale=k ** -0.5, device='cuda', gen_device='cuda')
+    c.fill_(float('nan'))
+    yan.gemm_bf16_tn(a, b, c)
+    bt = b.float().t()
+    for r0 in range(0, m, 512):
+        ref = (a[r0:r0 + 512].float() @ bt).double()
+        got = c[r0:r0 + 512].double()
+        diff = 1 - 2 * (got * ref).sum().item() / ((got * got).sum().item() + (ref * ref).sum().item())
+        assert diff < BF16_TOL, (r0, diff)
+
+
 # ----------------------------------------------------------------------------- FP8 block-scaled
 def _fp8_ref(a8, sa, b8, sb):
     return oracle.gemm_fp8_block_scaled_ref(_np(a8), sa.cpu().numpy(), _np(b8), sb.cpu().numpy())

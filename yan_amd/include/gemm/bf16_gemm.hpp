@@ -257,7 +257,7 @@ dense_gemm_body_8w(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
     constexpr int LDS_ROWS_B = StB::PADDED_ROWS;
     constexpr int NUM_COPIES = StA::PASSES + StB::PASSES;
 
-    const XcdTileScheduler<> sched(m, n, BLOCK_M, BLOCK_N);
+    const XcdTileScheduler<> sched(m, n, BLOCK_M, BLOCK_N, (long long)k * sizeof(Elem));
     const int num_slots = sched.grid_size();
     const int lane = get_lane_id();
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWaveSize);

@@ -104,7 +104,8 @@ fp8_gemm_tile(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_sca
 
     static_assert(STAGES == 2 || (STAGES >= 3 && STAGES <= Cfg::MAX_RING_STAGES), "no ring of this depth for this tile");
 
-    const XcdTileScheduler<> sched(m, N, BLOCK_M, BLOCK_N);
+    // a plain GEMM whose operands outgrow the memory-side cache walks its tiles in region order (scheduler.hpp)
+    const XcdTileScheduler<> sched(m, N, BLOCK_M, BLOCK_N, kGemmType == GemmType::Normal ? (long long)K : 0);
     if constexpr (kGemmType == GemmType::GroupedMasked) {
         const int group = bid / sched.grid_size();
         bid -= group * sched.grid_size();
