@@ -77,6 +77,123 @@ struct Fp8TileConfig {
     static constexpr int  MAX_RING_STAGES = RING_CAPABLE ? (160 * 1024 / RING_STAGE_BYTES < RING_DEPTH_CAP ? 160 * 1024 / RING_STAGE_BYTES : RING_DEPTH_CAP) : 2;
 };
 
+// The MFMA operand of a 16-row atom whose rows start at `atom_rows` in a staged tile: lane group g holds bytes
+// [32 g, 32 g + 32) of its row, two 16-byte chunks at the offsets frag_offset<16> gives for chunks 2g and 2g + 1.
+__device__ __forceinline__ i32x8 fp8_read_frag(const uint8_t* atom_rows, int off0, int off1) {
+    const i32x4 lo = *reinterpret_cast<const i32x4*>(atom_rows + off0);
+    const i32x4 hi = *reinterpret_cast<const i32x4*>(atom_rows + off1);
+    return i32x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+}
+
+// One k-tile of a wave's slab: TN x TM atoms, software-pipelined by hand. `pa` / `pb` are the slab's first activation
+// and weight rows in the staged tile. Step t issues the MFMA of atom t (fresh zero accumulator) and folds in the partial
+// sums of atom t - DEPTH, whose MFMA has retired by then; the fragment of weight rows i+1 is fetched while rows i are
+// being multiplied; `row_hook(i)` runs once per row of atoms and is where the copies of the next k-tile are started.
+// sched_barrier keeps the compiler from regrouping the steps (it would otherwise hoist every MFMA and need a register
+// per partial sum). `sa`: the activation scales of this lane's row in each of the TM atoms; `sb`: the weight scales of
+// the one or two 128-wide blocks the slab touches, `rows_in_first_block` rows of atoms lying in the first.
+template <typename Cfg, int TN, int TM, int NB, typename RowHook>
+__device__ __forceinline__ void
+fp8_compute_k_tile(f32x4 (&acc)[TN][TM], const uint8_t* pa, const uint8_t* pb, const float (&sa)[TM], const float (&sb)[NB],
+                   int rows_in_first_block, int off0, int off1, RowHook&& row_hook) {
+    using Atom = MfmaFP8_16x16x128;
+    constexpr int T = TN * TM, DEPTH = 2, RING = 4;
+    i32x8 mf[TM], nf[2];
+    nf[0] = fp8_read_frag(pb, off0, off1);
+#pragma unroll
+    for (int j = 0; j < TM; ++j) mf[j] = fp8_read_frag(pa + j * 16 * kRowBytes, off0, off1);
+    float s[TM];
+    [[maybe_unused]] float s_first[TM], s_second[TM];
+    f32x4 p[RING];
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int t = 0; t < T + DEPTH; ++t) {
+        if (t < T) {
+            const int i = t / TM, j = t % TM;
+            if (j == 1 % TM) row_hook(i);
+            if (j == 0 && i + 1 < TN) nf[(i + 1) & 1] = fp8_read_frag(pb + (i + 1) * 16 * kRowBytes, off0, off1);
+            p[t % RING] = Atom::mma(nf[i & 1], mf[j], f32x4{0.f, 0.f, 0.f, 0.f});
+        }
+        if (t >= DEPTH) {
+            const int u = t - DEPTH, i = u / TM, j = u % TM;
+            if constexpr (Cfg::UNIFORM_SCALE_B) {
+                if (u == 0) {
+#pragma unroll
+                    for (int jj = 0; jj < TM; ++jj) s[jj] = sa[jj] * sb[0];
+                }
+            } else if (j == 0) {
+                // A slab that is not a divisor of 128 wide crosses at most one boundary between weight-scale
+                // blocks: rows of atoms below `rows_in_first_block` take block 0's scale, the others block 1's.
+                // Both products are formed once per k-tile and each row picks its own with a bit select under a
+                // wave-uniform mask: no branch, so the steps stay in one basic block.
+                static_assert(NB == 2, "a slab narrower than 128 touches at most two scale blocks");
+                if (i == 0) {
+#pragma unroll
+                    for (int jj = 0; jj < TM; ++jj) { s_first[jj] = sa[jj] * sb[0]; s_second[jj] = sa[jj] * sb[1]; }
+                }
+                const uint32_t pick_second = i >= rows_in_first_block ? 0xffffffffu : 0u;
+#pragma unroll
+                for (int jj = 0; jj < TM; ++jj)
+                    s[jj] = __builtin_bit_cast(float, (__builtin_bit_cast(uint32_t, s_second[jj]) & pick_second) |
+                                                      (__builtin_bit_cast(uint32_t, s_first[jj]) & ~pick_second));
+            }
+#pragma unroll
+            for (int r = 0; r < 4; ++r) acc[i][j][r] = __builtin_fmaf(p[u % RING][r], s[j], acc[i][j][r]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    }
+}
+
+// A wave's slab of sums out to memory as bf16. The 4 registers of atom (i, j) are n = n_slab + 16i + 4g + {0..3} of row
+// m = m_slab + 16j + col; stored straight from there a wave instruction writes 16 rows x 32 bytes. With `region` (LDS
+// of 16 * (2 WTN + 16) bytes that nobody else touches) the slab instead turns round through it, 16 rows at a time, and
+// is stored 16 bytes per lane in runs of 2 * WTN consecutive bytes per row; rows are 2 * WTN + 16 bytes apart in LDS,
+// which spreads the 8-byte writes of 16 rows over the banks. STAGED = false: the direct stores, `region` unused.
+// Rows outside [row_lo, row_hi) and columns from n on are not stored. `rsrc_out` addresses the output tile that starts
+// at (m0, n0); `lane` should be an opaque copy of the lane number made after the main loop, which has no registers to
+// spare for addresses computed ahead of time.
+template <typename Cfg, bool STAGED, int TN, int TM>
+__device__ __forceinline__ void
+fp8_store_slab(const f32x4 (&acc)[TN][TM], uint8_t* region, __amdgpu_buffer_rsrc_t rsrc_out, int m_slab, int n_slab, int m0, int n0,
+               int row_lo, int row_hi, int n, bool stream_out, int lane) {
+    const int col = lane % 16, g = lane / 16;
+    if constexpr (STAGED) {
+        {
+            static_assert(Cfg::WTN >= 32);
+            constexpr int PITCH = Cfg::WTN * 2 + 16;
+            constexpr int LANES_PER_ROW = Cfg::WTN / 8, ROWS_PER_STORE = kWaveSize / LANES_PER_ROW, STORES = ceil_div(16, ROWS_PER_STORE);
+            const int r_in = lane / LANES_PER_ROW, c = lane % LANES_PER_ROW;
+            const int nn = n_slab + 8 * c;
+#pragma unroll
+            for (int j = 0; j < TM; ++j) {
+#pragma unroll
+                for (int i = 0; i < TN; ++i)
+                    *reinterpret_cast<bf16x4*>(region + col * PITCH + (16 * i + 4 * g) * 2) = pack4(acc[i][j], __bf16{});
+#pragma unroll
+                for (int q = 0; q < STORES; ++q) {
+                    const int row = ROWS_PER_STORE * q + r_in, mm = m_slab + 16 * j + row;
+                    const i32x4 v = *reinterpret_cast<const i32x4*>(region + row * PITCH + c * 16);
+                    // a slab width that does not divide 64 lanes leaves the last lanes, and rows past 16, without work
+                    const bool live = mm >= row_lo && mm < row_hi && nn < n && r_in < ROWS_PER_STORE && row < 16;
+                    if (live) buffer_store_16(v, rsrc_out, uint32_t((mm - m0) * n + nn - n0) * 2u, stream_out);
+                }
+                __builtin_amdgcn_sched_barrier(0);      // one 16-row pass at a time: the registers are full of sums
+            }
+        }
+    } else {
+#pragma unroll
+        for (int j = 0; j < TM; ++j) {
+            const int mm = m_slab + j * 16 + col;
+            if (mm < row_lo || mm >= row_hi) continue;
+#pragma unroll
+            for (int i = 0; i < TN; ++i) {
+                const int nn = n_slab + i * 16 + 4 * g;
+                if (nn < n) buffer_store_8(pack4(acc[i][j], __bf16{}), rsrc_out, uint32_t((mm - m0) * n + nn - n0) * 2u, stream_out);
+            }
+        }
+    }
+}
+
 // Normal:            lhs [m, K], rhs [N, K], out [m, N]; grouped_layout unused.
 // GroupedContiguous: lhs [m, K] is the concatenation of the groups' rows, every group padded to a multiple of 128
 //                    rows (BLOCK_M divides 128); grouped_layout[i] is the group of row i, negative for padding rows,
@@ -166,11 +283,7 @@ fp8_gemm_tile(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_sca
     [[maybe_unused]] const int rows_in_first_block = (128 - (n_slab & 127)) / 16;     // only for slabs that straddle blocks
 
     const int off0 = frag_offset<16>(lane, 2 * g), off1 = frag_offset<16>(lane, 2 * g + 1);
-    auto read_frag = [&](const uint8_t* atom_rows) {
-        const i32x4 lo = *reinterpret_cast<const i32x4*>(atom_rows + off0);
-        const i32x4 hi = *reinterpret_cast<const i32x4*>(atom_rows + off1);
-        return i32x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-    };
+    auto read_frag = [&](const uint8_t* atom_rows) { return fp8_read_frag(atom_rows, off0, off1); };
 
     f32x4 acc[TN][TM];
 
@@ -187,60 +300,11 @@ fp8_gemm_tile(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_sca
         load_weight_scales(kb);
     };
 
-    // One k-tile: TN x TM atoms, software-pipelined by hand. Step t issues the MFMA of atom t (fresh zero
-    // accumulator) and folds in the partial sums of atom t - DEPTH, whose MFMA has retired by then; the fragment of
-    // weight rows i+1 is fetched while rows i are being multiplied; `row_hook(i)` runs once per row of atoms and
-    // is where the copies of the next k-tile are started. sched_barrier keeps the compiler from regrouping the
-    // steps (it would otherwise hoist every MFMA and need a register per partial sum).
+    // One k-tile staged at (la, lb): fp8_compute_k_tile on this wave's slab.
     auto compute_tile = [&](const uint8_t* la, const uint8_t* lb, const float (&sa)[TM], const float (&sb)[NB],
                             auto&& row_hook) {
-        constexpr int T = TN * TM, DEPTH = 2, RING = 4;
-        const uint8_t* pa = la + wm * Cfg::WTM * kRowBytes;
-        const uint8_t* pb = lb + wn * Cfg::WTN * kRowBytes;
-        i32x8 mf[TM], nf[2];
-        nf[0] = read_frag(pb);
-#pragma unroll
-        for (int j = 0; j < TM; ++j) mf[j] = read_frag(pa + j * 16 * kRowBytes);
-        float s[TM];
-        [[maybe_unused]] float s_first[TM], s_second[TM];
-        f32x4 p[RING];
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int t = 0; t < T + DEPTH; ++t) {
-            if (t < T) {
-                const int i = t / TM, j = t % TM;
-                if (j == 1 % TM) row_hook(i);
-                if (j == 0 && i + 1 < TN) nf[(i + 1) & 1] = read_frag(pb + (i + 1) * 16 * kRowBytes);
-                p[t % RING] = Atom::mma(nf[i & 1], mf[j], f32x4{0.f, 0.f, 0.f, 0.f});
-            }
-            if (t >= DEPTH) {
-                const int u = t - DEPTH, i = u / TM, j = u % TM;
-                if constexpr (Cfg::UNIFORM_SCALE_B) {
-                    if (u == 0) {
-#pragma unroll
-                        for (int jj = 0; jj < TM; ++jj) s[jj] = sa[jj] * sb[0];
-                    }
-                } else if (j == 0) {
-                    // A slab that is not a divisor of 128 wide crosses at most one boundary between weight-scale
-                    // blocks: rows of atoms below `rows_in_first_block` take block 0's scale, the others block 1's.
-                    // Both products are formed once per k-tile and each row picks its own with a bit select under a
-                    // wave-uniform mask: no branch, so the steps stay in one basic block.
-                    static_assert(NB == 2, "a slab narrower than 128 touches at most two scale blocks");
-                    if (i == 0) {
-#pragma unroll
-                        for (int jj = 0; jj < TM; ++jj) { s_first[jj] = sa[jj] * sb[0]; s_second[jj] = sa[jj] * sb[1]; }
-                    }
-                    const uint32_t pick_second = i >= rows_in_first_block ? 0xffffffffu : 0u;
-#pragma unroll
-                    for (int jj = 0; jj < TM; ++jj)
-                        s[jj] = __builtin_bit_cast(float, (__builtin_bit_cast(uint32_t, s_second[jj]) & pick_second) |
-                                                          (__builtin_bit_cast(uint32_t, s_first[jj]) & ~pick_second));
-                }
-#pragma unroll
-                for (int r = 0; r < 4; ++r) acc[i][j][r] = __builtin_fmaf(p[u % RING][r], s[j], acc[i][j][r]);
-            }
-            __builtin_amdgcn_sched_barrier(0);
-        }
+        fp8_compute_k_tile<Cfg>(acc, la + wm * Cfg::WTM * kRowBytes, lb + wn * Cfg::WTN * kRowBytes, sa, sb, rows_in_first_block,
+                                off0, off1, row_hook);
     };
 
     // Two LDS stages, one k-tile (= one scale block) of prefetch; the scales of the next block travel in
@@ -445,11 +509,8 @@ fp8_gemm_tile(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_sca
     }
     }
 
-    // Epilogue: the 4 registers of atom (i, j) are n = n_slab + 16i + 4g + {0..3} of row m = m_slab + 16j + col.
-    // Stored straight from there a wave instruction writes 16 rows x 32 bytes. Slabs of 32 columns or more instead turn
-    // round through the LDS stage that was consumed last (the only one no copy is on its way into), 16 rows at a time,
-    // and are stored 16 bytes per lane in runs of 2 * WTN consecutive bytes per row. Rows are WTN * 2 + 16 bytes apart
-    // in LDS, which spreads the 8-byte writes of 16 rows over the banks.
+    // Epilogue (fp8_store_slab): slabs of 32 columns or more turn round through the LDS stage that was consumed last (the
+    // only one no copy is on its way into) when the rows of the output are 16-byte aligned.
     // An output larger than the L2s together (8 x 4 MB) is stored with the non-temporal hint: kept in L2 it pushes out
     // the operand panels the other workgroups of the XCD are about to read.
     bool staged = false;
@@ -457,61 +518,188 @@ fp8_gemm_tile(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_sca
     const bool stream_out = size_t(m) * N * 2 * (kGemmType == GemmType::GroupedMasked ? num_slots / sched.grid_size() : 1) > (size_t(32) << 20);
     const __amdgpu_buffer_rsrc_t rsrc_out = make_out_rsrc(out + size_t(m0) * N + n0);
     if (staged) {
-        if constexpr (kStagedEpilogue) {
-            constexpr int PITCH = Cfg::WTN * 2 + 16, REGION = 16 * PITCH;
-            constexpr int LANES_PER_ROW = Cfg::WTN / 8, ROWS_PER_STORE = kWaveSize / LANES_PER_ROW, STORES = ceil_div(16, ROWS_PER_STORE);
-            static_assert(STORES >= 1 && (NW / 2) * REGION <= Cfg::LDS_ROWS_A * kRowBytes && (NW / 2) * REGION <= Cfg::LDS_ROWS_B * kRowBytes);
-            // every wave has read the last k-tile (a bare barrier: __syncthreads() would also wait for the copies still
-            // on their way into the other stages, which nobody will read)
-            __builtin_amdgcn_s_waitcnt(waitcnt_imm(kNoWaitVm, 0));
-            asm volatile("" ::: "memory");
-            __builtin_amdgcn_s_barrier();
-            asm volatile("" ::: "memory");
-            // Everything the epilogue derives from the lane number is derived here, behind an opaque copy of it: the
-            // main loop has no registers to spare for addresses computed ahead of time.
-            int lane_late = lane;
-            asm volatile("" : "+v"(lane_late));
-            if (LW > NW && wave >= NW) return;          // waves that only copy
-            uint8_t* region = (wave < NW / 2 ? epi_a : epi_b) + (wave % (NW / 2)) * REGION;
-            const int col_late = lane_late % 16, g_late = lane_late / 16;
-            const int r_in = lane_late / LANES_PER_ROW, c = lane_late % LANES_PER_ROW;
-            const int nn = n_slab + 8 * c;
-#pragma unroll
-            for (int j = 0; j < TM; ++j) {
-#pragma unroll
-                for (int i = 0; i < TN; ++i)
-                    *reinterpret_cast<bf16x4*>(region + col_late * PITCH + (16 * i + 4 * g_late) * 2) = pack4(acc[i][j], __bf16{});
-#pragma unroll
-                for (int q = 0; q < STORES; ++q) {
-                    const int row = ROWS_PER_STORE * q + r_in, mm = m_slab + 16 * j + row;
-                    const i32x4 v = *reinterpret_cast<const i32x4*>(region + row * PITCH + c * 16);
-                    // a slab width that does not divide 64 lanes leaves the last lanes, and rows past 16, without work
-                    bool live = mm < m && nn < N && r_in < ROWS_PER_STORE && row < 16;
-                    if constexpr (kTwoHalves) live = live && mm >= pass_lo[pass] && mm < pass_hi[pass];
-                    if (live) buffer_store_16(v, rsrc_out, uint32_t((mm - m0) * N + nn - n0) * 2u, stream_out);
-                }
-                __builtin_amdgcn_sched_barrier(0);      // one 16-row pass at a time: the registers are full of sums
-            }
-        }
+        constexpr int REGION = 16 * (Cfg::WTN * 2 + 16);
+        static_assert(!kStagedEpilogue || ((NW / 2) * REGION <= Cfg::LDS_ROWS_A * kRowBytes && (NW / 2) * REGION <= Cfg::LDS_ROWS_B * kRowBytes));
+        // every wave has read the last k-tile (a bare barrier: __syncthreads() would also wait for the copies still
+        // on their way into the other stages, which nobody will read)
+        __builtin_amdgcn_s_waitcnt(waitcnt_imm(kNoWaitVm, 0));
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        if (LW > NW && wave >= NW) return;          // waves that only copy
+        // Everything the epilogue derives from the lane number is derived behind an opaque copy of it: the main loop
+        // has no registers to spare for addresses computed ahead of time.
+        int lane_late = lane;
+        asm volatile("" : "+v"(lane_late));
+        uint8_t* region = (wave < NW / 2 ? epi_a : epi_b) + (wave % (NW / 2)) * REGION;
+        fp8_store_slab<Cfg, kStagedEpilogue>(acc, region, rsrc_out, m_slab, n_slab, m0, n0, pass_lo[pass], pass_hi[pass], N, stream_out, lane_late);
     } else {
         if (LW > NW && wave >= NW) return;              // waves that only copy
-#pragma unroll
-        for (int j = 0; j < TM; ++j) {
-            const int mm = m_slab + j * 16 + col;
-            if (mm >= m) continue;
-            if constexpr (kTwoHalves) { if (mm < pass_lo[pass] || mm >= pass_hi[pass]) continue; }
-#pragma unroll
-            for (int i = 0; i < TN; ++i) {
-                const int nn = n_slab + i * 16 + 4 * g;
-                if (nn < N) buffer_store_8(pack4(acc[i][j], __bf16{}), rsrc_out, uint32_t((mm - m0) * N + nn - n0) * 2u, stream_out);
-            }
-        }
+        fp8_store_slab<Cfg, false>(acc, nullptr, rsrc_out, m_slab, n_slab, m0, n0, pass_lo[pass], pass_hi[pass], N, stream_out, lane);
     }
     }   // pass
 }
 
-// Workgroup b runs slots b, b + gridDim.x, ...: exactly one when the launcher starts a workgroup per slot, a walk over
-// several when the caller caps the number of compute units (the reference's persistent kernel under `num_sms`,
+// Whether a tile configuration runs the persistent walk below: the plain GEMM on two LDS stages with sizes known at
+// compile time and an even number of k-tiles (every tile then starts in stage 0).
+template <int SHAPE_N, int SHAPE_K, int STAGES, GemmType kGemmType>
+constexpr bool kFp8PersistentWalk = STAGES == 2 && kGemmType == GemmType::Normal && SHAPE_N > 0 && SHAPE_K > 0 && (SHAPE_K / 128) % 2 == 0;
+
+// The plain GEMM on two LDS stages as a persistent walk: workgroup b takes slots b, b + gridDim.x, ... (the launcher
+// starts one workgroup per CU, or as many as the caller's cap allows) and overlaps the seams between them. The copies of
+// the next tile's first k-tile and its first scales start during the last k-tile of the current one, every wave waits
+// for them in front of the epilogue, and the output stores drain while the next tile's first k-tile is being
+// multiplied. With a workgroup per tile every tile paid for its first loads, its store drain and a workgroup launch:
+// 4096 x 7168 x 7168 runs 1.5 % faster this way, 4096 x 24576 x 1536 5 %, 4096 x 32768 x 512 15 %. Same bits: the sum
+// over K is formed in the same order.
+// What a wave needs to know of a tile is wave-uniform: the per-lane parts of every address (the lane's row within a copy
+// pass, its row within the slab) do not depend on the tile, and the tile's first row rides in the scalar offset.
+template <int SHAPE_N, int SHAPE_K, int BLOCK_M, int BLOCK_N>
+__device__ __forceinline__ void
+fp8_gemm_walk(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_scales,
+              const uint8_t* __restrict__ rhs, const float* __restrict__ rhs_scales,
+              __bf16* __restrict__ out, int m, int sa_stride_m, int sa_stride_k, int num_slots) {
+    using Cfg = Fp8TileConfig<BLOCK_M, BLOCK_N>;
+    constexpr int NW = Cfg::NUM_WAVES, TN = Cfg::WTN / 16, TM = Cfg::WTM / 16, NB = Cfg::SCALE_B_PER_SLAB;
+    constexpr int N = SHAPE_N, K = SHAPE_K, NUM_K_BLOCKS = K / 128, NUM_N_BLOCKS = ceil_div(N, 128);
+    static_assert(NUM_K_BLOCKS % 2 == 0 && Cfg::WTN >= 32);
+    using StA = TileStager<BLOCK_M, NW>;
+    using StB = TileStager<BLOCK_N, NW>;
+    constexpr int NUM_COPIES = StA::PASSES + StB::PASSES, SPREAD_ROWS = TN >= 2 ? TN / 2 : 1;
+
+    const XcdTileScheduler<> sched(m, N, BLOCK_M, BLOCK_N, (long long)K);
+    const int lane = get_lane_id();
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWaveSize);
+    const int wn = wave % Cfg::WAVES_N, wm = wave / Cfg::WAVES_N;
+    const int g = lane / 16, col = lane % 16;
+
+    const __amdgpu_buffer_rsrc_t rsrc_a = make_rsrc(lhs, uint32_t(m) * K);
+    const __amdgpu_buffer_rsrc_t rsrc_b = make_rsrc(rhs, uint32_t(N) * K);
+    const uint32_t sa_bytes = (uint32_t(m - 1) * sa_stride_m + uint32_t(NUM_K_BLOCKS - 1) * sa_stride_k + 1) * 4;
+    const __amdgpu_buffer_rsrc_t rsrc_sa = make_rsrc(lhs_scales, sa_bytes);
+    const bool stream_out = size_t(m) * N * 2 > (size_t(32) << 20);
+
+    struct TileIo {
+        int m0, n0;
+        int base_blk, rows_in_first_block;      // weight-scale blocks of the slab
+        bool valid;
+    };
+    auto open_tile = [&](int slot) {
+        TileIo t;
+        const TileCoord coord = slot < num_slots ? sched.tile_of(slot) : TileCoord{0, 0, false};
+        t.valid = coord.valid;
+        // no tile: activation rows past the matrix (its copies move zeros, its scale loads return zeros), weight tile 0
+        t.m0 = coord.valid ? coord.m_idx * BLOCK_M : sched.tiles_m * BLOCK_M;
+        t.n0 = coord.n_idx * BLOCK_N;
+        const int n_slab = t.n0 + wn * Cfg::WTN;
+        t.base_blk = n_slab / 128;
+        t.rows_in_first_block = (128 - (n_slab & 127)) / 16;
+        return t;
+    };
+    StA stage_a;
+    StB stage_b;
+    stage_a.init(0, K, wave, lane);
+    stage_b.init(0, K, wave, lane);
+    const uint32_t sa_voff = uint32_t(wm * Cfg::WTM + col) * sa_stride_m * 4;
+    const int off0 = frag_offset<16>(lane, 2 * g), off1 = frag_offset<16>(lane, 2 * g + 1);
+
+    f32x4 acc[TN][TM];
+    float sa_next[TM], sb_next[NB], sa_cur[TM], sb_cur[NB];
+    auto load_scales = [&](const TileIo& t, int kb) {
+#pragma unroll
+        for (int j = 0; j < TM; ++j)
+            sa_next[j] = buffer_load_f32(rsrc_sa, sa_voff, (kb * sa_stride_k + (t.m0 + j * 16) * sa_stride_m) * 4);
+#pragma unroll
+        for (int b = 0; b < NB; ++b) sb_next[b] = rhs_scales[min(t.base_blk + b, NUM_N_BLOCKS - 1) * NUM_K_BLOCKS + kb];
+    };
+
+    __shared__ __attribute__((aligned(1024))) uint8_t lds_a0[Cfg::LDS_ROWS_A * kRowBytes];
+    __shared__ __attribute__((aligned(1024))) uint8_t lds_b0[Cfg::LDS_ROWS_B * kRowBytes];
+    __shared__ __attribute__((aligned(1024))) uint8_t lds_a1[Cfg::LDS_ROWS_A * kRowBytes];
+    __shared__ __attribute__((aligned(1024))) uint8_t lds_b1[Cfg::LDS_ROWS_B * kRowBytes];
+
+    // One k-tile of tile `t`, staged in (a_cur, b_cur) and known to have landed when `landed`; meanwhile the copies of
+    // k-tile `kb_src` of tile `src` go into (a_nxt, b_nxt) and its scales into registers (`src` is `t` itself, or the
+    // next tile during the last k-tile).
+    auto k_step = [&](const TileIo& t, const uint8_t* a_cur, const uint8_t* b_cur, uint8_t* a_nxt, uint8_t* b_nxt,
+                      const TileIo& src, int kb_src, bool landed) {
+        const int a_byte0 = src.m0 * K + kb_src * kRowBytes, b_byte0 = src.n0 * K + kb_src * kRowBytes;
+#pragma unroll
+        for (int j = 0; j < TM; ++j) sa_cur[j] = sa_next[j];
+#pragma unroll
+        for (int b = 0; b < NB; ++b) sb_cur[b] = sb_next[b];
+        if (!landed) {
+            wait_for_copies();
+            __syncthreads();
+        }
+        load_scales(src, kb_src);
+        fp8_compute_k_tile<Cfg>(acc, a_cur + wm * Cfg::WTM * kRowBytes, b_cur + wn * Cfg::WTN * kRowBytes, sa_cur, sb_cur,
+                                t.rows_in_first_block, off0, off1, [&](int row) {
+#pragma unroll
+            for (int d = 0; d < NUM_COPIES; ++d) {
+                if (d * SPREAD_ROWS / NUM_COPIES != row) continue;
+                if (d < StA::PASSES) stage_a.issue_pass(rsrc_a, a_nxt, a_byte0, wave, d);
+                else stage_b.issue_pass(rsrc_b, b_nxt, b_byte0, wave, d - StA::PASSES);
+            }
+        });
+    };
+
+    int slot = blockIdx.x;
+    TileIo cur = open_tile(slot);
+    if (!cur.valid) return;
+    stage_a.issue(rsrc_a, lds_a0, cur.m0 * K, wave);
+    stage_b.issue(rsrc_b, lds_b0, cur.n0 * K, wave);
+    load_scales(cur, 0);
+    wait_for_copies();
+    __syncthreads();
+    while (true) {
+        slot += gridDim.x;
+        const TileIo nxt = open_tile(slot);
+#pragma unroll
+        for (int i = 0; i < TN; ++i)
+#pragma unroll
+            for (int j = 0; j < TM; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+        // k-tile 0 has landed for every wave: the barrier in front of the loop, or the one in front of the last epilogue
+        k_step(cur, lds_a0, lds_b0, lds_a1, lds_b1, cur, 1, true);
+        for (int kb = 1; kb + 2 < NUM_K_BLOCKS; kb += 2) {
+            k_step(cur, lds_a1, lds_b1, lds_a0, lds_b0, cur, kb + 1, false);
+            k_step(cur, lds_a0, lds_b0, lds_a1, lds_b1, cur, kb + 2, false);
+        }
+        // the last k-tile, in stage 1; stage 0 takes the first k-tile of the next tile
+        k_step(cur, lds_a1, lds_b1, lds_a0, lds_b0, nxt, 0, false);
+        // the sums are complete here: without this the compiler moves the last folds down into the epilogue, next to their
+        // first use, and parks the partial sums they wait for in scratch memory
+#pragma unroll
+        for (int i = 0; i < TN; ++i)
+#pragma unroll
+            for (int j = 0; j < TM; ++j) asm volatile("" : "+v"(acc[i][j]));
+
+        // every wave has read the last k-tile and the next tile's first k-tile has landed; then the epilogue through stage 1
+        wait_for_copies();
+        __syncthreads();
+        {
+            constexpr int REGION = 16 * (Cfg::WTN * 2 + 16);
+            static_assert((NW / 2) * REGION <= Cfg::LDS_ROWS_A * kRowBytes && (NW / 2) * REGION <= Cfg::LDS_ROWS_B * kRowBytes);
+            const __amdgpu_buffer_rsrc_t rsrc_out = make_out_rsrc(out + size_t(cur.m0) * N + cur.n0);
+            int lane_late = lane;
+            asm volatile("" : "+v"(lane_late));
+            uint8_t* region = (wave < NW / 2 ? lds_a1 : lds_b1) + (wave % (NW / 2)) * REGION;
+            fp8_store_slab<Cfg, (N % 8) == 0>(acc, region, rsrc_out, cur.m0 + wm * Cfg::WTM, cur.n0 + wn * Cfg::WTN, cur.m0, cur.n0,
+                                              0, m, N, stream_out, lane_late);
+        }
+        if (!nxt.valid) break;
+        cur = nxt;
+        // the next tile's second k-tile is copied into the stage the epilogue went through: every wave has to be out of it
+        __builtin_amdgcn_s_waitcnt(waitcnt_imm(kNoWaitVm, 0));
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+    }
+}
+
+// Workgroup b runs slots b, b + gridDim.x, ...: the persistent walk above where it applies; otherwise exactly one slot
+// when the launcher starts a workgroup per slot, and a plain loop over several when the caller caps the number of compute
+// units (the reference's persistent kernel under `num_sms`,
 // yan/include/gemm/fp8_gemm.cuh:40, scheduler.cuh:39-58). Between two tiles every wave must have left the epilogue of
 // the first (which reads the LDS stage the second one's first copies go into).
 template <int SHAPE_N, int SHAPE_K, int BLOCK_M, int BLOCK_N, GemmType kGemmType = GemmType::Normal, int STAGES = 2>
@@ -520,6 +708,10 @@ fp8_gemm_kernel(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_s
                 const uint8_t* __restrict__ rhs, const float* __restrict__ rhs_scales,
                 __bf16* __restrict__ out, int m, int n_rt, int k_rt, int sa_stride_m, int sa_stride_k,
                 const int* __restrict__ grouped_layout, int sa_stride_g, int num_slots) {
+    if constexpr (kFp8PersistentWalk<SHAPE_N, SHAPE_K, STAGES, kGemmType>) {
+        fp8_gemm_walk<SHAPE_N, SHAPE_K, BLOCK_M, BLOCK_N>(lhs, lhs_scales, rhs, rhs_scales, out, m, sa_stride_m, sa_stride_k, num_slots);
+        return;
+    }
     for (int slot = blockIdx.x; slot < num_slots; slot += gridDim.x) {
         fp8_gemm_tile<SHAPE_N, SHAPE_K, BLOCK_M, BLOCK_N, kGemmType, STAGES>(lhs, lhs_scales, rhs, rhs_scales, out, m, n_rt, k_rt,
                                                                              sa_stride_m, sa_stride_k, grouped_layout, sa_stride_g,
@@ -597,7 +789,14 @@ public:
         if (uint64_t(BLOCK_M) * n * 2 >= kOutOfRange) return hipErrorInvalidValue;
         using Cfg = Fp8TileConfig<BLOCK_M, BLOCK_N>;
         const XcdTileScheduler<> sched(m, n, BLOCK_M, BLOCK_N);
-        const int slots = sched.grid_size(), grid = capped_grid(slots, num_sms, device_cu_count());
+        const int slots = sched.grid_size();
+        int grid = capped_grid(slots, num_sms, device_cu_count());
+        if constexpr (kFp8PersistentWalk<int(SHAPE_N), int(SHAPE_K), int(kNumStages), GemmType::Normal>) {
+            // persistent: one workgroup per CU (a multiple of the 8 XCDs, so a workgroup's tiles stay on one XCD), or as
+            // many as the caller's cap allows
+            const int cus = device_cu_count() / kNumXCD * kNumXCD;
+            grid = capped_grid(slots < cus ? slots : cus, num_sms, device_cu_count());
+        }
         hipLaunchKernelGGL((fp8_gemm_kernel<SHAPE_N, SHAPE_K, BLOCK_M, BLOCK_N, GemmType::Normal, int(kNumStages)>), dim3(grid),
                            dim3(fp8_launch_waves(BLOCK_M, BLOCK_N, int(kNumStages)) * kWaveSize), 0, stream, static_cast<const uint8_t*>(lhs), lhs_scales,
                            static_cast<const uint8_t*>(rhs), rhs_scales, reinterpret_cast<__bf16*>(out), m, n, k,
