@@ -222,6 +222,22 @@ NUM_SMS_CAP = 64
 CAPPED_SHAPES = [(2048, 4096, 1024), (512, 4096, 2048), (300, 2112, 640)]
 
 
+# A problem of 6 x 3 tiles of 256 x 256 (18: not a multiple of the 8 XCDs, so some XCDs' ranges end in an empty slot) run by
+# 3 and 5 workgroups: walks that cross the XCDs' ranges. (m, n, k), caps.
+ODD_CAP_CASE = ((1300, 768, 512), (3, 5))
+
+
+def odd_cap_plans(cap: int):
+    """((name, keys, arg_defs, includes, template) of the FP8 kernel, the same of the dense kernel) for ODD_CAP_CASE on
+    256 x 256 tiles; the dense kernel takes its cap as a key, the FP8 kernel as a launch argument."""
+    from yan_amd.jit_kernels import bf16_gemm, gemm
+    (m, n, k), _ = ODD_CAP_CASE
+    name, keys, arg_defs, code_template = fp8_explicit_tile_plan(256, 256, n, k)
+    dense_keys = {'BLOCK_M': 256, 'BLOCK_N': 256, 'NUM_STAGES': 2, 'NUM_SMS': cap}
+    return ((name, keys, arg_defs, gemm.includes, code_template),
+            ('gemm_bf16_tn', dense_keys, bf16_gemm._arg_defs(torch.bfloat16), bf16_gemm.includes, bf16_gemm.template))
+
+
 # Shapes run with empirical tile selection (YAN_TUNE_TILES=1): three candidate tiles each, for both GEMMs.
 TUNED_SHAPES = [(4096, 5120, 5120), (2048, 7168, 7168)]
 
@@ -277,6 +293,9 @@ def jit_kernels_in_use(num_cus: int = 256):
         add(name, arg_defs, gemm.includes, code_template, keys)
         name, keys, arg_defs, _, code_template = gemm.fp8_kernel_plan(m, n, k, num_cus, True)
         add(name, arg_defs, gemm.includes, code_template, keys)
+    for cap in (0,) + ODD_CAP_CASE[1]:
+        for name, keys, arg_defs, includes, code_template in odd_cap_plans(cap):
+            add(name, arg_defs, includes, code_template, keys)
     for m, n, k in TUNED_SHAPES:
         name, keys, space, arg_defs = bf16_gemm.dense_tuning_plan(m, n, k, torch.bfloat16, num_cus)
         for extra in space:

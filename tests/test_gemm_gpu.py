@@ -566,6 +566,34 @@ def test_num_sms_caps_the_workgroups_without_changing_a_bit(m, n, k):
         yan.set_num_sms(full)
 
 
+@pytest.mark.parametrize('cap', testing.ODD_CAP_CASE[1])
+def test_walks_under_a_cap_that_is_no_multiple_of_the_xcds_reach_every_tile(cap):
+    """18 tiles of 256 x 256 leave an empty slot at the end of six of the eight XCDs' ranges; 3 or 5 persistent workgroups
+    walk across those ranges and must not stop at the first empty slot. Both persistent kernels, against their own
+    uncapped launch (same bits: a tile's sum does not depend on which workgroup runs it) and the oracle."""
+    (m, n, k), _ = testing.ODD_CAP_CASE
+    _announce('odd num_sms cap', cap, m, n, k)
+    stream = torch.cuda.current_stream()
+    (fp8_name, fp8_keys, fp8_defs, fp8_inc, fp8_tmpl), _ = testing.odd_cap_plans(cap)
+    rt = jit.build(fp8_name, fp8_defs, jit.generate(fp8_inc, fp8_defs, jit.cpp_format(fp8_tmpl, fp8_keys)))
+    (a8, sa), (b8, sb), out = testing.make_fp8_case(m, n, k, seed=23, device='cuda', col_major_scales=True)
+    capped = torch.full_like(out, float('nan'))
+    assert rt(a8, sa, b8, sb, out, m, stream, yan.get_num_sms(), 0) == 0
+    assert rt(a8, sa, b8, sb, capped, m, stream, cap, 0) == 0
+    assert torch.equal(capped, out)
+    assert oracle.calc_diff(_np(out), _fp8_ref(a8, sa, b8, sb)) < 1e-5
+    a, b, c = testing.make_bf16_case(m, n, k, seed=24, device='cuda')
+    results = []
+    for this_cap in (0, cap):
+        _, (name, keys, defs, inc, tmpl) = testing.odd_cap_plans(this_cap)
+        drt = jit.build(name, defs, jit.generate(inc, defs, jit.cpp_format(tmpl, keys)))
+        c = torch.full_like(c, float('nan'))
+        assert drt(m, n, k, a, b, c, stream) == 0
+        results.append(c)
+    assert torch.equal(results[0], results[1])
+    assert oracle.calc_diff(_np(results[1]), oracle.gemm_bf16_tn_ref(_np(a), _np(b))) < BF16_TOL
+
+
 def test_num_sms_cap_is_what_runs_at_the_headline_size():
     """cfg3 under a cap of 64 of 256 compute units: identical bits, and two to four times the time, i.e. the cap is the
     number of compute units that work (448 tiles: 7 rounds of 64 instead of 1.75 rounds of 256). Less than four times:

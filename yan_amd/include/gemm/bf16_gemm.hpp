@@ -397,7 +397,13 @@ dense_gemm_body_8w(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
         }
     };
 
-    int slot = blockIdx.x;
+    // The next slot of this workgroup's walk that holds a tile. Under a cap that is not a multiple of the 8 XCDs a walk
+    // crosses the XCDs' ranges, and an empty slot at the end of one range can be followed by a tile of another.
+    auto seek = [&](int slot) {
+        while (slot < num_slots && !sched.tile_of(slot).valid) slot += gridDim.x;
+        return slot;
+    };
+    int slot = seek(blockIdx.x);
     TileIo cur = open_tile(slot);
     if (!cur.valid) return;
 #pragma unroll
@@ -405,7 +411,7 @@ dense_gemm_body_8w(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
     open_next();
     fetch_first(lds_a0, lds_b0);
     while (true) {
-        slot += gridDim.x;
+        slot = seek(slot + gridDim.x);
         const TileIo nxt = open_tile(slot);
 #pragma unroll
         for (int i = 0; i < TN; ++i)

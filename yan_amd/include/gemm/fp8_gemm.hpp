@@ -644,7 +644,13 @@ fp8_gemm_walk(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_sca
         });
     };
 
-    int slot = blockIdx.x;
+    // The next slot of this workgroup's walk that holds a tile. Under a cap that is not a multiple of the 8 XCDs a walk
+    // crosses the XCDs' ranges, and an empty slot at the end of one range can be followed by a tile of another.
+    auto seek = [&](int slot) {
+        while (slot < num_slots && !sched.tile_of(slot).valid) slot += gridDim.x;
+        return slot;
+    };
+    int slot = seek(blockIdx.x);
     TileIo cur = open_tile(slot);
     if (!cur.valid) return;
     stage_a.issue(rsrc_a, lds_a0, cur.m0 * K, wave);
@@ -653,7 +659,7 @@ fp8_gemm_walk(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_sca
     wait_for_copies();
     __syncthreads();
     while (true) {
-        slot += gridDim.x;
+        slot = seek(slot + gridDim.x);
         const TileIo nxt = open_tile(slot);
 #pragma unroll
         for (int i = 0; i < TN; ++i)
