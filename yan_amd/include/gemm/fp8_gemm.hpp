@@ -77,6 +77,12 @@ struct Fp8TileConfig {
     static constexpr int  MAX_RING_STAGES = RING_CAPABLE ? (160 * 1024 / RING_STAGE_BYTES < RING_DEPTH_CAP ? 160 * 1024 / RING_STAGE_BYTES : RING_DEPTH_CAP) : 2;
 };
 
+// The two LDS stages of the 256-row tiles (operand tiles of Fp8TileConfig::LDS_ROWS_A / LDS_ROWS_B rows each), declared
+// once in the kernel and handed to whichever of its bodies runs; unused by the ring tiles, which declare their own ring.
+struct Fp8TwoStages {
+    uint8_t *a0, *b0, *a1, *b1;
+};
+
 // The MFMA operand of a 16-row atom whose rows start at `atom_rows` in a staged tile: lane group g holds bytes
 // [32 g, 32 g + 32) of its row, two 16-byte chunks at the offsets frag_offset<16> gives for chunks 2g and 2g + 1.
 __device__ __forceinline__ i32x8 fp8_read_frag(const uint8_t* atom_rows, int off0, int off1) {
@@ -208,7 +214,7 @@ __device__ __forceinline__ void
 fp8_gemm_tile(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_scales,
               const uint8_t* __restrict__ rhs, const float* __restrict__ rhs_scales,
               __bf16* __restrict__ out, int m, int n_rt, int k_rt, int sa_stride_m, int sa_stride_k,
-              const int* __restrict__ grouped_layout, int sa_stride_g, int bid, int num_slots) {
+              const int* __restrict__ grouped_layout, int sa_stride_g, int bid, int num_slots, Fp8TwoStages two_stages) {
     using Cfg  = Fp8TileConfig<BLOCK_M, BLOCK_N>;
     using Atom = MfmaFP8_16x16x128;
     // NW waves compute (and copy); LW are launched: the extra ones of the decode tiles only copy.
@@ -352,10 +358,10 @@ fp8_gemm_tile(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_sca
 #pragma unroll
         for (int j = 0; j < TM; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
     if constexpr (STAGES == 2) {
-    __shared__ __attribute__((aligned(1024))) uint8_t lds_a0[Cfg::LDS_ROWS_A * kRowBytes];
-    __shared__ __attribute__((aligned(1024))) uint8_t lds_b0[Cfg::LDS_ROWS_B * kRowBytes];
-    __shared__ __attribute__((aligned(1024))) uint8_t lds_a1[Cfg::LDS_ROWS_A * kRowBytes];
-    __shared__ __attribute__((aligned(1024))) uint8_t lds_b1[Cfg::LDS_ROWS_B * kRowBytes];
+    uint8_t* const lds_a0 = two_stages.a0;
+    uint8_t* const lds_b0 = two_stages.b0;
+    uint8_t* const lds_a1 = two_stages.a1;
+    uint8_t* const lds_b1 = two_stages.b1;
     stage_a.issue(rsrc_a, lds_a0, 0, wave);
     stage_b.issue(rsrc_b, lds_b0, 0, wave);
     load_scales(0);
@@ -540,16 +546,18 @@ fp8_gemm_tile(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_sca
     }   // pass
 }
 
-// Whether a tile configuration runs the persistent walk below: the plain GEMM on two LDS stages with sizes known at
-// compile time and an even number of k-tiles (every tile then starts in stage 0).
-template <int SHAPE_N, int SHAPE_K, int STAGES, GemmType kGemmType>
-constexpr bool kFp8PersistentWalk = STAGES == 2 && kGemmType == GemmType::Normal && SHAPE_N > 0 && SHAPE_K > 0 && (SHAPE_K / 128) % 2 == 0;
+// Whether a problem runs the persistent walk below: the plain GEMM on two LDS stages with an even number of k-tiles
+// (every tile then starts in stage 0).
+template <int STAGES, GemmType kGemmType>
+__host__ __device__ constexpr bool fp8_walks(int k) {
+    return STAGES == 2 && kGemmType == GemmType::Normal && (k / 128) % 2 == 0;
+}
 
 // The plain GEMM on two LDS stages as a persistent walk: workgroup b takes slots b, b + gridDim.x, ... (the launcher
 // starts one workgroup per CU, or as many as the caller's cap allows) and overlaps the seams between them. The copies of
 // the next tile's first k-tile and its first scales start during the last k-tile of the current one, every wave waits
 // for them in front of the epilogue, and the output stores drain while the next tile's first k-tile is being
-// multiplied. With a workgroup per tile every tile paid for its first loads, its store drain and a workgroup launch:
+// multiplied. With a workgroup per tile every tile pays for its first loads, its store drain and a workgroup launch:
 // 4096 x 7168 x 7168 runs 1.5 % faster this way, 4096 x 24576 x 1536 5 %, 4096 x 32768 x 512 15 %. Same bits: the sum
 // over K is formed in the same order.
 // What a wave needs to know of a tile is wave-uniform: the per-lane parts of every address (the lane's row within a copy
@@ -558,11 +566,13 @@ template <int SHAPE_N, int SHAPE_K, int BLOCK_M, int BLOCK_N>
 __device__ __forceinline__ void
 fp8_gemm_walk(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_scales,
               const uint8_t* __restrict__ rhs, const float* __restrict__ rhs_scales,
-              __bf16* __restrict__ out, int m, int sa_stride_m, int sa_stride_k, int num_slots) {
+              __bf16* __restrict__ out, int m, int n_rt, int k_rt, int sa_stride_m, int sa_stride_k, int num_slots, Fp8TwoStages two_stages) {
     using Cfg = Fp8TileConfig<BLOCK_M, BLOCK_N>;
     constexpr int NW = Cfg::NUM_WAVES, TN = Cfg::WTN / 16, TM = Cfg::WTM / 16, NB = Cfg::SCALE_B_PER_SLAB;
-    constexpr int N = SHAPE_N, K = SHAPE_K, NUM_K_BLOCKS = K / 128, NUM_N_BLOCKS = ceil_div(N, 128);
-    static_assert(NUM_K_BLOCKS % 2 == 0 && Cfg::WTN >= 32);
+    // SHAPE_N / SHAPE_K == 0 selects the run-time sizes (ahead-of-time library); the JIT bakes them in.
+    const int N = SHAPE_N ? SHAPE_N : n_rt, K = SHAPE_K ? SHAPE_K : k_rt;
+    const int NUM_K_BLOCKS = K / 128, NUM_N_BLOCKS = ceil_div(N, 128);          // NUM_K_BLOCKS is even: the caller checked
+    static_assert(Cfg::WTN >= 32);
     using StA = TileStager<BLOCK_M, NW>;
     using StB = TileStager<BLOCK_N, NW>;
     constexpr int NUM_COPIES = StA::PASSES + StB::PASSES, SPREAD_ROWS = TN >= 2 ? TN / 2 : 1;
@@ -613,10 +623,10 @@ fp8_gemm_walk(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_sca
         for (int b = 0; b < NB; ++b) sb_next[b] = rhs_scales[min(t.base_blk + b, NUM_N_BLOCKS - 1) * NUM_K_BLOCKS + kb];
     };
 
-    __shared__ __attribute__((aligned(1024))) uint8_t lds_a0[Cfg::LDS_ROWS_A * kRowBytes];
-    __shared__ __attribute__((aligned(1024))) uint8_t lds_b0[Cfg::LDS_ROWS_B * kRowBytes];
-    __shared__ __attribute__((aligned(1024))) uint8_t lds_a1[Cfg::LDS_ROWS_A * kRowBytes];
-    __shared__ __attribute__((aligned(1024))) uint8_t lds_b1[Cfg::LDS_ROWS_B * kRowBytes];
+    uint8_t* const lds_a0 = two_stages.a0;
+    uint8_t* const lds_b0 = two_stages.b0;
+    uint8_t* const lds_a1 = two_stages.a1;
+    uint8_t* const lds_b1 = two_stages.b1;
 
     // One k-tile of tile `t`, staged in (a_cur, b_cur) and known to have landed when `landed`; meanwhile the copies of
     // k-tile `kb_src` of tile `src` go into (a_nxt, b_nxt) and its scales into registers (`src` is `t` itself, or the
@@ -690,8 +700,12 @@ fp8_gemm_walk(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_sca
             int lane_late = lane;
             asm volatile("" : "+v"(lane_late));
             uint8_t* region = (wave < NW / 2 ? lds_a1 : lds_b1) + (wave % (NW / 2)) * REGION;
-            fp8_store_slab<Cfg, (N % 8) == 0>(acc, region, rsrc_out, cur.m0 + wm * Cfg::WTM, cur.n0 + wn * Cfg::WTN, cur.m0, cur.n0,
-                                              0, m, N, stream_out, lane_late);
+            if ((N % 8) == 0)
+                fp8_store_slab<Cfg, true>(acc, region, rsrc_out, cur.m0 + wm * Cfg::WTM, cur.n0 + wn * Cfg::WTN, cur.m0, cur.n0,
+                                          0, m, N, stream_out, lane_late);
+            else
+                fp8_store_slab<Cfg, false>(acc, region, rsrc_out, cur.m0 + wm * Cfg::WTM, cur.n0 + wn * Cfg::WTN, cur.m0, cur.n0,
+                                           0, m, N, stream_out, lane_late);
         }
         if (!nxt.valid) break;
         cur = nxt;
@@ -714,14 +728,26 @@ fp8_gemm_kernel(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_s
                 const uint8_t* __restrict__ rhs, const float* __restrict__ rhs_scales,
                 __bf16* __restrict__ out, int m, int n_rt, int k_rt, int sa_stride_m, int sa_stride_k,
                 const int* __restrict__ grouped_layout, int sa_stride_g, int num_slots) {
-    if constexpr (kFp8PersistentWalk<SHAPE_N, SHAPE_K, STAGES, kGemmType>) {
-        fp8_gemm_walk<SHAPE_N, SHAPE_K, BLOCK_M, BLOCK_N>(lhs, lhs_scales, rhs, rhs_scales, out, m, sa_stride_m, sa_stride_k, num_slots);
-        return;
+    Fp8TwoStages two_stages = {nullptr, nullptr, nullptr, nullptr};
+    if constexpr (STAGES == 2) {
+        using Cfg = Fp8TileConfig<BLOCK_M, BLOCK_N>;
+        __shared__ __attribute__((aligned(1024))) uint8_t lds_a0[Cfg::LDS_ROWS_A * kRowBytes];
+        __shared__ __attribute__((aligned(1024))) uint8_t lds_b0[Cfg::LDS_ROWS_B * kRowBytes];
+        __shared__ __attribute__((aligned(1024))) uint8_t lds_a1[Cfg::LDS_ROWS_A * kRowBytes];
+        __shared__ __attribute__((aligned(1024))) uint8_t lds_b1[Cfg::LDS_ROWS_B * kRowBytes];
+        two_stages = {lds_a0, lds_b0, lds_a1, lds_b1};
+    }
+    if constexpr (fp8_walks<STAGES, kGemmType>(SHAPE_K)) {
+        if (SHAPE_K != 0 || fp8_walks<STAGES, kGemmType>(k_rt)) {
+            fp8_gemm_walk<SHAPE_N, SHAPE_K, BLOCK_M, BLOCK_N>(lhs, lhs_scales, rhs, rhs_scales, out, m, n_rt, k_rt, sa_stride_m, sa_stride_k,
+                                                              num_slots, two_stages);
+            return;
+        }
     }
     for (int slot = blockIdx.x; slot < num_slots; slot += gridDim.x) {
         fp8_gemm_tile<SHAPE_N, SHAPE_K, BLOCK_M, BLOCK_N, kGemmType, STAGES>(lhs, lhs_scales, rhs, rhs_scales, out, m, n_rt, k_rt,
                                                                              sa_stride_m, sa_stride_k, grouped_layout, sa_stride_g,
-                                                                             slot, num_slots);
+                                                                             slot, num_slots, two_stages);
         if (slot + int(gridDim.x) < num_slots) __syncthreads();
     }
 }
@@ -797,7 +823,7 @@ public:
         const XcdTileScheduler<> sched(m, n, BLOCK_M, BLOCK_N);
         const int slots = sched.grid_size();
         int grid = capped_grid(slots, num_sms, device_cu_count());
-        if constexpr (kFp8PersistentWalk<int(SHAPE_N), int(SHAPE_K), int(kNumStages), GemmType::Normal>) {
+        if (fp8_walks<int(kNumStages), GemmType::Normal>(k)) {
             // persistent: one workgroup per CU (a multiple of the 8 XCDs, so a workgroup's tiles stay on one XCD), or as
             // many as the caller's cap allows
             const int cus = device_cu_count() / kNumXCD * kNumXCD;
