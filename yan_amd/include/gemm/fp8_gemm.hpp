@@ -229,17 +229,32 @@ fp8_gemm_tile(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_sca
 
     // a plain GEMM whose operands outgrow the memory-side cache walks its tiles in region order (scheduler.hpp)
     const XcdTileScheduler<> sched(m, N, BLOCK_M, BLOCK_N, kGemmType == GemmType::Normal ? (long long)K : 0);
+    TileCoord tile;
     if constexpr (kGemmType == GemmType::GroupedMasked) {
-        const int group = bid / sched.grid_size();
-        bid -= group * sched.grid_size();
+        int group;
+        if (m % BLOCK_M == 0) {
+            // Whole tiles per group: the groups' tile grids stacked along m are one grid, and an XCD's range of it lies in
+            // one or two groups, so that the 32 tiles it runs at once share weight panels through its L2. Numbering the
+            // slots group by group instead deals every group's tiles out to all 8 XCDs, each of which then holds a few
+            // tiles of every group and as many different weight panels.
+            const XcdTileScheduler<> stacked((num_slots / sched.grid_size()) * m, N, BLOCK_M, BLOCK_N);
+            if (bid >= stacked.grid_size()) return;
+            tile = stacked.tile_of(bid);
+            group = tile.m_idx / sched.tiles_m;
+            tile.m_idx -= group * sched.tiles_m;
+        } else {
+            group = bid / sched.grid_size();
+            tile = sched.tile_of(bid - group * sched.grid_size());
+        }
         lhs        += size_t(group) * m * K;
         lhs_scales += size_t(group) * sa_stride_g;
         out        += size_t(group) * m * N;
         rhs        += size_t(group) * N * K;
         rhs_scales += size_t(group) * NUM_N_BLOCKS * NUM_K_BLOCKS;
         m = min(m, grouped_layout[group]);        // rows of this group that exist; tiles past them leave at once
+    } else {
+        tile = sched.tile_of(bid);
     }
-    const TileCoord tile = sched.tile_of(bid);
     if (!tile.valid) return;
     const int m0 = tile.m_idx * BLOCK_M, n0 = tile.n_idx * BLOCK_N;
     if (m0 >= m) return;
