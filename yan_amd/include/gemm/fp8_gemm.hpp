@@ -5,8 +5,9 @@
 // and K block :55-61), which in the reference is an unfinished Hopper kernel built on TMA descriptors, cluster
 // barriers and warpgroup MMAs. This is a different kernel for gfx950:
 //   * macro tile BLOCK_M x BLOCK_N x 128 (one scale block per k-tile, 128-byte rows); 8 waves, two per SIMD, for
-//     the tiles from 64 x 64 up (get_num_waves in mfma_utils.hpp), so one wave's scale arithmetic and LDS traffic hide
-//     under the other's MFMAs and eight waves issue the copies; 4 waves below that;
+//     the tiles from 256 x 128 up and for the tiles from 64 x 64 up whose sides are multiples of 64 (get_num_waves in
+//     mfma_utils.hpp), so one wave's scale arithmetic and LDS traffic hide under the other's MFMAs and eight waves issue
+//     the copies; 4 waves otherwise;
 //   * HBM -> LDS with buffer_load ... lds (tile_io.hpp) into two LDS stages for the 256-row tiles (160 to 256 columns) and
 //     into a ring of 3 to 12 stages for the smaller tiles, which run problems bound by operand streaming; the tiles of the
 //     decode shapes (32 x 32, 64 x 32) consume their ring four k-tiles per barrier, with four more waves that only copy;
@@ -17,7 +18,10 @@
 //   * the running sums stay in architectural VGPRs (the VALU cannot address AGPRs): 128 per wave;
 //   * the output leaves through LDS: each wave turns its slab round through the stage that was consumed last and stores
 //     16 bytes per lane in row runs of 2 * WTN bytes (non-temporal when the output is larger than the L2s together);
-//   * m is a run-time argument with tails predicated; N and K are compile-time;
+//   * the plain GEMM on the 256-row tiles is a persistent walk: one workgroup per compute unit takes tile after tile and
+//     overlaps the seams (fp8_gemm_walk); every other case runs a workgroup per tile, or a plain loop under a cap;
+//   * m is a run-time argument with tails predicated; N and K are compile-time in the JIT kernels and run-time (template
+//     arguments 0) in the ahead-of-time library;
 //   * grouped (mixture-of-experts) layouts, the reference's GemmType::GroupedContiguous / GroupedMasked hooks
 //     (yan/include/gemm/scheduler.cuh:7-11,31-48, `int* grouped_layout` of fp8_gemm.cuh:41): every output tile
 //     belongs to one group, which picks the [N, K] weight matrix and its scale table; the rest of the kernel
