@@ -1003,6 +1003,24 @@ def test_capi_seeded_random_shapes_against_device_references():
         assert torch.equal(keep, c_buf[:, n:])
 
 
+@pytest.mark.parametrize('cap', [0, 5])
+def test_capi_fp8_beyond_the_memory_side_cache_ragged_and_capped(cap):
+    """343 MB of FP8 operands with ragged edges through the C library: the persistent walk in region order (run-time N and
+    K), uncapped and with 5 workgroups crossing the XCDs' ranges; every 512-row block against the dequantised product on
+    the device."""
+    m, n, k = 6690, 19292, 13824
+    _announce('capi fp8 beyond the cache', m, n, k, cap)
+    (a8, sa), (b8, sb), out = testing.make_fp8_case(m, n, k, seed=31, device='cuda', gen_device='cuda', col_major_scales=True)
+    out.fill_(float('nan'))
+    assert capi.gemm_fp8_fp8_bf16_nt((a8, sa), (b8, sb), out, cap) == 0
+    bt = testing.dequant_rhs(b8, sb).t().contiguous()
+    for r0 in range(0, m, 512):
+        ref = (testing.dequant_lhs(a8[r0:r0 + 512], sa[r0:r0 + 512]) @ bt).double()
+        got = out[r0:r0 + 512].double()
+        diff = 1 - 2 * (got * ref).sum().item() / ((got * got).sum().item() + (ref * ref).sum().item())
+        assert diff < 1e-5, (r0, diff)
+
+
 def test_capi_rejects_bad_sizes_on_device():
     from yan_amd import capi
     a = torch.zeros(64, 64, dtype=torch.bfloat16, device='cuda')
