@@ -89,7 +89,8 @@ YAN_API int yan_m_grouped_gemm_fp8_fp8_bf16_nt_contiguous(const void* lhs, const
 
 /* masked: lhs [num_groups][m_max][k], out [num_groups][m_max][n], both contiguous; scale (g,i,kb) of lhs at
  *   lhs_scales[g*stride_g + i*stride_m + kb*stride_k]; masked_m (device, int32 [num_groups]) says how many leading rows
- *   of each group are valid; the other rows of `out` are not written. expected_m > 0 is a hint for the tile choice. */
+ *   of each group are valid; the other rows of `out` are not written. expected_m > 0 is a hint for the tile choice
+ *   and the launch order (the tile rows below it come first); results do not depend on it. */
 YAN_API int yan_m_grouped_gemm_fp8_fp8_bf16_nt_masked(const void* lhs, const float* lhs_scales, long long lhs_scales_stride_g,
                                               long long lhs_scales_stride_m, long long lhs_scales_stride_k, const void* rhs,
                                               const float* rhs_scales, void* out, const int* masked_m, int num_groups,

@@ -160,7 +160,8 @@ int yan_m_grouped_gemm_fp8_fp8_bf16_nt_masked(const void* lhs, const float* lhs_
     if (bm == BM && bn == BN)                                                                                        \
         return int(yan::Gemm<0, 0, BM, BN, 128, 1, yan::Fp8TileConfig<BM, BN>::MAX_RING_STAGES, 1, yan::GemmType::GroupedMasked>::run_grouped(                 \
             static_cast<__hip_bfloat16*>(out), lhs, lhs_scales, int(lhs_scales_stride_m), int(lhs_scales_stride_k),  \
-            int(lhs_scales_stride_g), rhs, rhs_scales, masked_m, num_groups, m_max, n, k, static_cast<hipStream_t>(stream), num_sms));
+            int(lhs_scales_stride_g), rhs, rhs_scales, masked_m, num_groups, m_max, n, k, static_cast<hipStream_t>(stream), num_sms, \
+            expected_m));
     YAN_GROUPED_CASE(256, 256) YAN_GROUPED_CASE(256, 128) YAN_GROUPED_CASE(128, 256) YAN_GROUPED_CASE(128, 128)
     YAN_GROUPED_CASE(64, 128) YAN_GROUPED_CASE(64, 64)
 #undef YAN_GROUPED_CASE

@@ -81,6 +81,41 @@ struct Fp8TileConfig {
     static constexpr int  MAX_RING_STAGES = RING_CAPABLE ? (160 * 1024 / RING_STAGE_BYTES < RING_DEPTH_CAP ? 160 * 1024 / RING_STAGE_BYTES : RING_DEPTH_CAP) : 2;
 };
 
+// Slot numbering of the masked layout. Only the first masked_m[g] rows of a group exist, and the caller's `expected_m`
+// says how many that usually is: the tile rows below it come first, all groups' stacked along m into one grid (an XCD's
+// range of it lies in one or two groups, so the 32 tiles it runs at once share weight panels through its L2), the tile
+// rows above it afterwards in a second grid of the same kind. A workgroup whose tile does not exist leaves at once, but
+// it still takes a compute unit to start: numbered group by group, existing and empty tiles alternate and the existing
+// ones start in ever smaller waves as the empty ones get out of their way (8 groups x 128 rows of which 64 exist: 58 us
+// against 42 us when the rows are 64). Same on the host (slot count) and on the device (slot -> group, tile).
+struct MaskedSlots {
+    XcdTileScheduler<> likely, rest;
+    int tiles_m, likely_rows, likely_slots;
+
+    __host__ __device__ MaskedSlots(int num_groups, int m, int n, int block_m, int block_n, int expected_m)
+        : likely(0, 0, block_m, block_n), rest(0, 0, block_m, block_n) {
+        tiles_m = ceil_div(m, block_m);
+        likely_rows = expected_m > 0 ? ceil_div(expected_m, block_m) : tiles_m;
+        likely_rows = likely_rows < tiles_m ? likely_rows : tiles_m;
+        likely = XcdTileScheduler<>(num_groups * likely_rows * block_m, n, block_m, block_n);
+        rest   = XcdTileScheduler<>(num_groups * (tiles_m - likely_rows) * block_m, n, block_m, block_n);
+        likely_slots = likely.grid_size();
+    }
+
+    __host__ __device__ long long num_slots() const { return (long long)likely_slots + rest.grid_size(); }
+
+    // group and tile (within the group's [m, n] problem) of a slot
+    __host__ __device__ TileCoord tile_of(int slot, int* group) const {
+        const bool first = slot < likely_slots;
+        const int rows = first ? likely_rows : tiles_m - likely_rows;
+        TileCoord t = first ? likely.tile_of(slot) : rest.tile_of(slot - likely_slots);
+        if (!t.valid) { *group = 0; return t; }
+        *group = t.m_idx / rows;
+        t.m_idx = t.m_idx % rows + (first ? 0 : likely_rows);
+        return t;
+    }
+};
+
 // The two LDS stages of the 256-row tiles (operand tiles of Fp8TileConfig::LDS_ROWS_A / LDS_ROWS_B rows each), declared
 // once in the kernel and handed to whichever of its bodies runs; unused by the ring tiles, which declare their own ring.
 struct Fp8TwoStages {
@@ -209,8 +244,8 @@ fp8_store_slab(const f32x4 (&acc)[TN][TM], uint8_t* region, __amdgpu_buffer_rsrc
 //                    rows (BLOCK_M divides 128); grouped_layout[i] is the group of row i, negative for padding rows,
 //                    whose tiles are skipped; rhs [G, N, K], rhs_scales [G, ceil(N/128), K/128].
 // GroupedMasked:     lhs [G, m, K], out [G, m, N], rhs as above; only the first grouped_layout[g] rows of group g
-//                    are computed; lhs_scales of group g start at g * sa_stride_g floats. The grid is G times the
-//                    grid of one [m, N] problem.
+//                    are computed; lhs_scales of group g start at g * sa_stride_g floats. Slots are numbered by
+//                    MaskedSlots: the tile rows below `expected_m` of all groups first.
 // STAGES: 2 = two LDS stages with the next k-tile's scales in registers; 3.. = a ring of that many stages.
 // One output tile (one slot of the launch: `bid` is what blockIdx.x would be with a workgroup per slot).
 template <int SHAPE_N, int SHAPE_K, int BLOCK_M, int BLOCK_N, GemmType kGemmType, int STAGES>
@@ -218,7 +253,7 @@ __device__ __forceinline__ void
 fp8_gemm_tile(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_scales,
               const uint8_t* __restrict__ rhs, const float* __restrict__ rhs_scales,
               __bf16* __restrict__ out, int m, int n_rt, int k_rt, int sa_stride_m, int sa_stride_k,
-              const int* __restrict__ grouped_layout, int sa_stride_g, int bid, int num_slots, Fp8TwoStages two_stages) {
+              const int* __restrict__ grouped_layout, int sa_stride_g, int bid, int num_groups, int expected_m, Fp8TwoStages two_stages) {
     using Cfg  = Fp8TileConfig<BLOCK_M, BLOCK_N>;
     using Atom = MfmaFP8_16x16x128;
     // NW waves compute (and copy); LW are launched: the extra ones of the decode tiles only copy.
@@ -236,20 +271,7 @@ fp8_gemm_tile(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_sca
     TileCoord tile;
     if constexpr (kGemmType == GemmType::GroupedMasked) {
         int group;
-        if (m % BLOCK_M == 0) {
-            // Whole tiles per group: the groups' tile grids stacked along m are one grid, and an XCD's range of it lies in
-            // one or two groups, so that the 32 tiles it runs at once share weight panels through its L2. Numbering the
-            // slots group by group instead deals every group's tiles out to all 8 XCDs, each of which then holds a few
-            // tiles of every group and as many different weight panels.
-            const XcdTileScheduler<> stacked((num_slots / sched.grid_size()) * m, N, BLOCK_M, BLOCK_N);
-            if (bid >= stacked.grid_size()) return;
-            tile = stacked.tile_of(bid);
-            group = tile.m_idx / sched.tiles_m;
-            tile.m_idx -= group * sched.tiles_m;
-        } else {
-            group = bid / sched.grid_size();
-            tile = sched.tile_of(bid - group * sched.grid_size());
-        }
+        tile = MaskedSlots(num_groups, m, N, BLOCK_M, BLOCK_N, expected_m).tile_of(bid, &group);
         lhs        += size_t(group) * m * K;
         lhs_scales += size_t(group) * sa_stride_g;
         out        += size_t(group) * m * N;
@@ -540,7 +562,7 @@ fp8_gemm_tile(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_sca
     // the operand panels the other workgroups of the XCD are about to read.
     bool staged = false;
     if constexpr (kStagedEpilogue) staged = (N % 8) == 0;
-    const bool stream_out = size_t(m) * N * 2 * (kGemmType == GemmType::GroupedMasked ? num_slots / sched.grid_size() : 1) > (size_t(32) << 20);
+    const bool stream_out = size_t(m) * N * 2 * (kGemmType == GemmType::GroupedMasked ? num_groups : 1) > (size_t(32) << 20);
     const __amdgpu_buffer_rsrc_t rsrc_out = make_out_rsrc(out + size_t(m0) * N + n0);
     if (staged) {
         constexpr int REGION = 16 * (Cfg::WTN * 2 + 16);
@@ -746,7 +768,7 @@ __global__ void __launch_bounds__((fp8_launch_waves(BLOCK_M, BLOCK_N, STAGES) * 
 fp8_gemm_kernel(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_scales,
                 const uint8_t* __restrict__ rhs, const float* __restrict__ rhs_scales,
                 __bf16* __restrict__ out, int m, int n_rt, int k_rt, int sa_stride_m, int sa_stride_k,
-                const int* __restrict__ grouped_layout, int sa_stride_g, int num_slots) {
+                const int* __restrict__ grouped_layout, int sa_stride_g, int num_slots, int num_groups, int expected_m) {
     Fp8TwoStages two_stages = {nullptr, nullptr, nullptr, nullptr};
     if constexpr (STAGES == 2) {
         using Cfg = Fp8TileConfig<BLOCK_M, BLOCK_N>;
@@ -766,7 +788,7 @@ fp8_gemm_kernel(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_s
     for (int slot = blockIdx.x; slot < num_slots; slot += gridDim.x) {
         fp8_gemm_tile<SHAPE_N, SHAPE_K, BLOCK_M, BLOCK_N, kGemmType, STAGES>(lhs, lhs_scales, rhs, rhs_scales, out, m, n_rt, k_rt,
                                                                              sa_stride_m, sa_stride_k, grouped_layout, sa_stride_g,
-                                                                             slot, num_slots, two_stages);
+                                                                             slot, num_groups, expected_m, two_stages);
         if (slot + int(gridDim.x) < num_slots) __syncthreads();
     }
 }
@@ -797,11 +819,12 @@ public:
 
     // Grouped layouts (see the kernel's comment). `m` is the total number of rows (contiguous) or the rows
     // allotted to each group (masked); `grouped_layout` is a device array of m (contiguous) or num_groups (masked)
-    // ints; `lhs_scales_stride_g` is used by the masked layout only. n and k as in run_sized.
+    // ints; `lhs_scales_stride_g` is used by the masked layout only, as is `expected_m` (the rows of a group that usually
+    // exist; 0: all of them): it orders the slots, the result does not depend on it. n and k as in run_sized.
     static hipError_t run_grouped(__hip_bfloat16* out, const void* lhs, const float* lhs_scales, int lhs_scales_stride_m,
                                   int lhs_scales_stride_k, int lhs_scales_stride_g, const void* rhs, const float* rhs_scales,
                                   const int* grouped_layout, int num_groups, int m, int n, int k, hipStream_t stream,
-                                  int num_sms = 0) {
+                                  int num_sms = 0, int expected_m = 0) {
         static_assert(kGemmType != GemmType::Normal);
         if (m == 0 || n == 0 || num_groups == 0) return hipSuccess;
         if (m < 0 || n < 0 || k <= 0 || num_groups < 0 || (n % 4) != 0 || (k % 128) != 0) return hipErrorInvalidValue;
@@ -813,14 +836,18 @@ public:
         // output stores address a tile with 32-bit byte offsets from its first element: BLOCK_M rows of n elements
         if (uint64_t(BLOCK_M) * n * 2 >= kOutOfRange) return hipErrorInvalidValue;
         using Cfg = Fp8TileConfig<BLOCK_M, BLOCK_N>;
+        if (m_pad * num_groups >= kOutOfRange) return hipErrorInvalidValue;
         const XcdTileScheduler<> sched(m, n, BLOCK_M, BLOCK_N);
-        const uint64_t slots = uint64_t(sched.grid_size()) * (kGemmType == GemmType::GroupedMasked ? num_groups : 1);
+        const uint64_t slots = kGemmType == GemmType::GroupedMasked
+                                   ? uint64_t(MaskedSlots(num_groups, m, n, BLOCK_M, BLOCK_N, expected_m).num_slots())
+                                   : uint64_t(sched.grid_size());
         if (slots >= kOutOfRange) return hipErrorInvalidValue;
         const int grid = capped_grid(int(slots), num_sms, device_cu_count());
         hipLaunchKernelGGL((fp8_gemm_kernel<SHAPE_N, SHAPE_K, BLOCK_M, BLOCK_N, kGemmType, int(kNumStages)>), dim3(grid),
                            dim3(fp8_launch_waves(BLOCK_M, BLOCK_N, int(kNumStages)) * kWaveSize), 0, stream, static_cast<const uint8_t*>(lhs), lhs_scales,
                            static_cast<const uint8_t*>(rhs), rhs_scales, reinterpret_cast<__bf16*>(out), m, n, k,
-                           lhs_scales_stride_m, lhs_scales_stride_k, grouped_layout, lhs_scales_stride_g, int(slots));
+                           lhs_scales_stride_m, lhs_scales_stride_k, grouped_layout, lhs_scales_stride_g, int(slots), num_groups,
+                           expected_m);
         return hipGetLastError();
     }
 
@@ -851,7 +878,7 @@ public:
         hipLaunchKernelGGL((fp8_gemm_kernel<SHAPE_N, SHAPE_K, BLOCK_M, BLOCK_N, GemmType::Normal, int(kNumStages)>), dim3(grid),
                            dim3(fp8_launch_waves(BLOCK_M, BLOCK_N, int(kNumStages)) * kWaveSize), 0, stream, static_cast<const uint8_t*>(lhs), lhs_scales,
                            static_cast<const uint8_t*>(rhs), rhs_scales, reinterpret_cast<__bf16*>(out), m, n, k,
-                           lhs_scales_stride_m, lhs_scales_stride_k, static_cast<const int*>(nullptr), 0, slots);
+                           lhs_scales_stride_m, lhs_scales_stride_k, static_cast<const int*>(nullptr), 0, slots, 1, 0);
         return hipGetLastError();
     }
 };

@@ -34,14 +34,14 @@ using GemmType = Gemm<N, K, BLOCK_M, BLOCK_N, 128, kNumGroups, kNumStages, kNumT
 // Launch kernel
 __return_code = static_cast<int>(GemmType::run_grouped(out, lhs, lhs_scales, lhs_scales_stride_m, lhs_scales_stride_k,
                                                        lhs_scales_stride_g, rhs, rhs_scales, grouped_layout,
-                                                       kNumGroups, m, N, K, stream, num_sms));
+                                                       kNumGroups, m, N, K, stream, num_sms, expected_m));
 """
 
 arg_defs = (('lhs', torch.float8_e4m3fn), ('lhs_scales', torch.float),
             ('rhs', torch.float8_e4m3fn), ('rhs_scales', torch.float),
             ('out', torch.bfloat16), ('grouped_layout', torch.int), ('m', int),
             ('stream', torch.cuda.Stream), ('num_sms', int), ('smem_size', int),
-            ('lhs_scales_stride_m', int), ('lhs_scales_stride_k', int), ('lhs_scales_stride_g', int))
+            ('lhs_scales_stride_m', int), ('lhs_scales_stride_k', int), ('lhs_scales_stride_g', int), ('expected_m', int))
 
 
 @functools.lru_cache(maxsize=None)
@@ -62,6 +62,7 @@ def grouped_kernel_plan(gemm_type: str, num_groups: int, m: int, n: int, k: int,
 
 
 def _launch(gemm_type, num_groups, plan_m, m, n, k, lhs, lhs_scales, rhs, rhs_scales, out, layout, strides):
+    # `strides`: the three strides of the activation scales, then expected_m (masked layout; 0 otherwise)
     num_sms = get_num_sms()
     name, keys, defs, smem_size = grouped_kernel_plan(gemm_type, num_groups, plan_m, n, k, num_sms)
     args = (lhs, lhs_scales, rhs, rhs_scales, out, layout, m, torch.cuda.current_stream(), num_sms, smem_size, *strides)
@@ -105,7 +106,7 @@ def m_grouped_gemm_fp8_fp8_bf16_nt_contiguous(lhs: Tuple[torch.Tensor, torch.Ten
     if m == 0:
         return
     _launch('GroupedContiguous', num_groups, m, m, n, k, lhs, lhs_scales, rhs, rhs_scales, out, m_indices,
-            (lhs_scales.stride(0), lhs_scales.stride(1), 0))
+            (lhs_scales.stride(0), lhs_scales.stride(1), 0, 0))
 
 
 def m_grouped_gemm_fp8_fp8_bf16_nt_masked(lhs: Tuple[torch.Tensor, torch.Tensor],
@@ -118,7 +119,8 @@ def m_grouped_gemm_fp8_fp8_bf16_nt_masked(lhs: Tuple[torch.Tensor, torch.Tensor]
     lhs: (e4m3fn `[num_groups, m_max, k]` contiguous, fp32 scales `[num_groups, m_max, ceil(k/128)]` in any strided layout)
     rhs: (e4m3fn `[num_groups, n, k]`, fp32 scales `[num_groups, ceil(n/128), ceil(k/128)]`), both contiguous
     out: bf16 `[num_groups, m_max, n]` contiguous
-    masked_m: int32 `[num_groups]`; expected_m: a hint for the typical masked_m (tile choice only)
+    masked_m: int32 `[num_groups]`; expected_m: a hint for the typical masked_m: it picks the tile and puts the tile rows
+              below it first in the launch order; results do not depend on it
     """
     lhs, lhs_scales = lhs
     rhs, rhs_scales = rhs
@@ -141,4 +143,4 @@ def m_grouped_gemm_fp8_fp8_bf16_nt_masked(lhs: Tuple[torch.Tensor, torch.Tensor]
     if m == 0 or num_groups == 0:
         return
     _launch('GroupedMasked', num_groups, min(expected_m, m), m, n, k, lhs, lhs_scales, rhs, rhs_scales, out, masked_m,
-            (lhs_scales.stride(1), lhs_scales.stride(2), lhs_scales.stride(0)))
+            (lhs_scales.stride(1), lhs_scales.stride(2), lhs_scales.stride(0), min(expected_m, m)))
