@@ -6,6 +6,7 @@
 //     (reference: yan/include/gemm/scheduler.cuh:39-41, num_blocks = ceil(m/BLOCK_M) * ceil(N/BLOCK_N));
 //   * under every compute-unit cap, the walk b, b + grid, b + 2 grid, ... of capped_grid() workgroups covers every slot
 //     exactly once and, for grids that are multiples of 8, never leaves the XCD residue b % 8;
+//   * the masked layout's slot numbering (MaskedSlots) visits every (group, tile) once, likely tile rows first;
 //   * the same holds in region order (operand rows long enough that the problem outgrows the memory-side cache), whose
 //     choice of region is pinned for a few measured shapes.
 #include "gemm/scheduler.hpp"
@@ -70,6 +71,29 @@ int main() {
                 }
             }
     }
+    // the masked layout's slot numbering: every (group, tile) exactly once, the tile rows below expected_m before the others
+    for (int groups : {1, 3, 8, 17})
+        for (int tm = 1; tm <= 9; tm += (tm < 3 ? 1 : 3))
+            for (int tn : {1, 5, 16, 33})
+                for (int expected : {0, 1, 100, 257, 100000}) {
+                    const int bm = 128, bn = 256, m = (tm - 1) * bm + 1, n = (tn - 1) * bn + 1;
+                    const yan::MaskedSlots slots(groups, m, n, bm, bn, expected);
+                    CHECK(slots.num_slots() % yan::kNumXCD == 0 && slots.num_slots() < (long long)groups * tm * tn + 2 * yan::kNumXCD);
+                    std::vector<int> seen(size_t(groups) * tm * tn, 0);
+                    const int likely_rows = expected <= 0 ? tm : ((expected + bm - 1) / bm < tm ? (expected + bm - 1) / bm : tm);
+                    bool rest_seen = false;
+                    for (int s = 0; s < slots.num_slots(); ++s) {
+                        int g = -1;
+                        const yan::TileCoord t = slots.tile_of(s, &g);
+                        if (!t.valid) continue;
+                        CHECK(g >= 0 && g < groups && t.m_idx >= 0 && t.m_idx < tm && t.n_idx >= 0 && t.n_idx < tn);
+                        ++seen[(size_t(g) * tm + t.m_idx) * tn + t.n_idx];
+                        if (t.m_idx >= likely_rows) rest_seen = true;
+                        else CHECK(!rest_seen);
+                    }
+                    for (int v : seen) CHECK(v == 1);
+                    ++cases;
+                }
     // what the traffic model picks for shapes that were measured (bf16, 256 x 256 tiles)
     {
         const int m = 0, n = 0, bm = 256, bn = 256;

@@ -81,41 +81,6 @@ struct Fp8TileConfig {
     static constexpr int  MAX_RING_STAGES = RING_CAPABLE ? (160 * 1024 / RING_STAGE_BYTES < RING_DEPTH_CAP ? 160 * 1024 / RING_STAGE_BYTES : RING_DEPTH_CAP) : 2;
 };
 
-// Slot numbering of the masked layout. Only the first masked_m[g] rows of a group exist, and the caller's `expected_m`
-// says how many that usually is: the tile rows below it come first, all groups' stacked along m into one grid (an XCD's
-// range of it lies in one or two groups, so the 32 tiles it runs at once share weight panels through its L2), the tile
-// rows above it afterwards in a second grid of the same kind. A workgroup whose tile does not exist leaves at once, but
-// it still takes a compute unit to start: numbered group by group, existing and empty tiles alternate and the existing
-// ones start in ever smaller waves as the empty ones get out of their way (8 groups x 128 rows of which 64 exist: 58 us
-// against 42 us when the rows are 64). Same on the host (slot count) and on the device (slot -> group, tile).
-struct MaskedSlots {
-    XcdTileScheduler<> likely, rest;
-    int tiles_m, likely_rows, likely_slots;
-
-    __host__ __device__ MaskedSlots(int num_groups, int m, int n, int block_m, int block_n, int expected_m)
-        : likely(0, 0, block_m, block_n), rest(0, 0, block_m, block_n) {
-        tiles_m = ceil_div(m, block_m);
-        likely_rows = expected_m > 0 ? ceil_div(expected_m, block_m) : tiles_m;
-        likely_rows = likely_rows < tiles_m ? likely_rows : tiles_m;
-        likely = XcdTileScheduler<>(num_groups * likely_rows * block_m, n, block_m, block_n);
-        rest   = XcdTileScheduler<>(num_groups * (tiles_m - likely_rows) * block_m, n, block_m, block_n);
-        likely_slots = likely.grid_size();
-    }
-
-    __host__ __device__ long long num_slots() const { return (long long)likely_slots + rest.grid_size(); }
-
-    // group and tile (within the group's [m, n] problem) of a slot
-    __host__ __device__ TileCoord tile_of(int slot, int* group) const {
-        const bool first = slot < likely_slots;
-        const int rows = first ? likely_rows : tiles_m - likely_rows;
-        TileCoord t = first ? likely.tile_of(slot) : rest.tile_of(slot - likely_slots);
-        if (!t.valid) { *group = 0; return t; }
-        *group = t.m_idx / rows;
-        t.m_idx = t.m_idx % rows + (first ? 0 : likely_rows);
-        return t;
-    }
-};
-
 // The two LDS stages of the 256-row tiles (operand tiles of Fp8TileConfig::LDS_ROWS_A / LDS_ROWS_B rows each), declared
 // once in the kernel and handed to whichever of its bodies runs; unused by the ring tiles, which declare their own ring.
 struct Fp8TwoStages {

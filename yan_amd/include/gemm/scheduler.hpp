@@ -77,6 +77,11 @@ struct XcdTileScheduler {
         if (region_rows) return region_tile_of(bid);
         const int t = (bid % kNumXCD) * per_xcd + bid / kNumXCD;
         if (t >= total) return {0, 0, false};
+        return band_tile(t);
+    }
+
+    // Tile number t of the band-order sequence.
+    __host__ __device__ TileCoord band_tile(int t) const {
         const int band      = GROUP_M * tiles_n;
         const int first_m   = (t / band) * GROUP_M;
         const int band_rows = (tiles_m - first_m) < GROUP_M ? (tiles_m - first_m) : GROUP_M;
@@ -84,21 +89,33 @@ struct XcdTileScheduler {
         return {first_m + in_band % band_rows, in_band / band_rows, true};
     }
 
-    // Region order. Full rounds of 256 tiles hand XCD x the x-th run of 32 consecutive tiles of the sequence (one patch
-    // when the region is whole); the tiles left after the full rounds are dealt out in 8 equal runs. The sequence: region
+    // Slot -> position in a tile sequence, dealt out in rounds: full rounds of 256 tiles hand XCD x the x-th run of 32
+    // consecutive tiles; the tiles left after the full rounds are dealt out in 8 equal runs. -1: an empty slot.
+    __host__ __device__ int dealt_position(int bid) const {
+        const int x = bid % kNumXCD, q = bid / kNumXCD;
+        const int full = total / ROUND, rest = total - full * ROUND;
+        if (q < full * PATCH) return ((q / PATCH) * kNumXCD + x) * PATCH + q % PATCH;
+        const int run = ceil_div(rest, kNumXCD), q_rest = q - full * PATCH;
+        const int t = full * ROUND + x * run + q_rest;
+        return (q_rest >= run || t >= total) ? -1 : t;
+    }
+
+    // Band order dealt out in rounds: an XCD's 32 concurrent tiles are still a patch of one band, but consecutive patches
+    // go to different XCDs. For grids whose tiles differ in cost by position (the masked layout: a group may have few rows
+    // or none), where a contiguous range per XCD would leave some XCDs with all the work.
+    __host__ __device__ TileCoord dealt_band_tile_of(int bid) const {
+        const int t = dealt_position(bid);
+        if (t < 0) return {0, 0, false};
+        return band_tile(t);
+    }
+
+    // Region order, dealt out in rounds (a run of 32 consecutive tiles is one patch when the region is whole). The sequence: region
     // by region; inside a region patch rows of GROUP_M, inside a patch row patches of 4 columns, inside a patch column by
     // column. Regions, patch rows and patches at the lower and right edges are smaller, which shifts the runs against
     // the patches but loses no tile.
     __host__ __device__ TileCoord region_tile_of(int bid) const {
-        const int x = bid % kNumXCD, q = bid / kNumXCD;
-        const int full = total / ROUND, rest = total - full * ROUND;
-        int t;
-        if (q < full * PATCH) t = ((q / PATCH) * kNumXCD + x) * PATCH + q % PATCH;
-        else {
-            const int run = ceil_div(rest, kNumXCD), q_rest = q - full * PATCH;
-            t = full * ROUND + x * run + q_rest;
-            if (q_rest >= run || t >= total) return {0, 0, false};
-        }
+        const int t = dealt_position(bid);
+        if (t < 0) return {0, 0, false};
         int rb, cb, hh, ww, p;        // region (rb, cb) of hh x ww tiles, position p inside it
         if (rows_outer) {
             rb = t / (region_rows * tiles_n);
@@ -121,6 +138,42 @@ struct XcdTileScheduler {
         const int pc = in_row / (ph * PATCH_COLS);                               // patch
         const int in_patch = in_row - pc * ph * PATCH_COLS;
         return {rb * region_rows + pr * GROUP_M + in_patch % ph, cb * region_cols + pc * PATCH_COLS + in_patch / ph, true};
+    }
+};
+
+// Slot numbering of the masked layout. Only the first masked_m[g] rows of a group exist, and the caller's `expected_m`
+// says how many that usually is: the tile rows below it come first, all groups' stacked along m into one grid whose
+// patches of 8 x 4 tiles are dealt out to the XCDs in turn (the 32 tiles an XCD runs at once lie in one or two groups and
+// share weight panels through its L2; consecutive patches go to different XCDs, so a group with few rows or none does not
+// leave one XCD idle), the tile rows above it afterwards in a second grid of the same kind. A workgroup whose tile does not exist leaves at once, but
+// it still takes a compute unit to start: numbered group by group, existing and empty tiles alternate and the existing
+// ones start in ever smaller waves as the empty ones get out of their way (8 groups x 128 rows of which 64 exist: 58 us
+// against 42 us when the rows are 64). Same on the host (slot count) and on the device (slot -> group, tile).
+struct MaskedSlots {
+    XcdTileScheduler<> likely, rest;
+    int tiles_m, likely_rows, likely_slots;
+
+    __host__ __device__ MaskedSlots(int num_groups, int m, int n, int block_m, int block_n, int expected_m)
+        : likely(0, 0, block_m, block_n), rest(0, 0, block_m, block_n) {
+        tiles_m = ceil_div(m, block_m);
+        likely_rows = expected_m > 0 ? ceil_div(expected_m, block_m) : tiles_m;
+        likely_rows = likely_rows < tiles_m ? likely_rows : tiles_m;
+        likely = XcdTileScheduler<>(num_groups * likely_rows * block_m, n, block_m, block_n);
+        rest   = XcdTileScheduler<>(num_groups * (tiles_m - likely_rows) * block_m, n, block_m, block_n);
+        likely_slots = likely.grid_size();
+    }
+
+    __host__ __device__ long long num_slots() const { return (long long)likely_slots + rest.grid_size(); }
+
+    // group and tile (within the group's [m, n] problem) of a slot
+    __host__ __device__ TileCoord tile_of(int slot, int* group) const {
+        const bool first = slot < likely_slots;
+        const int rows = first ? likely_rows : tiles_m - likely_rows;
+        TileCoord t = first ? likely.dealt_band_tile_of(slot) : rest.dealt_band_tile_of(slot - likely_slots);
+        if (!t.valid) { *group = 0; return t; }
+        *group = t.m_idx / rows;
+        t.m_idx = t.m_idx % rows + (first ? 0 : likely_rows);
+        return t;
     }
 };
 
