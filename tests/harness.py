@@ -214,6 +214,9 @@ GROUPED_MASKED_TEST_CASES = [
     (4, 1024, 4096, 7168, (1024, 900, 512, 1), 1024),
     (2, 40, 192, 256, (40, 7), 40),                  # the committed fixture
     (2, 128, 512, 512, (128, 40), 128),              # the group of the graph-replay test
+    # many groups, few rows of many: tile rows above expected_m exist in some groups, groups without rows, an odd group count
+    (17, 384, 320, 384, (384, 0, 5, 64, 65, 0, 0, 200, 1, 384, 128, 129, 0, 7, 300, 64, 2), 64),
+    (8, 1000, 512, 256, (0, 1000, 0, 0, 999, 130, 0, 1), 5000),      # a hint beyond m_max
 ]
 
 
