@@ -111,7 +111,7 @@ YAN_API int yan_per_block_cast_to_fp8(const void* w, int w_is_fp32, void* q, flo
 
 /* Macro tile the library uses for a problem: op 0 = dense 16-bit, 1 = FP8 block-scaled, 2 = FP8 grouped contiguous
  * (m = total rows, and `k` carries the number of groups instead of the depth), 3 = fp32. Writes BLOCK_M / BLOCK_N.
- * For op 1 with few activation rows the answer is (16 * atoms, 16): the weight-streaming kernel.
+ * For ops 0 and 1 with few activation rows the answer is (16 * atoms, 16): the weight-streaming kernels.
  * Host-only (no device call). Stands where the reference leaves tile choice to the caller's keys
  * (yan/jit_kernels/cute_gemm.py:41, yan/jit_kernels/gemm.py:13-16). Returns 0, or 1 for an unknown op. */
 YAN_API int yan_gemm_select_tile(int op, int m, int n, int k, int num_cus, int* block_m, int* block_n);

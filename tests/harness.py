@@ -160,12 +160,16 @@ DENSE_TEST_SHAPES = [
     (4096, 5120, 512), (4000, 5000, 520), (2048, 7168, 256), (2047, 7100, 264), (4096, 6144, 256), (4090, 6100, 72),
     # the 192-wide tiles of the ring kernel (wave slabs of 96 columns), whole and ragged
     (2048, 2112, 264), (2000, 2100, 136), (1024, 2112, 264), (1000, 2100, 72),
+    # a handful of rows over up to 4096 weight rows: the weight-streaming kernel with one and two activation atoms, the
+    # last workgroup partly past n, fewer K blocks than waves ((1, 64, 64) above), more than one pass over the waves
+    (1, 4096, 7168), (16, 2112, 1024), (7, 1156, 512), (17, 4096, 2048), (32, 272, 4096), (20, 100, 2112),
 ]
 # (shape, tile the cost model must pick): the shapes above exist for these tiles
 DENSE_TILE_OF_SHAPE = {(4096, 5120, 512): (256, 160), (4000, 5000, 520): (256, 160), (2048, 7168, 256): (256, 224),
                        (2047, 7100, 264): (256, 224), (4096, 6144, 256): (256, 192), (4090, 6100, 72): (256, 192),
                        (3000, 5000, 1000): (256, 256), (8192, 8192, 8192): (256, 256),
-                       (2048, 2112, 264): (128, 192), (2000, 2100, 136): (128, 192), (1024, 2112, 264): (64, 192), (1000, 2100, 72): (64, 192)}
+                       (2048, 2112, 264): (128, 192), (2000, 2100, 136): (128, 192), (1024, 2112, 264): (64, 192), (1000, 2100, 72): (64, 192),
+                       (1, 4096, 7168): (16, 16), (7, 1156, 512): (16, 16), (17, 4096, 2048): (32, 16), (20, 100, 2112): (32, 16)}
 # (m, n, k) of the reference's own dense test (tests/test_cute.py:21-22: m in (256, 4096) x six (k, n) pairs)
 REFERENCE_DENSE_TEST_SHAPES = [(m, n, k) for m in (256, 4096)
                                for k, n in ((5120, 5120), (1536, 24576), (512, 32768), (16384, 7168), (7168, 2048), (2048, 7168))]

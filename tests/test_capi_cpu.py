@@ -44,7 +44,7 @@ def test_version_and_tile_selection_match_python(lib):
               (1, 128, 128), (300, 96, 640), (1, 4096, 7168), (17, 4096, 1024), (33, 2112, 640), (64, 7168, 2048), (65, 7168, 2048), (257, 2112, 1024), (256, 24576, 1536), (4096, 2048, 7168), (129, 320, 128)]
     for m, n, k in shapes:
         for cus in (256, 128, 80):
-            assert capi.select_tile(0, m, n, k, cus) == heuristics.get_best_dense_config(m, n, k, cus), (m, n, k, cus)
+            assert capi.select_tile(0, m, n, k, cus) == heuristics.get_dense_tile(m, n, k, cus), (m, n, k, cus)
             assert capi.select_tile(1, m, n, k, cus) == heuristics.get_fp8_tile(m, n, k, cus), (m, n, k, cus)
     for m, n in [(4096, 4096), (32768, 4096), (128, 7168), (256, 200), (1024, 24576)]:
         for cus in (256, 80):

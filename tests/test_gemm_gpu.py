@@ -129,6 +129,23 @@ def test_dense_closed_forms_are_exact():
     assert oracle.calc_diff(_np(out), oracle.gemm_bf16_tn_ref(_np(a), _np(b))) < BF16_TOL
 
 
+@pytest.mark.parametrize('m,n,k', [(7, 1156, 512), (20, 100, 2112)])
+def test_dense_weight_streaming_kernel_leaves_its_neighbours_alone(m, n, k):
+    """A handful of rows runs one workgroup per 16 weight rows, the last one partly past n: rows from m on and the columns
+    past n of the last workgroup stay untouched, JIT entry and C library give the same bits."""
+    from yan_amd.jit_kernels import heuristics
+    _announce('dense weight streaming', m, n, k)
+    assert heuristics.get_dense_tile(m, n, k, yan.get_num_sms())[1] == 16
+    a, b, _ = testing.make_bf16_case(m, n, k, seed=6, device='cuda')
+    big = torch.full((m + 2, n), 7.0, dtype=torch.bfloat16, device='cuda')
+    yan.gemm_bf16_tn(a, b, big[:m])
+    assert bool((big[m:] == 7.0).all())
+    assert oracle.calc_diff(_np(big[:m]), oracle.gemm_bf16_tn_ref(_np(a), _np(b))) < BF16_TOL
+    again = torch.empty(m, n, dtype=torch.bfloat16, device='cuda')
+    assert capi.gemm_bf16_tn(a, b, again) == 0
+    assert torch.equal(again, big[:m])
+
+
 def test_dense_baseline_8192_cubed():
     """cfg2: rows sampled against the oracle, the whole matrix against a chunked fp32 matmul on the device."""
     m = n = k = 8192

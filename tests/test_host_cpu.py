@@ -69,9 +69,16 @@ def test_dense_shapes_of_the_gpu_suite_reach_every_tile_of_the_8_wave_kernel():
     import harness
     for shape, tile in harness.DENSE_TILE_OF_SHAPE.items():
         assert shape in harness.DENSE_TEST_SHAPES
-        assert heuristics.get_best_dense_config(*shape, 256) == tile, shape
-        assert heuristics.get_dense_num_stages(*tile) == (2 if tile[0] == 256 else {(128, 192): 4, (64, 192): 5}[tile])
-    assert {t for t in harness.DENSE_TILE_OF_SHAPE.values()} == {(256, 160), (256, 192), (256, 224), (256, 256), (128, 192), (64, 192)}
+        assert heuristics.get_dense_tile(*shape, 256) == tile, shape
+        if tile[1] != 16:
+            assert heuristics.get_dense_num_stages(*tile) == (2 if tile[0] == 256 else {(128, 192): 4, (64, 192): 5}[tile])
+    assert {t for t in harness.DENSE_TILE_OF_SHAPE.values()} == {(256, 160), (256, 192), (256, 224), (256, 256), (128, 192), (64, 192),
+                                                                 (16, 16), (32, 16)}
+    # the weight-streaming kernel: one round of workgroups, whole K blocks, two atoms only on long K
+    assert heuristics.get_skinny_dense_config(16, 4096, 7168, 256) == 1 and heuristics.get_skinny_dense_config(16, 4112, 7168, 256) == 0
+    assert heuristics.get_skinny_dense_config(16, 4096, 7176, 256) == 0 and heuristics.get_skinny_dense_config(33, 4096, 7168, 256) == 0
+    assert heuristics.get_skinny_dense_config(32, 4096, 1024, 256) == 0 and heuristics.get_skinny_dense_config(32, 4096, 2048, 256) == 2
+    assert heuristics.get_skinny_dense_config(16, 1024, 7168, 64) == 1 and heuristics.get_skinny_dense_config(16, 2048, 7168, 64) == 0
 
 
 def test_kernel_plans_keep_reference_keys_and_argument_order():

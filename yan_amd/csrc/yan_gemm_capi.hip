@@ -5,6 +5,7 @@
 #include "gemm/bf16_gemm.hpp"
 #include "gemm/fp8_gemm.hpp"
 #include "gemm/fp8_gemm_skinny.hpp"
+#include "gemm/bf16_gemm_skinny.hpp"
 #include "gemm/fp8_cast.hpp"
 #include "gemm/simple_gemm.hpp"
 
@@ -62,13 +63,25 @@ int device_cus() {
     return cus;
 }
 
-template <typename Atom, typename Elem>
+// Activation atoms of the weight-streaming dense kernel, or 0 for the tiled kernels (get_skinny_dense_config in heuristics.py).
+int dense_skinny_atoms(int m, int n, int k, int num_cus) {
+    if (n < 16 || n > 16 * num_cus || (n % 4) != 0 || k <= 0 || (k % 64) != 0) return 0;
+    if (m > 0 && m <= 16) return 1;
+    if (m > 16 && m <= 32 && k >= 2048) return 2;
+    return 0;
+}
+
+template <typename Atom, typename SkinnyAtom, typename Elem>
 int dense(int m, int n, int k, const void* a, const void* b, void* c, void* stream) {
     if (m == 0 || n == 0) return 0;
     if (m < 0 || n < 0) return int(hipErrorInvalidValue);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (const int atoms = dense_skinny_atoms(m, n, k, device_cus())) {
+        if (atoms == 1) return int(yan::launch_dense_skinny<SkinnyAtom, Elem, 1, 8>(m, n, k, a, b, c, s));
+        return int(yan::launch_dense_skinny<SkinnyAtom, Elem, 2, 8>(m, n, k, a, b, c, s));
+    }
     int bm = 0, bn = 0;
     pick(kDenseTiles, m, n, device_cus(), &bm, &bn);
-    hipStream_t s = static_cast<hipStream_t>(stream);
 #define YAN_DENSE_CASE(BM, BN) if (bm == BM && bn == BN) return int(yan::launch_dense<Atom, Elem, BM, BN>(m, n, k, a, b, c, s));
 #define YAN_DENSE_CASE_8W(BM, BN) if (bm == BM && bn == BN) return int(yan::launch_dense<Atom, Elem, BM, BN, 2>(m, n, k, a, b, c, s));
     YAN_DENSE_CASE_8W(256, 256) YAN_DENSE_CASE_8W(256, 224) YAN_DENSE_CASE_8W(256, 192) YAN_DENSE_CASE_8W(256, 160)
@@ -84,11 +97,11 @@ int dense(int m, int n, int k, const void* a, const void* b, void* c, void* stre
 extern "C" {
 
 int yan_gemm_bf16_tn(int m, int n, int k, const void* a, const void* b, void* c, void* stream) {
-    return dense<yan::MfmaBF16_32x32x16, __bf16>(m, n, k, a, b, c, stream);
+    return dense<yan::MfmaBF16_32x32x16, yan::MfmaBF16_16x16x32, __bf16>(m, n, k, a, b, c, stream);
 }
 
 int yan_gemm_fp16_tn(int m, int n, int k, const void* a, const void* b, void* c, void* stream) {
-    return dense<yan::MfmaF16_32x32x16, _Float16>(m, n, k, a, b, c, stream);
+    return dense<yan::MfmaF16_32x32x16, yan::MfmaF16_16x16x32, _Float16>(m, n, k, a, b, c, stream);
 }
 
 int yan_gemm_float_nt(int m, int n, int k, float alpha, const float* a, int lda, const float* b, int ldb, float beta,
@@ -182,9 +195,11 @@ int yan_per_block_cast_to_fp8(const void* w, int w_is_fp32, void* q, float* scal
 }
 
 int yan_gemm_select_tile(int op, int m, int n, int k, int num_cus, int* block_m, int* block_n) {
-    (void)k;
     if (!block_m || !block_n || num_cus <= 0) return 1;
-    if (op == 0) pick(kDenseTiles, m, n, num_cus, block_m, block_n);
+    if (op == 0) {
+        if (const int atoms = dense_skinny_atoms(m, n, k, num_cus)) { *block_m = 16 * atoms; *block_n = 16; }
+        else pick(kDenseTiles, m, n, num_cus, block_m, block_n);
+    }
     else if (op == 1) {
         if (const int atoms = skinny_atoms(m, n, num_cus)) { *block_m = 16 * atoms; *block_n = 16; }
         else pick(kFp8Tiles, m, n, num_cus, block_m, block_n);
@@ -195,6 +210,6 @@ int yan_gemm_select_tile(int op, int m, int n, int k, int num_cus, int* block_m,
     return 0;
 }
 
-const char* yan_gemm_version(void) { return "yan-gemm gfx950 11 dense + 7 fp32 + 10 fp8 tile variants + 1 weight-streaming fp8 variant + 12 grouped fp8 variants + 4 quantiser kernels"; }
+const char* yan_gemm_version(void) { return "yan-gemm gfx950 11 dense + 2 weight-streaming dense + 7 fp32 + 10 fp8 tile variants + 1 weight-streaming fp8 variant + 12 grouped fp8 variants + 4 quantiser kernels"; }
 
 } // extern "C"

@@ -29,6 +29,7 @@
 #include "mfma_utils.hpp"
 #include "scheduler.hpp"
 #include "tile_io.hpp"
+#include "bf16_gemm_skinny.hpp"
 
 namespace yan {
 
@@ -581,11 +582,14 @@ inline hipError_t launch_dense(int m, int n, int k, const void* a, const void* b
 template <int BLOCK_M, int BLOCK_N, int NUM_STAGES>
 inline hipError_t gemm_tn(int m, int n, int k, const __hip_bfloat16* A, const __hip_bfloat16* B, __hip_bfloat16* C,
                           hipStream_t stream, int num_sms = 0) {
-    return yan::launch_dense<yan::MfmaBF16_32x32x16, __bf16, BLOCK_M, BLOCK_N, NUM_STAGES>(m, n, k, A, B, C, stream, num_sms);
+    // BLOCK_N == 16 names the weight-streaming kernel for up to BLOCK_M activation rows (bf16_gemm_skinny.hpp)
+    if constexpr (BLOCK_N == 16) return yan::launch_dense_skinny<yan::MfmaBF16_16x16x32, __bf16, BLOCK_M / 16, 8>(m, n, k, A, B, C, stream);
+    else return yan::launch_dense<yan::MfmaBF16_32x32x16, __bf16, BLOCK_M, BLOCK_N, NUM_STAGES>(m, n, k, A, B, C, stream, num_sms);
 }
 
 // fp16 in, fp32 accumulate, fp16 out.
 template <int BLOCK_M, int BLOCK_N, int NUM_STAGES>
 inline hipError_t gemm_tn(int m, int n, int k, const __half* A, const __half* B, __half* C, hipStream_t stream, int num_sms = 0) {
-    return yan::launch_dense<yan::MfmaF16_32x32x16, _Float16, BLOCK_M, BLOCK_N, NUM_STAGES>(m, n, k, A, B, C, stream, num_sms);
+    if constexpr (BLOCK_N == 16) return yan::launch_dense_skinny<yan::MfmaF16_16x16x32, _Float16, BLOCK_M / 16, 8>(m, n, k, A, B, C, stream);
+    else return yan::launch_dense<yan::MfmaF16_32x32x16, _Float16, BLOCK_M, BLOCK_N, NUM_STAGES>(m, n, k, A, B, C, stream, num_sms);
 }

@@ -12,7 +12,7 @@ import functools
 
 import torch
 
-from .heuristics import get_best_dense_config, get_dense_num_stages, get_dense_tile_space, tuning_enabled
+from .heuristics import get_best_dense_config, get_dense_num_stages, get_dense_tile_space, get_skinny_dense_config, tuning_enabled
 from .tuner import FrozenKeys, jit_tuner
 from .utils import get_num_sms, get_num_sms_cap
 
@@ -36,8 +36,12 @@ def _arg_defs(dtype: torch.dtype):
 def dense_kernel_plan(m: int, n: int, k: int, dtype: torch.dtype, num_cus: int, num_sms_cap: int = 0):
     """(name, keys, arg_defs) of the JIT kernel a call with these sizes uses; needs no GPU. `num_cus` steers the tile
     choice, `num_sms_cap` (0 = none) is the number of workgroups the launch may start."""
-    block_m, block_n = get_best_dense_config(m, n, k, num_cus)
     name = 'gemm_bf16_tn' if dtype == torch.bfloat16 else 'gemm_fp16_tn'
+    skinny_atoms = get_skinny_dense_config(m, n, k, num_cus)
+    if skinny_atoms:
+        # the weight-streaming kernel for a handful of rows: BLOCK_N = 16 names it, its n / 16 workgroups are within any cap
+        return name, FrozenKeys({'BLOCK_M': 16 * skinny_atoms, 'BLOCK_N': 16, 'NUM_STAGES': 1, 'NUM_SMS': 0}), _arg_defs(dtype)
+    block_m, block_n = get_best_dense_config(m, n, k, num_cus)
     keys = FrozenKeys({'BLOCK_M': block_m, 'BLOCK_N': block_n, 'NUM_STAGES': get_dense_num_stages(block_m, block_n), 'NUM_SMS': num_sms_cap})
     return name, keys, _arg_defs(dtype)
 
@@ -65,7 +69,7 @@ def _gemm_16bit_tn(a: torch.Tensor, b: torch.Tensor, c: torch.Tensor, dtype: tor
 
     stream = torch.cuda.current_stream()
     args = (m, n, k, a, b, c, stream)
-    if tuning_enabled():
+    if tuning_enabled() and not get_skinny_dense_config(m, n, k, get_num_sms()):
         name, keys, space, arg_defs = dense_tuning_plan(m, n, k, dtype, get_num_sms(), get_num_sms_cap())
     else:
         (name, keys, arg_defs), space = dense_kernel_plan(m, n, k, dtype, get_num_sms(), get_num_sms_cap()), ()

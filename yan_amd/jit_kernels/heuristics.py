@@ -115,6 +115,30 @@ def get_skinny_fp8_config(m: int, n: int, k: int, num_cus: int) -> int:
     return 0
 
 
+def get_skinny_dense_config(m: int, n: int, k: int, num_cus: int) -> int:
+    """Number of 16-row activation atoms (1 or 2) when the weight-streaming dense kernel should run instead of the tiled
+    one, else 0: up to 32 activation rows, few enough weight rows that its n/16 workgroups fit the chip in one round, and
+    whole 128-byte K blocks. The smallest dense tile gives a workgroup 64 weight rows: n = 4096 puts 64 of 256 compute
+    units to work. Measured call to call with the weights cycling through more matrices than the caches hold (bf16,
+    n = 4096, k = 7168; weight-streaming vs 64 x 64 tiles): m = 1: 14.5 vs 25.9 us, m = 16: 18.3 vs 27.0, m = 17: 21.3 vs
+    27.1, m = 32: 25.4 vs 30.1, m = 48: 30.7 vs 33.3 (three atoms: not offered), m = 64: a tie; n = 2112 alike. Beyond one
+    round of workgroups the tiles win (n = 7168, k = 2048: 11.7 vs 10.2 us at m = 1; n = 16384, k = 4096: 34.0 vs 30.7),
+    and two atoms lose on short K (k = 1024: 7.2 vs 6.0 us)."""
+    if n < 16 or n > 16 * num_cus or n % 4 or k <= 0 or k % 64:
+        return 0
+    if 0 < m <= 16:
+        return 1
+    if 16 < m <= 32 and k >= 2048:
+        return 2
+    return 0
+
+
+def get_dense_tile(m: int, n: int, k: int, num_cus: int) -> Tuple[int, int]:
+    """(BLOCK_M, BLOCK_N) of the dense kernel that runs: (16 * atoms, 16) for the weight-streaming kernel."""
+    atoms = get_skinny_dense_config(m, n, k, num_cus)
+    return (16 * atoms, 16) if atoms else get_best_dense_config(m, n, k, num_cus)
+
+
 def get_fp8_tile(m: int, n: int, k: int, num_cus: int) -> Tuple[int, int]:
     """(BLOCK_M, BLOCK_N) of the FP8 kernel that runs: (16 * atoms, 16) for the weight-streaming kernel."""
     atoms = get_skinny_fp8_config(m, n, k, num_cus)
