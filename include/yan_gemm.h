@@ -73,6 +73,26 @@ YAN_API int yan_gemm_fp8_fp8_bf16_nt(const void* lhs, const float* lhs_scales, l
                              long long lhs_scales_stride_k, const void* rhs, const float* rhs_scales, void* out,
                              int m, int n, int k, void* stream, int num_sms);
 
+/* The same GEMM with K split over 2 to 4 workgroups per output tile where that pays: problems whose tiles would leave
+ * compute units idle and whose K is long (m up to a few hundred, k from about 4096: 64 x 4096 x 7168 runs 64 x 64 tiles in
+ * four parts). The parts leave fp32 partial sums in `workspace`; the part that arrives last adds them up in the order of
+ * their K ranges, so a result does not depend on which part that was, and stores the tile. Results are within the
+ * tolerance of the plain entry point but not bit-identical to it (a different order of summation); every other problem
+ * runs exactly as through the plain entry point.
+ *   workspace        device memory of at least yan_gemm_fp8_split_k_workspace_bytes() bytes (16.0 MB), whose first
+ *                    yan_gemm_fp8_split_k_counter_bytes() bytes (arrival counters) the caller zero-fills once, before the
+ *                    first call; every call leaves them zero again, so one workspace serves calls of any shapes;
+ *   workspace_bytes  its size; less than the problem's plan needs is hipErrorInvalidValue.
+ * Calls that share a workspace must not overlap on the device (same stream, or otherwise ordered).
+ * This is the `split` half of the reference's tile/split heuristics, which its template leaves to the caller's keys
+ * (yan/jit_kernels/gemm.py:13-18); yan_gemm_select_split_k below says what a problem gets. */
+YAN_API long long yan_gemm_fp8_split_k_workspace_bytes(void);
+YAN_API long long yan_gemm_fp8_split_k_counter_bytes(void);
+YAN_API int yan_gemm_fp8_fp8_bf16_nt_split_k(const void* lhs, const float* lhs_scales, long long lhs_scales_stride_m,
+                                     long long lhs_scales_stride_k, const void* rhs, const float* rhs_scales, void* out,
+                                     int m, int n, int k, void* stream, int num_sms, void* workspace,
+                                     long long workspace_bytes);
+
 /* Grouped (mixture-of-experts) forms of the FP8 GEMM: group g has its own weights rhs[g] ([n,k] e4m3) and scale table
  * rhs_scales[g] ([ceil(n/128)][k/128]); both arrays are contiguous over g. Arithmetic per row as above.
  * They fill in the reference's GemmType::GroupedContiguous / GroupedMasked and `int* grouped_layout` hooks
@@ -115,6 +135,11 @@ YAN_API int yan_per_block_cast_to_fp8(const void* w, int w_is_fp32, void* q, flo
  * Host-only (no device call). Stands where the reference leaves tile choice to the caller's keys
  * (yan/jit_kernels/cute_gemm.py:41, yan/jit_kernels/gemm.py:13-16). Returns 0, or 1 for an unknown op. */
 YAN_API int yan_gemm_select_tile(int op, int m, int n, int k, int num_cus, int* block_m, int* block_n);
+
+/* Split-K plan of the plain FP8 GEMM on `num_cus` compute units: writes the tile and the number of parts, or
+ * block_m = block_n = 0 and split_k = 1 when K is not split (then yan_gemm_select_tile names the tile). Host-only.
+ * Returns 0, or 1 for a null pointer or num_cus <= 0. */
+YAN_API int yan_gemm_select_split_k(int m, int n, int k, int num_cus, int* block_m, int* block_n, int* split_k);
 
 /* "yan-gemm gfx950 <n> dense + <n> fp32 + <n> fp8 tile variants + <n> weight-streaming fp8 variant + ...". */
 YAN_API const char* yan_gemm_version(void);

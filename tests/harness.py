@@ -200,6 +200,18 @@ FP8_TILE_OF_SHAPE = {(1024, 2112, 256): (128, 128), (1000, 2100, 384): (128, 128
 # multiply): listed so that their kernels are compiled ahead of time as well.
 FP8_SIDE_SHAPES = [(1024, 4096, 7168), (8192, 4096, 7168), (200, 384, 512), (1152, 512, 512), (128, 4096, 1024), (128, 320, 384),
                    (256, 200, 128), (256, 512, 512)]
+# Problems the split-K plan covers on 256 compute units, with the (BLOCK_M, BLOCK_N, SPLIT_K) it makes (a CPU test keeps this
+# true): every ring tile, every factor, ragged m and n, n that is no multiple of 8 (direct stores), K ranges of unequal
+# length (29 k-tiles in 2 parts, 43 and 56 in 3).
+FP8_SPLIT_K_PLAN_OF_SHAPE = {
+    (17, 196, 3584): (32, 32, 2), (33, 196, 5504): (32, 32, 3), (64, 196, 7168): (32, 32, 4), (31, 516, 3712): (32, 32, 2),
+    (33, 2112, 5376): (64, 32, 3), (50, 1536, 7168): (64, 32, 4), (64, 2112, 7168): (64, 32, 3),
+    (100, 2112, 5376): (64, 64, 3), (65, 1536, 7168): (64, 64, 4),
+    (200, 3076, 3584): (64, 128, 2), (100, 4100, 5376): (64, 128, 3), (129, 2112, 7168): (64, 128, 4),
+    (300, 4100, 4608): (128, 128, 2), (200, 4100, 5376): (128, 128, 3), (129, 4096, 7168): (128, 128, 4),
+    (64, 4096, 7168): (64, 64, 4), (128, 4096, 7168): (64, 128, 4),
+}
+FP8_SPLIT_K_SHAPES = [s for s in FP8_SPLIT_K_PLAN_OF_SHAPE if s not in ((64, 4096, 7168), (128, 4096, 7168))]
 # Grouped FP8 GEMMs: (rows per group, n, k, blocks of padding rows) and (groups, m_max, n, k, masked_m, expected_m).
 # Long groups on 256-row tiles whose two 128-row halves belong to different groups, or one of them to padding: a padding
 # block between the groups (negative entry) and one at the end; group 1 has 63 blocks, so it starts and the run ends on
@@ -284,10 +296,14 @@ def jit_kernels_in_use(num_cus: int = 256):
     for m, n, k in REFERENCE_FLOAT_TEST_SHAPES + FLOAT_TEST_SHAPES + [(5120, 2048, 4096)]:
         name, keys, arg_defs = simple_gemm.float_kernel_plan(m, n, num_cus)
         add(name, arg_defs, simple_gemm.includes, simple_gemm.template, keys)
-    for m, n, k in FP8_TEST_SHAPES + FP8_SIDE_SHAPES:
+    for m, n, k in FP8_TEST_SHAPES + FP8_SIDE_SHAPES + FP8_SPLIT_K_SHAPES:
         for token_contiguous in (True, False) if m else ():     # both layouts of the activation scales
             name, keys, arg_defs, _, code_template = gemm.fp8_kernel_plan(m, n, k, num_cus, token_contiguous)
             add(name, arg_defs, gemm.includes, code_template, keys)
+            split = gemm.fp8_split_k_plan(m, n, k, num_cus, token_contiguous)
+            if split is not None:
+                name, keys, arg_defs, code_template = split
+                add(name, arg_defs, gemm.includes, code_template, keys)
     for m, n, k in CAPPED_SHAPES:
         for cus, cap in ((num_cus, 0), (num_cus, NUM_SMS_CAP), (NUM_SMS_CAP, NUM_SMS_CAP)):
             name, keys, arg_defs = bf16_gemm.dense_kernel_plan(m, n, k, torch.bfloat16, cus, cap)

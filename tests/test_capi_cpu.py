@@ -7,6 +7,7 @@ import subprocess
 
 import pytest
 
+import yan_amd as yan
 from yan_amd import capi
 from yan_amd.jit_kernels import heuristics
 
@@ -23,7 +24,7 @@ def _declared(repo_root):
 
 def test_library_exports_every_declared_symbol(lib, repo_root):
     declared = _declared(repo_root)
-    assert declared == sorted(capi.SYMBOLS) and len(declared) == 10
+    assert declared == sorted(capi.SYMBOLS) and len(declared) == 14
     for name in declared:
         assert hasattr(lib, name), name
     out = subprocess.check_output(['nm', '-D', '--defined-only', os.path.join(repo_root, 'yan_amd', 'csrc', 'libyan_gemm.so')], text=True)
@@ -54,7 +55,20 @@ def test_version_and_tile_selection_match_python(lib):
                  (256, 256), (512, 4096), (1024, 1024), (2048, 2048), (256, 32768)]:
         for cus in (256, 80):
             assert capi.select_tile(3, m, n, 512, cus) == heuristics.get_best_float_config(m, n, cus), (m, n, cus)
+    # the split-K plan of the plain FP8 GEMM: same rule, same numbers on both sides
+    plans = 0
+    for m in (1, 16, 17, 32, 33, 50, 64, 65, 100, 128, 129, 200, 256, 300, 512, 700, 1024, 4096):
+        for n in (100, 196, 516, 1536, 2112, 4096, 4100, 7168, 16384, 24576):
+            for k in (128, 1536, 2048, 3072, 3200, 4608, 6144, 7168, 16384):
+                for cus in (256, 64, 40, 8):
+                    plan = capi.select_split_k(m, n, k, cus)
+                    assert plan == heuristics.get_split_k_fp8_config(m, n, k, cus), (m, n, k, cus)
+                    plans += plan is not None
+    assert plans > 500
+    assert lib.yan_gemm_fp8_split_k_workspace_bytes() == yan.gemm.SPLIT_K_WORKSPACE_BYTES == 16 * 1024 + 256 * 128 * 128 * 4
+    assert lib.yan_gemm_fp8_split_k_counter_bytes() == yan.gemm.SPLIT_K_COUNTER_BYTES
     bm, bn = ctypes.c_int(), ctypes.c_int()
+    assert lib.yan_gemm_select_split_k(64, 4096, 7168, 0, ctypes.byref(bm), ctypes.byref(bn), ctypes.byref(bm)) == 1
     assert lib.yan_gemm_select_tile(7, 1, 1, 1, 256, ctypes.byref(bm), ctypes.byref(bn)) == 1
     assert lib.yan_gemm_select_tile(0, 1, 1, 1, 0, ctypes.byref(bm), ctypes.byref(bn)) == 1
 

@@ -476,6 +476,75 @@ def test_fp8_decode_shapes_are_repeatable():
     assert oracle.calc_diff(_np(first_one), _fp8_ref(e8, se, f8, sf)) < 1e-5
 
 
+@pytest.mark.parametrize('m,n,k', testing.FP8_SPLIT_K_SHAPES)
+@pytest.mark.parametrize('col_major', [False, True])
+def test_split_k_parity_vs_oracle(m, n, k, col_major):
+    """Problems whose K the entry point splits over 2 to 4 workgroups per tile (every ring tile, every factor, ragged edges,
+    K ranges of unequal length): parity against the oracle to the bar of the unsplit kernel, the same bits from the
+    library's split-K entry point, which writes nothing past row m, and arrival counters back at zero."""
+    plan = yan.gemm.fp8_split_k_plan(m, n, k, yan.get_num_sms(), col_major)
+    assert plan is not None and (plan[1]['BLOCK_M'], plan[1]['BLOCK_N'], plan[1]['SPLIT_K']) == testing.FP8_SPLIT_K_PLAN_OF_SHAPE[(m, n, k)]
+    _announce('fp8 split-k', m, n, k, plan[1]['BLOCK_M'], plan[1]['BLOCK_N'], plan[1]['SPLIT_K'], 'col-major' if col_major else 'row-major')
+    (a8, sa), (b8, sb), out = testing.make_fp8_case(m, n, k, seed=42, device='cuda', col_major_scales=col_major)
+    out.fill_(float('nan'))
+    yan.gemm_fp8_fp8_bf16_nt((a8, sa), (b8, sb), out)
+    torch.cuda.synchronize()
+    got, ref = _np(out), _fp8_ref(a8, sa, b8, sb)
+    assert np.isfinite(got).all()
+    assert oracle.calc_diff(got, ref) < 1e-5
+    assert bool(np.all(np.abs(got - ref) <= np.abs(ref) * 2.0 ** -7 + 1e-4 * np.abs(ref).max()))
+    workspace = capi.split_k_workspace()
+    padded = torch.full((m + 3, n), 7.0, dtype=torch.bfloat16, device='cuda')
+    assert capi.gemm_fp8_fp8_bf16_nt_split_k((a8, sa), (b8, sb), padded, workspace) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(padded[:m], out) and bool((padded[m:] == 7.0).all())
+    counters = capi.load().yan_gemm_fp8_split_k_counter_bytes()
+    assert int(workspace[:counters].view(torch.int32).abs().sum()) == 0
+
+
+def test_split_k_launches_of_different_shapes_share_a_workspace():
+    """One workspace per stream serves every split-K launch on it: shapes with different tiles and factors interleaved,
+    the caches flushed between some rounds so that the parts arrive in another order, give the same bits every time (the
+    part that arrives last adds the parts up in the order of their K ranges, whichever it is)."""
+    shapes = [(64, 4096, 7168), (33, 2112, 5376), (300, 4100, 4608), (129, 2112, 7168), (17, 196, 3584)]
+    cases = [testing.make_fp8_case(*shape, seed=5 + i, device='cuda', gen_device='cuda') for i, shape in enumerate(shapes)]
+    firsts = []
+    for (lhs, rhs, out) in cases:
+        yan.gemm_fp8_fp8_bf16_nt(lhs, rhs, out)
+        firsts.append(out.clone())
+    for ((a8, sa), (b8, sb), out), first in zip(cases, firsts):
+        assert float(yan.calc_diff(first.float(), testing.dequant_lhs(a8, sa) @ testing.dequant_rhs(b8, sb).t())) < 1e-5
+    flush = torch.empty(512 << 18, dtype=torch.int, device='cuda')
+    for it in range(12):
+        if it % 3 == 0:
+            flush.zero_()
+        for (lhs, rhs, out) in cases:
+            out.fill_(float('nan'))
+            yan.gemm_fp8_fp8_bf16_nt(lhs, rhs, out)
+        for (_, _, out), first in zip(cases, firsts):
+            assert torch.equal(out, first), it
+
+
+def test_split_k_entry_point_checks_its_workspace():
+    """A workspace smaller than the plan needs, or none, is an error and launches nothing; problems whose K is not split
+    do not look at it."""
+    (a8, sa), (b8, sb), out = testing.make_fp8_case(64, 4096, 7168, seed=1, device='cuda', gen_device='cuda')
+    out.fill_(3.0)
+    small = torch.zeros(1 << 20, dtype=torch.uint8, device='cuda')
+    assert capi.gemm_fp8_fp8_bf16_nt_split_k((a8, sa), (b8, sb), out, small) == 1          # hipErrorInvalidValue
+    lib = capi.load()
+    assert lib.yan_gemm_fp8_fp8_bf16_nt_split_k(a8.data_ptr(), sa.data_ptr(), sa.stride(0), sa.stride(1), b8.data_ptr(), sb.data_ptr(),
+                                                out.data_ptr(), 64, 4096, 7168, None, 0, None, 1 << 30) == 1
+    torch.cuda.synchronize()
+    assert bool((out == 3.0).all())
+    (c8, sc), (d8, sd), out2 = testing.make_fp8_case(300, 96, 640, seed=2, device='cuda')
+    assert capi.select_split_k(300, 96, 640, yan.get_num_sms()) is None
+    assert capi.gemm_fp8_fp8_bf16_nt_split_k((c8, sc), (d8, sd), out2, small) == 0
+    plain = torch.zeros_like(out2)
+    assert capi.gemm_fp8_fp8_bf16_nt((c8, sc), (d8, sd), plain) == 0
+    assert torch.equal(out2, plain)
+
+
 @pytest.mark.parametrize('m,n,k', [(128, 4096, 7168), (512, 4096, 2048), (1024, 7168, 1024)])
 def test_ring_of_stages_is_race_free(m, n, k):
     """Tiles below 256 x 256 keep several k-tiles in flight in a ring of LDS stages, synchronised by counting the
@@ -919,7 +988,13 @@ def test_capi_fp8_matches_oracle_and_jit(m, n, k):
     assert capi.gemm_fp8_fp8_bf16_nt((a8, yan.get_col_major_tensor(sa)), (b8, sb), out_cm) == 0
     out_jit = torch.zeros_like(out)
     yan.gemm_fp8_fp8_bf16_nt((a8, sa), (b8, sb), out_jit)
-    assert torch.equal(out, out_cm) and torch.equal(out, out_jit)
+    assert torch.equal(out, out_cm)
+    if yan.gemm.fp8_split_k_plan(m, n, k, yan.get_num_sms()) is None:
+        assert torch.equal(out, out_jit)
+    else:       # the JIT entry splits K; so does the library when it is handed a workspace: same plan, same bits
+        out_split = torch.zeros_like(out)
+        assert capi.gemm_fp8_fp8_bf16_nt_split_k((a8, sa), (b8, sb), out_split, capi.split_k_workspace()) == 0
+        assert torch.equal(out_split, out_jit) and oracle.calc_diff(_np(out_jit), _fp8_ref(a8, sa, b8, sb)) < 1e-5
 
 
 def test_entry_points_replay_correctly_from_a_captured_graph():

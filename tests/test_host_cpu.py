@@ -51,6 +51,42 @@ def test_tile_heuristics_fill_256_cus():
     assert ranked == sorted(ranked) and len(ranked) == len(heuristics._FP8_TILES)
 
 
+def test_split_k_plans():
+    """K is split when the unsplit tiles leave the chip short of work and K is long; every plan fits one round of
+    workgroups and the workspace, leaves each part 14 k-tiles or more, and the shapes of the GPU suite get the plans the
+    suite expects (every ring tile, every factor)."""
+    import harness
+    plan = heuristics.get_split_k_fp8_config
+    assert plan(64, 4096, 7168, 256) == (64, 64, 4) and plan(32, 2112, 7168, 256) == (32, 32, 3)
+    assert plan(256, 7168, 7168, 256) == (128, 128, 2) and plan(128, 7168, 16384, 256) == (128, 128, 4)
+    # short K, a weight matrix that takes as long to stream as to multiply, work for every compute unit, few rows
+    assert plan(64, 7168, 2048, 256) is None and plan(64, 16384, 7168, 256) is None and plan(4096, 7168, 7168, 256) is None
+    assert plan(16, 4096, 7168, 256) is None and plan(0, 4096, 7168, 256) is None
+    for shape, expected in harness.FP8_SPLIT_K_PLAN_OF_SHAPE.items():
+        assert plan(*shape, 256) == expected, shape
+    assert {(bm, bn) for bm, bn, _ in harness.FP8_SPLIT_K_PLAN_OF_SHAPE.values()} == set(heuristics._FP8_SPLIT_K_TILE_US)
+    assert {s for _, _, s in harness.FP8_SPLIT_K_PLAN_OF_SHAPE.values()} == set(heuristics.FP8_SPLIT_K_FACTORS)
+    for m in (17, 33, 64, 100, 129, 256, 300, 512, 1024):
+        for n in (196, 1536, 2112, 4096, 4100, 7168, 24576):
+            for k in (1536, 3072, 3200, 4608, 7168, 16384):
+                for cus in (256, 64, 8):
+                    p = plan(m, n, k, cus)
+                    if p is None:
+                        continue
+                    bm, bn, split = p
+                    slots = yan.ceil_div(yan.ceil_div(m, bm) * yan.ceil_div(n, bn), 8) * 8
+                    assert slots * split <= cus and yan.ceil_div(k // 128, split) >= 14
+                    assert gemm.SPLIT_K_COUNTER_BYTES + slots * split * bm * bn * 4 <= gemm.SPLIT_K_WORKSPACE_BYTES
+                    assert slots * 8 * 4 <= gemm.SPLIT_K_COUNTER_BYTES
+                    assert heuristics.get_fp8_num_stages(bm, bn) > 2          # a ring tile
+    name, keys, defs, tmpl = gemm.fp8_split_k_plan(64, 4096, 7168, 256)
+    assert name == 'gemm_fp8_fp8_bf16_nt_split_k' and keys['SPLIT_K'] == 4 and defs[-2:] == (('workspace', torch.uint8), ('workspace_bytes', int))
+    assert 'run_split_k<4>' in yan.jit.cpp_format(tmpl, keys)
+    strided = gemm.fp8_split_k_plan(64, 4096, 7168, 256, False)
+    assert strided[0].endswith('_strided') and strided[2][-2:] == (('lhs_scales_stride_m', int), ('lhs_scales_stride_k', int))
+    assert gemm.fp8_split_k_plan(4096, 7168, 7168, 256) is None
+
+
 def test_fp8_shapes_of_the_gpu_suite_reach_every_tile_of_the_cost_table():
     import harness
     for shape, tile in harness.FP8_TILE_OF_SHAPE.items():

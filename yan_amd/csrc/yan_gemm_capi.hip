@@ -9,6 +9,8 @@
 #include "gemm/fp8_cast.hpp"
 #include "gemm/simple_gemm.hpp"
 
+#include <mutex>
+
 namespace {
 
 struct TileCost { int bm, bn; double per_area; };
@@ -53,6 +55,38 @@ int skinny_atoms(int m, int n, int num_cus) {
     return (m > 0 && m <= 16 && n >= 16 && n <= 16 * num_cus) ? 1 : 0;
 }
 
+// Split-K plan of the plain FP8 GEMM (get_split_k_fp8_config in heuristics.py): false when K is not split.
+struct SplitKTile { int bm, bn; double us_per_k_tile; };
+constexpr SplitKTile kSplitKTiles[] = {{32, 32, 0.133}, {64, 32, 0.192}, {64, 64, 0.296}, {64, 128, 0.395}, {128, 128, 0.51}};
+constexpr int kSplitKFactors[] = {2, 3, 4};
+
+bool pick_split_k(int m, int n, int k, int num_cus, int* bm, int* bn, int* split_k) {
+    if (m <= 0 || n <= 0 || k <= 0 || skinny_atoms(m, n, num_cus)) return false;
+    const int k_tiles = k / 128;
+    int ubm = 0, ubn = 0;
+    pick(kFp8Tiles, m, n, num_cus, &ubm, &ubn);
+    double unsplit_us = -1;
+    for (const SplitKTile& t : kSplitKTiles)
+        if (t.bm == ubm && t.bn == ubn) unsplit_us = t.us_per_k_tile;
+    if (unsplit_us < 0 || (long long)((m + ubm - 1) / ubm) * ((n + ubn - 1) / ubn) > num_cus) return false;
+    const double floor = double((long long)n * k) / 6.0e6;
+    const double unsplit_time = k_tiles * unsplit_us;
+    const double base = unsplit_time > floor ? unsplit_time : floor;
+    double best = -1;
+    for (const SplitKTile& t : kSplitKTiles) {
+        if (t.bm > 32 && t.bm >= 2 * m) continue;
+        const long long tiles = (long long)((m + t.bm - 1) / t.bm) * ((n + t.bn - 1) / t.bn);
+        for (const int s : kSplitKFactors) {
+            const int per_part = (k_tiles + s - 1) / s;
+            if ((tiles + 7) / 8 * 8 * s > (num_cus < 256 ? num_cus : 256) || per_part < 14) continue;
+            const double loop = per_part * t.us_per_k_tile + 0.5 + double(s * t.bm * t.bn * 4) / 1024 * 0.0125;
+            const double time = loop > floor ? loop : floor;
+            if (best < 0 || time < best) { best = time; *bm = t.bm; *bn = t.bn; *split_k = s; }
+        }
+    }
+    return best >= 0 && base - best >= 0.10 * (base + 3.5);
+}
+
 int device_cus() {
     static int cus = 0;
     if (cus == 0) {
@@ -92,6 +126,45 @@ int dense(int m, int n, int k, const void* a, const void* b, void* c, void* stre
     return int(hipErrorInvalidValue);
 }
 
+// The plain FP8 GEMM. With a workspace, problems the split-K plan covers run split (a workspace too small for the plan is
+// an error); without one, and for every other problem, a workgroup per tile as before.
+int fp8_plain(const void* lhs, const float* lhs_scales, long long lhs_scales_stride_m, long long lhs_scales_stride_k,
+              const void* rhs, const float* rhs_scales, void* out, int m, int n, int k, void* stream, int num_sms,
+              void* workspace, size_t workspace_bytes) {
+    if (m == 0 || n == 0) return 0;
+    if (m < 0 || n < 0 || k <= 0) return int(hipErrorInvalidValue);
+    // the kernel addresses the scale tensor with 32-bit byte offsets
+    const long long last = (long long)(m - 1) * lhs_scales_stride_m + (long long)(k / 128 - 1) * lhs_scales_stride_k;
+    if (lhs_scales_stride_m < 0 || lhs_scales_stride_k < 0 || last >= (1ll << 28)) return int(hipErrorInvalidValue);
+    const int cus = (num_sms > 0 && num_sms < device_cus()) ? num_sms : device_cus();
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    __hip_bfloat16* o = static_cast<__hip_bfloat16*>(out);
+    if (skinny_atoms(m, n, cus))
+        return int(yan::launch_fp8_skinny<0, 0, 1, 8>(o, lhs, lhs_scales, int(lhs_scales_stride_m), int(lhs_scales_stride_k), rhs,
+                                                      rhs_scales, m, n, k, s));
+    int bm = 0, bn = 0, split_k = 1;
+    if (workspace && pick_split_k(m, n, k, cus, &bm, &bn, &split_k)) {
+#define YAN_SPLIT_K_CASE(BM, BN, S)                                                                                  \
+    if (bm == BM && bn == BN && split_k == S)                                                                        \
+        return int(yan::Gemm<0, 0, BM, BN, 128, 1, yan::Fp8TileConfig<BM, BN>::MAX_RING_STAGES, 1, yan::GemmType::Normal>::run_split_k<S>( \
+            o, lhs, lhs_scales, int(lhs_scales_stride_m), int(lhs_scales_stride_k), rhs, rhs_scales, m, n, k, s, workspace, workspace_bytes));
+#define YAN_SPLIT_K_TILE(BM, BN) YAN_SPLIT_K_CASE(BM, BN, 2) YAN_SPLIT_K_CASE(BM, BN, 3) YAN_SPLIT_K_CASE(BM, BN, 4)
+        YAN_SPLIT_K_TILE(32, 32) YAN_SPLIT_K_TILE(64, 32) YAN_SPLIT_K_TILE(64, 64) YAN_SPLIT_K_TILE(64, 128) YAN_SPLIT_K_TILE(128, 128)
+#undef YAN_SPLIT_K_TILE
+#undef YAN_SPLIT_K_CASE
+        return int(hipErrorInvalidValue);
+    }
+    pick(kFp8Tiles, m, n, cus, &bm, &bn);
+#define YAN_FP8_CASE(BM, BN)                                                                                         \
+    if (bm == BM && bn == BN)                                                                                        \
+        return int(yan::Gemm<0, 0, BM, BN, 128, 1, yan::Fp8TileConfig<BM, BN>::MAX_RING_STAGES, 1, yan::GemmType::Normal>::run_sized(                          \
+            o, lhs, lhs_scales, int(lhs_scales_stride_m), int(lhs_scales_stride_k), rhs, rhs_scales, m, n, k, s, num_sms, 0));
+    YAN_FP8_CASE(256, 256) YAN_FP8_CASE(256, 192) YAN_FP8_CASE(256, 160) YAN_FP8_CASE(256, 128) YAN_FP8_CASE(128, 256) YAN_FP8_CASE(128, 128) YAN_FP8_CASE(64, 128) YAN_FP8_CASE(64, 64)
+    YAN_FP8_CASE(64, 32) YAN_FP8_CASE(32, 32)
+#undef YAN_FP8_CASE
+    return int(hipErrorInvalidValue);
+}
+
 } // namespace
 
 extern "C" {
@@ -112,27 +185,19 @@ int yan_gemm_float_nt(int m, int n, int k, float alpha, const float* a, int lda,
 int yan_gemm_fp8_fp8_bf16_nt(const void* lhs, const float* lhs_scales, long long lhs_scales_stride_m,
                              long long lhs_scales_stride_k, const void* rhs, const float* rhs_scales, void* out,
                              int m, int n, int k, void* stream, int num_sms) {
-    if (m == 0 || n == 0) return 0;
-    if (m < 0 || n < 0 || k <= 0) return int(hipErrorInvalidValue);
-    // the kernel addresses the scale tensor with 32-bit byte offsets
-    const long long last = (long long)(m - 1) * lhs_scales_stride_m + (long long)(k / 128 - 1) * lhs_scales_stride_k;
-    if (lhs_scales_stride_m < 0 || lhs_scales_stride_k < 0 || last >= (1ll << 28)) return int(hipErrorInvalidValue);
-    const int cus = (num_sms > 0 && num_sms < device_cus()) ? num_sms : device_cus();
-    hipStream_t s = static_cast<hipStream_t>(stream);
-    __hip_bfloat16* o = static_cast<__hip_bfloat16*>(out);
-    if (skinny_atoms(m, n, cus))
-        return int(yan::launch_fp8_skinny<0, 0, 1, 8>(o, lhs, lhs_scales, int(lhs_scales_stride_m), int(lhs_scales_stride_k), rhs,
-                                                      rhs_scales, m, n, k, s));
-    int bm = 0, bn = 0;
-    pick(kFp8Tiles, m, n, cus, &bm, &bn);
-#define YAN_FP8_CASE(BM, BN)                                                                                         \
-    if (bm == BM && bn == BN)                                                                                        \
-        return int(yan::Gemm<0, 0, BM, BN, 128, 1, yan::Fp8TileConfig<BM, BN>::MAX_RING_STAGES, 1, yan::GemmType::Normal>::run_sized(                          \
-            o, lhs, lhs_scales, int(lhs_scales_stride_m), int(lhs_scales_stride_k), rhs, rhs_scales, m, n, k, s, num_sms, 0));
-    YAN_FP8_CASE(256, 256) YAN_FP8_CASE(256, 192) YAN_FP8_CASE(256, 160) YAN_FP8_CASE(256, 128) YAN_FP8_CASE(128, 256) YAN_FP8_CASE(128, 128) YAN_FP8_CASE(64, 128) YAN_FP8_CASE(64, 64)
-    YAN_FP8_CASE(64, 32) YAN_FP8_CASE(32, 32)
-#undef YAN_FP8_CASE
-    return int(hipErrorInvalidValue);
+    return fp8_plain(lhs, lhs_scales, lhs_scales_stride_m, lhs_scales_stride_k, rhs, rhs_scales, out, m, n, k, stream, num_sms,
+                     nullptr, 0);
+}
+
+long long yan_gemm_fp8_split_k_workspace_bytes(void) { return (long long)yan::kSplitKWorkspaceBytes; }
+long long yan_gemm_fp8_split_k_counter_bytes(void) { return (long long)yan::kSplitKCounterBytes; }
+
+int yan_gemm_fp8_fp8_bf16_nt_split_k(const void* lhs, const float* lhs_scales, long long lhs_scales_stride_m,
+                                     long long lhs_scales_stride_k, const void* rhs, const float* rhs_scales, void* out,
+                                     int m, int n, int k, void* stream, int num_sms, void* workspace, long long workspace_bytes) {
+    if (!workspace || workspace_bytes < 0) return int(hipErrorInvalidValue);
+    return fp8_plain(lhs, lhs_scales, lhs_scales_stride_m, lhs_scales_stride_k, rhs, rhs_scales, out, m, n, k, stream, num_sms,
+                     workspace, size_t(workspace_bytes));
 }
 
 int yan_m_grouped_gemm_fp8_fp8_bf16_nt_contiguous(const void* lhs, const float* lhs_scales, long long lhs_scales_stride_m,
@@ -210,6 +275,12 @@ int yan_gemm_select_tile(int op, int m, int n, int k, int num_cus, int* block_m,
     return 0;
 }
 
-const char* yan_gemm_version(void) { return "yan-gemm gfx950 11 dense + 2 weight-streaming dense + 7 fp32 + 10 fp8 tile variants + 1 weight-streaming fp8 variant + 12 grouped fp8 variants + 4 quantiser kernels"; }
+int yan_gemm_select_split_k(int m, int n, int k, int num_cus, int* block_m, int* block_n, int* split_k) {
+    if (!block_m || !block_n || !split_k || num_cus <= 0) return 1;
+    if (!pick_split_k(m, n, k, num_cus, block_m, block_n, split_k)) { *block_m = *block_n = 0; *split_k = 1; }
+    return 0;
+}
+
+const char* yan_gemm_version(void) { return "yan-gemm gfx950 11 dense + 2 weight-streaming dense + 7 fp32 + 10 fp8 tile variants + 15 split-K fp8 variants + 1 weight-streaming fp8 variant + 12 grouped fp8 variants + 4 quantiser kernels"; }
 
 } // extern "C"

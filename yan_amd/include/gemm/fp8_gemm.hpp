@@ -20,6 +20,9 @@
 //     16 bytes per lane in row runs of 2 * WTN bytes (non-temporal when the output is larger than the L2s together);
 //   * the plain GEMM on the 256-row tiles is a persistent walk: one workgroup per compute unit takes tile after tile and
 //     overlaps the seams (fp8_gemm_walk); every other case runs a workgroup per tile, or a plain loop under a cap;
+//   * problems with long K and fewer tiles than compute units split K over SPLIT_K workgroups per tile on the ring tiles
+//     (fp8_gemm_split_k_kernel, the `split` of the reference's tile/split heuristics): the parts meet in a caller-provided
+//     workspace, the last to arrive adds them up in the order of their K ranges and stores the tile (fp8_meet_partials);
 //   * m is a run-time argument with tails predicated; N and K are compile-time in the JIT kernels and run-time (template
 //     arguments 0) in the ahead-of-time library;
 //   * grouped (mixture-of-experts) layouts, the reference's GemmType::GroupedContiguous / GroupedMasked hooks
@@ -211,14 +214,63 @@ fp8_store_slab(const f32x4 (&acc)[TN][TM], uint8_t* region, __amdgpu_buffer_rsrc
 // GroupedMasked:     lhs [G, m, K], out [G, m, N], rhs as above; only the first grouped_layout[g] rows of group g
 //                    are computed; lhs_scales of group g start at g * sa_stride_g floats. Slots are numbered by
 //                    MaskedSlots: the tile rows below `expected_m` of all groups first.
+// Where the SPLIT_K parts of a tile meet. Wave w of every part leaves its sums in `partials` (laid out as the registers
+// are: part, wave, atom, lane) and counts itself in at counters[tile * NW + w]; the wave that arrives last adds the parts
+// up in the order of their K ranges, whichever it was itself, puts the counter back to zero for the next launch and
+// returns true: it stores the tile. The counters must be zero before the first launch.
+// The parts run on different XCDs, whose L2s do not see each other's lines. The sums are therefore written and read at
+// device scope (cache policy sc1: written through to memory, read from there), as the counter is; a device-scope fence
+// instead would write back and invalidate the whole L2 of the XCD once per wave (measured: 45-110 us for a 10 us GEMM).
+constexpr int kDeviceScope = 16;        // cache-policy bit sc1 of gfx950 buffer instructions
+// The arrival counters take the first kSplitKCounterBytes of a split-K workspace whatever the problem, so that launches of
+// different shapes can share one; the largest plan of the tile heuristics (256 workgroups of 128 x 128 partial sums)
+// fits kSplitKWorkspaceBytes.
+constexpr size_t kSplitKCounterBytes = 16 * 1024, kSplitKWorkspaceBytes = kSplitKCounterBytes + size_t(256) * 128 * 128 * 4;
+template <int SPLIT_K, int NW, int TN, int TM>
+__device__ __forceinline__ bool
+fp8_meet_partials(f32x4 (&acc)[TN][TM], float* __restrict__ partials, unsigned* __restrict__ counters, int tile_slot, int split, int wave, int lane) {
+    constexpr uint32_t ATOM_BYTES = kWaveSize * 16, WAVE_BYTES = TN * TM * ATOM_BYTES, PART_BYTES = NW * WAVE_BYTES;
+    const __amdgpu_buffer_rsrc_t parts = make_rsrc(partials + size_t(tile_slot) * (SPLIT_K * PART_BYTES / 4), SPLIT_K * PART_BYTES);
+    const uint32_t lane_off = uint32_t(wave) * WAVE_BYTES + lane * 16;
+#pragma unroll
+    for (int i = 0; i < TN; ++i)
+#pragma unroll
+        for (int j = 0; j < TM; ++j)
+            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(i32x4, acc[i][j]), parts, lane_off + (i * TM + j) * ATOM_BYTES,
+                                                   split * PART_BYTES, kDeviceScope);
+    // the sums have reached memory before the count is taken
+    __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, kNoWaitLgkm));
+    asm volatile("" ::: "memory");
+    unsigned before = 0;
+    if (lane == 0) before = __hip_atomic_fetch_add(counters + tile_slot * NW + wave, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    before = __builtin_amdgcn_readfirstlane(before);
+    asm volatile("" ::: "memory");
+    if (before != SPLIT_K - 1) return false;
+#pragma unroll
+    for (int i = 0; i < TN; ++i)
+#pragma unroll
+        for (int j = 0; j < TM; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int s = 0; s < SPLIT_K; ++s)
+#pragma unroll
+        for (int i = 0; i < TN; ++i)
+#pragma unroll
+            for (int j = 0; j < TM; ++j)
+                acc[i][j] += __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(parts, lane_off + (i * TM + j) * ATOM_BYTES,
+                                                                                             s * PART_BYTES, kDeviceScope));
+    if (lane == 0) __hip_atomic_store(counters + tile_slot * NW + wave, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return true;
+}
+
 // STAGES: 2 = two LDS stages with the next k-tile's scales in registers; 3.. = a ring of that many stages.
 // One output tile (one slot of the launch: `bid` is what blockIdx.x would be with a workgroup per slot).
-template <int SHAPE_N, int SHAPE_K, int BLOCK_M, int BLOCK_N, GemmType kGemmType, int STAGES>
+template <int SHAPE_N, int SHAPE_K, int BLOCK_M, int BLOCK_N, GemmType kGemmType, int STAGES, int SPLIT_K = 1>
 __device__ __forceinline__ void
 fp8_gemm_tile(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_scales,
               const uint8_t* __restrict__ rhs, const float* __restrict__ rhs_scales,
               __bf16* __restrict__ out, int m, int n_rt, int k_rt, int sa_stride_m, int sa_stride_k,
-              const int* __restrict__ grouped_layout, int sa_stride_g, int bid, int num_groups, int expected_m, Fp8TwoStages two_stages) {
+              const int* __restrict__ grouped_layout, int sa_stride_g, int bid, int num_groups, int expected_m, Fp8TwoStages two_stages,
+              float* __restrict__ partials = nullptr, unsigned* __restrict__ counters = nullptr) {
     using Cfg  = Fp8TileConfig<BLOCK_M, BLOCK_N>;
     using Atom = MfmaFP8_16x16x128;
     // NW waves compute (and copy); LW are launched: the extra ones of the decode tiles only copy.
@@ -230,6 +282,19 @@ fp8_gemm_tile(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_sca
     const int NUM_K_BLOCKS = K / 128, NUM_N_BLOCKS = ceil_div(N, 128);
 
     static_assert(STAGES == 2 || (STAGES >= 3 && STAGES <= Cfg::MAX_RING_STAGES), "no ring of this depth for this tile");
+
+    // SPLIT_K > 1: launch slot `bid` is part `bid % SPLIT_K` of tile slot `bid / SPLIT_K`: the k-tiles [kb_lo, kb_hi) of it.
+    int kb_lo = 0, kb_hi = NUM_K_BLOCKS;
+    [[maybe_unused]] int split = 0;
+    if constexpr (SPLIT_K > 1) {
+        static_assert(kGemmType == GemmType::Normal && STAGES > 2, "K is split for plain GEMMs on ring tiles");
+        split = bid % SPLIT_K;
+        bid /= SPLIT_K;
+        const int per = ceil_div(NUM_K_BLOCKS, SPLIT_K);
+        kb_lo = min(split * per, NUM_K_BLOCKS);
+        kb_hi = min(kb_lo + per, NUM_K_BLOCKS);
+    }
+    [[maybe_unused]] const int tile_slot = bid;
 
     // a plain GEMM whose operands outgrow the memory-side cache walks its tiles in region order (scheduler.hpp)
     const XcdTileScheduler<> sched(m, N, BLOCK_M, BLOCK_N, kGemmType == GemmType::Normal ? (long long)K : 0);
@@ -279,6 +344,8 @@ fp8_gemm_tile(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_sca
 
     const __amdgpu_buffer_rsrc_t rsrc_a = make_rsrc(lhs, uint32_t(m) * K);
     __amdgpu_buffer_rsrc_t rsrc_b = make_rsrc(rhs, uint32_t(N) * K);
+    // copies of k-tiles past the end of the range keep the count of instructions in flight and move nothing
+    const __amdgpu_buffer_rsrc_t rsrc_none = make_rsrc(lhs, 0);
     TileStager<BLOCK_M, NW> stage_a;
     TileStager<BLOCK_N, NW> stage_b;
     stage_a.init(m0, K, wave, lane);
@@ -391,11 +458,12 @@ fp8_gemm_tile(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_sca
     __shared__ __attribute__((aligned(1024))) uint8_t ring[STAGES * STAGE_BYTES];
     const uint32_t scale_voff = uint32_t(m0 + lane) * sa_stride_m * 4;
     auto issue_op = [&](int d, int kb, uint8_t* stage) {
-        if (d < StA::PASSES) stage_a.issue_pass(rsrc_a, stage, kb * kRowBytes, wave, d);
-        else if (d < StA::PASSES + StB::PASSES) stage_b.issue_pass(rsrc_b, stage + A_BYTES, kb * kRowBytes, wave, d - StA::PASSES);
+        const bool live = kb < kb_hi;
+        if (d < StA::PASSES) stage_a.issue_pass(live ? rsrc_a : rsrc_none, stage, kb * kRowBytes, wave, d);
+        else if (d < StA::PASSES + StB::PASSES) stage_b.issue_pass(live ? rsrc_b : rsrc_none, stage + A_BYTES, kb * kRowBytes, wave, d - StA::PASSES);
         else {
             const int part = wave % SCALE_PARTS;                    // rows m0 + 64 * part + lane
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_sa, YAN_LDS_PTR(stage + TILE_BYTES + part * 256), 4,
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(live ? rsrc_sa : rsrc_none, YAN_LDS_PTR(stage + TILE_BYTES + part * 256), 4,
                                                      scale_voff, (kb * sa_stride_k + part * 64 * sa_stride_m) * 4, 0, 0);
         }
     };
@@ -421,22 +489,23 @@ fp8_gemm_tile(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_sca
     }
     auto issue_slot = [&](int sl, int kb, uint8_t* stage) {
         const int o = sl * LW + wave;
+        const bool live = kb < kb_hi;
         // which kind of operation a slot holds is known at compile time unless the slot straddles two kinds
         const bool data = sl * LW + LW - 1 < GROUPS_AB || (sl * LW < GROUPS_AB && o < GROUPS_AB);
         const bool in_a = sl * LW + LW - 1 < GA || (sl * LW < GA && o < GA);
         if (data) {
-            if (in_a) __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, YAN_LDS_PTR(stage + o * 8 * kRowBytes), kChunk, slot_voff[sl], kb * kRowBytes, 0, 0);
-            else __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, YAN_LDS_PTR(stage + o * 8 * kRowBytes), kChunk, slot_voff[sl], kb * kRowBytes, 0, 0);
+            if (in_a) __builtin_amdgcn_raw_ptr_buffer_load_lds(live ? rsrc_a : rsrc_none, YAN_LDS_PTR(stage + o * 8 * kRowBytes), kChunk, slot_voff[sl], kb * kRowBytes, 0, 0);
+            else __builtin_amdgcn_raw_ptr_buffer_load_lds(live ? rsrc_b : rsrc_none, YAN_LDS_PTR(stage + o * 8 * kRowBytes), kChunk, slot_voff[sl], kb * kRowBytes, 0, 0);
         } else {
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_sa, YAN_LDS_PTR(stage + TILE_BYTES), 4, scale_voff, kb * sa_stride_k * 4, 0, 0);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(live ? rsrc_sa : rsrc_none, YAN_LDS_PTR(stage + TILE_BYTES), 4, scale_voff, kb * sa_stride_k * 4, 0, 0);
         }
     };
 #pragma unroll
     for (int t = 0; t < STAGES - G; ++t)
 #pragma unroll
-        for (int sl = 0; sl < SLOTS; ++sl) issue_slot(sl, t, ring + t * STAGE_BYTES);
+        for (int sl = 0; sl < SLOTS; ++sl) issue_slot(sl, kb_lo + t, ring + t * STAGE_BYTES);
     int base = 0;          // ring position of the group's first k-tile; STAGES is a multiple of G, groups never wrap
-    for (int kb0 = 0; kb0 < NUM_K_BLOCKS; kb0 += G) {
+    for (int kb0 = kb_lo; kb0 < kb_hi; kb0 += G) {
         __builtin_amdgcn_s_waitcnt(waitcnt_imm((STAGES - 2 * G) * SLOTS, kNoWaitLgkm));
         asm volatile("" ::: "memory");
         __builtin_amdgcn_s_barrier();
@@ -473,7 +542,7 @@ fp8_gemm_tile(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_sca
         }
 #pragma unroll
         for (int t = 0; t < G; ++t) {
-            if (kb0 + t < NUM_K_BLOCKS) {          // wave-uniform; k-tiles past the end hold bytes of other rows
+            if (kb0 + t < kb_hi) {          // wave-uniform; nothing was copied for k-tiles past the end
 #pragma unroll
                 for (int i = 0; i < TN; ++i)
 #pragma unroll
@@ -492,10 +561,10 @@ fp8_gemm_tile(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_sca
 #pragma unroll
     for (int t = 0; t < STAGES - 1; ++t)
 #pragma unroll
-        for (int d = 0; d < OPS; ++d) issue_op(d, t, ring + t * STAGE_BYTES);
-    load_weight_scales(0);
+        for (int d = 0; d < OPS; ++d) issue_op(d, kb_lo + t, ring + t * STAGE_BYTES);
+    load_weight_scales(min(kb_lo, NUM_K_BLOCKS - 1));
     int st = 0;
-    for (int kb = 0; kb < NUM_K_BLOCKS; ++kb) {
+    for (int kb = kb_lo; kb < kb_hi; ++kb) {
 #pragma unroll
         for (int b = 0; b < NB; ++b) sb_cur[b] = sb_next[b];
         __builtin_amdgcn_s_waitcnt(waitcnt_imm((STAGES - 2) * OPS, kNoWaitLgkm));
@@ -543,10 +612,14 @@ fp8_gemm_tile(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_sca
         // has no registers to spare for addresses computed ahead of time.
         int lane_late = lane;
         asm volatile("" : "+v"(lane_late));
+        if constexpr (SPLIT_K > 1)
+            if (!fp8_meet_partials<SPLIT_K, NW, TN, TM>(acc, partials, counters, tile_slot, split, wave, lane_late)) return;
         uint8_t* region = (wave < NW / 2 ? epi_a : epi_b) + (wave % (NW / 2)) * REGION;
         fp8_store_slab<Cfg, kStagedEpilogue>(acc, region, rsrc_out, m_slab, n_slab, m0, n0, pass_lo[pass], pass_hi[pass], N, stream_out, lane_late);
     } else {
         if (LW > NW && wave >= NW) return;              // waves that only copy
+        if constexpr (SPLIT_K > 1)
+            if (!fp8_meet_partials<SPLIT_K, NW, TN, TM>(acc, partials, counters, tile_slot, split, wave, lane)) return;
         fp8_store_slab<Cfg, false>(acc, nullptr, rsrc_out, m_slab, n_slab, m0, n0, pass_lo[pass], pass_hi[pass], N, stream_out, lane);
     }
     }   // pass
@@ -758,6 +831,18 @@ fp8_gemm_kernel(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_s
     }
 }
 
+// The same tiles with K split SPLIT_K ways: launch slot s is part s % SPLIT_K of tile slot s / SPLIT_K.
+template <int SHAPE_N, int SHAPE_K, int BLOCK_M, int BLOCK_N, int STAGES, int SPLIT_K>
+__global__ void __launch_bounds__((fp8_launch_waves(BLOCK_M, BLOCK_N, STAGES) * kWaveSize))
+fp8_gemm_split_k_kernel(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_scales,
+                        const uint8_t* __restrict__ rhs, const float* __restrict__ rhs_scales,
+                        __bf16* __restrict__ out, int m, int n_rt, int k_rt, int sa_stride_m, int sa_stride_k,
+                        float* __restrict__ partials, unsigned* __restrict__ counters) {
+    fp8_gemm_tile<SHAPE_N, SHAPE_K, BLOCK_M, BLOCK_N, GemmType::Normal, STAGES, SPLIT_K>(
+        lhs, lhs_scales, rhs, rhs_scales, out, m, n_rt, k_rt, sa_stride_m, sa_stride_k, nullptr, 0, int(blockIdx.x), 1, 0,
+        Fp8TwoStages{nullptr, nullptr, nullptr, nullptr}, partials, counters);
+}
+
 // Host side of the kernel, shaped after the class the reference's JIT template instantiates
 // (yan/jit_kernels/gemm.py:20-30: Gemm<N, K, BLOCK_M, BLOCK_N, 128, 1, kNumStages, kNumTMAMulticast, Normal>::run).
 // BLOCK_K is fixed at 128. kNumStages is the number of LDS stages: 2, or a ring of 3 .. Fp8TileConfig::MAX_RING_STAGES
@@ -813,6 +898,41 @@ public:
                            static_cast<const uint8_t*>(rhs), rhs_scales, reinterpret_cast<__bf16*>(out), m, n, k,
                            lhs_scales_stride_m, lhs_scales_stride_k, grouped_layout, lhs_scales_stride_g, int(slots), num_groups,
                            expected_m);
+        return hipGetLastError();
+    }
+
+    // K split SPLIT_K ways over as many workgroups per tile (plain GEMM, ring tiles). `workspace` is device memory of at
+    // least split_k_workspace_bytes<SPLIT_K>(m, n) bytes: kSplitKCounterBytes of arrival counters, which must be zero before
+    // the first launch that uses the workspace and are zero again after every launch, then the partial sums. Launches of
+    // any shapes may share a workspace one after the other; launches that share one must not overlap.
+    template <int SPLIT_K>
+    static size_t split_k_workspace_bytes(int m, int n) {
+        const XcdTileScheduler<> sched(m, n, BLOCK_M, BLOCK_N);
+        return kSplitKCounterBytes + size_t(sched.grid_size()) * SPLIT_K * BLOCK_M * BLOCK_N * 4;
+    }
+    template <int SPLIT_K>
+    static hipError_t run_split_k(__hip_bfloat16* out, const void* lhs, const float* lhs_scales, int lhs_scales_stride_m,
+                                  int lhs_scales_stride_k, const void* rhs, const float* rhs_scales, int m, int n, int k,
+                                  hipStream_t stream, void* workspace, size_t workspace_bytes) {
+        static_assert(kGemmType == GemmType::Normal && SPLIT_K > 1);
+        if (m == 0 || n == 0) return hipSuccess;
+        if (m < 0 || n < 0 || k <= 0 || (n % 4) != 0 || (k % 128) != 0) return hipErrorInvalidValue;
+        if ((SHAPE_N && n != int(SHAPE_N)) || (SHAPE_K && k != int(SHAPE_K))) return hipErrorInvalidValue;
+        if (!out || !lhs || !lhs_scales || !rhs || !rhs_scales || !workspace) return hipErrorInvalidValue;
+        const uint64_t m_pad = uint64_t(ceil_div<uint32_t>(m, BLOCK_M)) * BLOCK_M, n_pad = uint64_t(ceil_div<uint32_t>(n, BLOCK_N)) * BLOCK_N;
+        if (m_pad * k >= kOutOfRange || n_pad * k >= kOutOfRange) return hipErrorInvalidValue;
+        if (uint64_t(BLOCK_M) * n * 2 >= kOutOfRange) return hipErrorInvalidValue;
+        const XcdTileScheduler<> sched(m, n, BLOCK_M, BLOCK_N);
+        // a counter per tile slot and wave; a workgroup per tile slot and part
+        if (uint64_t(sched.grid_size()) * Fp8TileConfig<BLOCK_M, BLOCK_N>::NUM_WAVES * 4 > kSplitKCounterBytes) return hipErrorInvalidValue;
+        if (workspace_bytes < split_k_workspace_bytes<SPLIT_K>(m, n)) return hipErrorInvalidValue;
+        const long long grid = (long long)sched.grid_size() * SPLIT_K;
+        unsigned* counters = static_cast<unsigned*>(workspace);
+        float* partials = reinterpret_cast<float*>(static_cast<uint8_t*>(workspace) + kSplitKCounterBytes);
+        hipLaunchKernelGGL((fp8_gemm_split_k_kernel<SHAPE_N, SHAPE_K, BLOCK_M, BLOCK_N, int(kNumStages), SPLIT_K>), dim3(int(grid)),
+                           dim3(fp8_launch_waves(BLOCK_M, BLOCK_N, int(kNumStages)) * kWaveSize), 0, stream, static_cast<const uint8_t*>(lhs), lhs_scales,
+                           static_cast<const uint8_t*>(rhs), rhs_scales, reinterpret_cast<__bf16*>(out), m, n, k,
+                           lhs_scales_stride_m, lhs_scales_stride_k, partials, counters);
         return hipGetLastError();
     }
 

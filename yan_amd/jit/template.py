@@ -28,6 +28,7 @@ _KINDS: Dict[Any, ArgKind] = {
     int: ArgKind('int', ctypes.c_int, 'int', 'int'),
     float: ArgKind('float', ctypes.c_float, 'float', 'float'),
     torch.int: ArgKind('torch.int', ctypes.c_void_p, 'void*', 'int*'),
+    torch.uint8: ArgKind('torch.uint8', ctypes.c_void_p, 'void*', 'uint8_t*'),      # raw device bytes (workspaces)
     torch.float: ArgKind('torch.float', ctypes.c_void_p, 'void*', 'float*'),
     torch.float16: ArgKind('torch.half', ctypes.c_void_p, 'void*', '__half*'),
     torch.bfloat16: ArgKind('torch.bfloat16', ctypes.c_void_p, 'void*', '__hip_bfloat16*'),

@@ -15,7 +15,8 @@ from typing import Tuple
 
 import torch
 
-from .heuristics import get_best_fp8_config, get_fp8_num_stages, get_fp8_tile_space, get_skinny_fp8_config, tuning_enabled
+from .heuristics import (get_best_fp8_config, get_fp8_num_stages, get_fp8_tile_space, get_skinny_fp8_config,
+                         get_split_k_fp8_config, tuning_enabled)
 from .tuner import FrozenKeys, jit_tuner
 from .utils import get_num_sms, ceil_div, get_col_major_tensor
 
@@ -54,6 +55,16 @@ __return_code = static_cast<int>(launch_fp8_skinny<N, K, BLOCK_M / 16, {NUM_WAVE
     out, lhs, lhs_scales, lhs_scales_stride_m, lhs_scales_stride_k, rhs, rhs_scales, m, N, K, stream));
 """
 
+# K split over SPLIT_K workgroups per tile; the parts meet in `workspace` (Gemm::run_split_k in gemm/fp8_gemm.hpp).
+_split_k_launch = """
+// Make a templated GEMM
+using GemmType = Gemm<N, K, BLOCK_M, BLOCK_N, 128, 1, kNumStages, kNumTMAMulticast, GemmType::Normal>;
+
+// Launch kernel
+__return_code = static_cast<int>(GemmType::run_split_k<{SPLIT_K}>(out, lhs, lhs_scales, lhs_scales_stride_m, lhs_scales_stride_k,
+                                                                  rhs, rhs_scales, m, N, K, stream, workspace, workspace_bytes));
+"""
+
 # The reference's keys and run-time names, nothing else (yan/jit_kernels/gemm.py:9-30): code that formats this template
 # with `N, K, BLOCK_M, BLOCK_N, NUM_STAGES, NUM_TMA_MULTICAST` and builds it with `arg_defs` gets the kernel for
 # token-contiguous activation scales.
@@ -68,11 +79,34 @@ strided_template = _keys_block + _tiled_launch
 strided_arg_defs = arg_defs + (('lhs_scales_stride_m', int), ('lhs_scales_stride_k', int))
 skinny_template = _keys_block + _token_contiguous_scales + _skinny_launch
 skinny_strided_template = _keys_block + _skinny_launch
+# Split-K kernels take their workspace as two more arguments (in front of the strides, when those are passed).
+split_k_template = _keys_block + _token_contiguous_scales + _split_k_launch
+split_k_strided_template = _keys_block + _split_k_launch
+split_k_arg_defs = arg_defs + (('workspace', torch.uint8), ('workspace_bytes', int))
+split_k_strided_arg_defs = split_k_arg_defs + (('lhs_scales_stride_m', int), ('lhs_scales_stride_k', int))
+# kSplitKCounterBytes and kSplitKWorkspaceBytes of gemm/fp8_gemm.hpp: arrival counters, then the partial sums of the
+# largest plan get_split_k_fp8_config makes.
+SPLIT_K_COUNTER_BYTES = 16 * 1024
+SPLIT_K_WORKSPACE_BYTES = SPLIT_K_COUNTER_BYTES + 256 * 128 * 128 * 4
+_split_k_workspaces = {}
+
+
+def split_k_workspace(device: torch.device, stream: torch.cuda.Stream) -> torch.Tensor:
+    """The workspace split-K launches on `stream` share: one per device and stream, made (and zeroed, on the current
+    stream) at the first call and kept. Launches on one stream run one after the other, which is what sharing needs; the
+    counters at its start are zero again after every launch."""
+    key = (device.index, stream.cuda_stream)
+    workspace = _split_k_workspaces.get(key)
+    if workspace is None:
+        workspace = torch.zeros(SPLIT_K_WORKSPACE_BYTES, dtype=torch.uint8, device=device)
+        _split_k_workspaces[key] = workspace
+    return workspace
 
 
 @functools.lru_cache(maxsize=None)
 def fp8_kernel_plan(m: int, n: int, k: int, num_cus: int, token_contiguous_scales: bool = True):
-    """(name, keys, arg_defs, smem_size, template) of the JIT kernel a call with these sizes uses; needs no GPU."""
+    """(name, keys, arg_defs, smem_size, template) of the JIT kernel a call with these sizes uses when K is not split
+    (`fp8_split_k_plan` says when it is); needs no GPU."""
     defs = arg_defs if token_contiguous_scales else strided_arg_defs
     # the tuner memoises per (name, keys): the two argument lists need two names
     name = 'gemm_fp8_fp8_bf16_nt' if token_contiguous_scales else 'gemm_fp8_fp8_bf16_nt_strided'
@@ -87,6 +121,21 @@ def fp8_kernel_plan(m: int, n: int, k: int, num_cus: int, token_contiguous_scale
             'NUM_TMA_MULTICAST': 1})
     smem_size = keys['NUM_STAGES'] * (block_m + block_n) * 128
     return name, keys, defs, smem_size, template if token_contiguous_scales else strided_template
+
+
+@functools.lru_cache(maxsize=None)
+def fp8_split_k_plan(m: int, n: int, k: int, num_cus: int, token_contiguous_scales: bool = True):
+    """(name, keys, arg_defs, template) of the split-K kernel a call with these sizes uses, or None when K is not split
+    (`get_split_k_fp8_config`); needs no GPU."""
+    plan = get_split_k_fp8_config(m, n, k, num_cus)
+    if plan is None:
+        return None
+    block_m, block_n, split_k = plan
+    keys = FrozenKeys({'N': n, 'K': k, 'BLOCK_M': block_m, 'BLOCK_N': block_n, 'NUM_STAGES': get_fp8_num_stages(block_m, block_n),
+                       'NUM_TMA_MULTICAST': 1, 'SPLIT_K': split_k})
+    if token_contiguous_scales:
+        return 'gemm_fp8_fp8_bf16_nt_split_k', keys, split_k_arg_defs, split_k_template
+    return 'gemm_fp8_fp8_bf16_nt_split_k_strided', keys, split_k_strided_arg_defs, split_k_strided_template
 
 
 @functools.lru_cache(maxsize=None)
@@ -135,12 +184,18 @@ def gemm_fp8_fp8_bf16_nt(lhs: Tuple[torch.Tensor, torch.Tensor],
     stride_m, stride_k = lhs_scales.stride()
     token_contiguous = (m == 1 or stride_m == 1) and (lhs_scales.size(1) == 1 or stride_k == m)
     name, keys, defs, smem_size, code_template = fp8_kernel_plan(m, n, k, num_sms, token_contiguous)
+    stream = torch.cuda.current_stream()
+    args = (lhs, lhs_scales, rhs, rhs_scales, out, m, stream, num_sms, smem_size)
     space = ()
     if tuning_enabled():
         tuning = fp8_tuning_plan(m, n, k, num_sms, token_contiguous)
         if tuning is not None:
             name, keys, space, defs, code_template = tuning
-    args = (lhs, lhs_scales, rhs, rhs_scales, out, m, torch.cuda.current_stream(), num_sms, smem_size)
+    else:
+        split = fp8_split_k_plan(m, n, k, num_sms, token_contiguous)
+        if split is not None:
+            name, keys, defs, code_template = split
+            args += (split_k_workspace(out.device, stream), SPLIT_K_WORKSPACE_BYTES)
     if not token_contiguous:
         args += (stride_m, stride_k)
     runtime = jit_tuner.compile_and_tune(name=name, keys=keys, space=space, includes=includes,

@@ -7,7 +7,7 @@ one workgroup per tile, one workgroup per CU at a time, so a launch costs
 `ceil(tiles / num_cus)` rounds of one tile time, and a tile's time grows with its MFMA work but shrinks per
 flop as the tile gets larger (fewer operand bytes fetched per flop).
 """
-from typing import List, Tuple
+from typing import List, Optional, Tuple
 
 from .utils import ceil_div
 
@@ -143,6 +143,52 @@ def get_fp8_tile(m: int, n: int, k: int, num_cus: int) -> Tuple[int, int]:
     """(BLOCK_M, BLOCK_N) of the FP8 kernel that runs: (16 * atoms, 16) for the weight-streaming kernel."""
     atoms = get_skinny_fp8_config(m, n, k, num_cus)
     return (16 * atoms, 16) if atoms else get_best_fp8_config(m, n, k, num_cus)
+
+
+# Split-K of the FP8 GEMM: microseconds a workgroup spends per k-tile on a ring tile when every compute unit runs one
+# (measured: m x 4096 x 7168, sizes at run time, 56 k-tiles, one round of workgroups). Only used to weigh split-K plans
+# against the unsplit pick of the cost table above.
+_FP8_SPLIT_K_TILE_US = {(32, 32): 0.133, (64, 32): 0.192, (64, 64): 0.296, (64, 128): 0.395, (128, 128): 0.51}
+FP8_SPLIT_K_FACTORS = (2, 3, 4)
+
+
+def get_split_k_fp8_config(m: int, n: int, k: int, num_cus: int) -> Optional[Tuple[int, int, int]]:
+    """(BLOCK_M, BLOCK_N, SPLIT_K) when the plain FP8 GEMM should split K over SPLIT_K workgroups per tile, else None.
+
+    A problem whose unsplit tiles fit the chip in one round is bound by what one compute unit can pull per k-tile
+    (60-65 GB/s whatever the tile), and every workgroup pulls the activation rows of its tile over all of K. With K split,
+    a larger tile on as many workgroups pulls fewer bytes per output; the price is a round trip of the partial sums
+    through memory, paid by the part that arrives last. Modelled time of a plan: k-tiles per part x the tile's time per
+    k-tile + 0.5 us + 12.5 ns per KB of partial sums the last part reads, never less than streaming the weights at 6 TB/s.
+    A plan is taken when it fits one round (tile slots x SPLIT_K <= num_cus), leaves every part at least 14 k-tiles and beats
+    the unsplit pick by a tenth of its modelled time plus 3.5 us of launch. On 36 shapes (m = 32..256, n = 1536..24576,
+    k = 1536..16384) swept with every tile and factor, weights cycling through more matrices than the caches hold, the
+    plan taken is the fastest measured or within 1 % of it wherever one is taken: 13 to 38 % faster than unsplit
+    (64 x 4096 x 7168: 64 x 64 tiles in four parts; 32 x 2112 x 7168: 32 x 32 in three); k = 2048 and n = 16384 or more
+    stay unsplit. Same rule as `pick_split_k` in yan_amd/csrc/yan_gemm_capi.hip (a CPU test keeps the two in step)."""
+    if get_skinny_fp8_config(m, n, k, num_cus) or m <= 0 or n <= 0:
+        return None
+    k_tiles = k // 128
+    unsplit = get_best_fp8_config(m, n, k, num_cus)
+    if unsplit not in _FP8_SPLIT_K_TILE_US or ceil_div(m, unsplit[0]) * ceil_div(n, unsplit[1]) > num_cus:
+        return None
+    floor = n * k / 6.0e6
+    base = max(k_tiles * _FP8_SPLIT_K_TILE_US[unsplit], floor)
+    best, best_plan = None, None
+    for (bm, bn), per_k_tile in _FP8_SPLIT_K_TILE_US.items():
+        if bm > 32 and bm >= 2 * m:
+            continue                # a tile more than twice as tall as the problem
+        tiles = ceil_div(m, bm) * ceil_div(n, bn)
+        for split in FP8_SPLIT_K_FACTORS:
+            # a workgroup per part of every tile slot (tiles rounded up to the 8 XCDs); 256 also bounds the workspace
+            if ceil_div(tiles, 8) * 8 * split > min(num_cus, 256) or ceil_div(k_tiles, split) < 14:
+                continue
+            t = max(ceil_div(k_tiles, split) * per_k_tile + 0.5 + (split * bm * bn * 4) / 1024 * 0.0125, floor)
+            if best is None or t < best:
+                best, best_plan = t, (bm, bn, split)
+    if best is not None and base - best >= 0.10 * (base + 3.5):
+        return best_plan
+    return None
 
 
 # (BLOCK_M, BLOCK_N) -> cost per unit of tile area; tiles below 128 rows split K over their four waves.
