@@ -93,6 +93,18 @@ YAN_API int yan_gemm_fp8_fp8_bf16_nt_split_k(const void* lhs, const float* lhs_s
                                      int m, int n, int k, void* stream, int num_sms, void* workspace,
                                      long long workspace_bytes);
 
+/* The split-K GEMM above for callers that cannot allocate or own a workspace (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc): the workspace is a device array inside the library, 16.0 MB
+ * (yan_gemm_fp8_split_k_workspace_bytes()) on every GPU the library runs on, held until the process ends; the call
+ * allocates nothing and frees nothing. Same arguments, same plans and same bits as yan_gemm_fp8_fp8_bf16_nt_split_k. A problem
+ * whose plan needed more than the array holds would return hipErrorInvalidValue without launching (no plan for up to 256
+ * compute units does). Every call on a GPU uses that GPU's one array, on whatever stream or host thread: calls that
+ * overlap on the device race; calls on one stream, or otherwise ordered, are safe, and each leaves the counters at zero.
+ * It has no counterpart in the reference. */
+YAN_API int yan_gemm_fp8_fp8_bf16_nt_static(const void* lhs, const float* lhs_scales, long long lhs_scales_stride_m,
+                                    long long lhs_scales_stride_k, const void* rhs, const float* rhs_scales, void* out,
+                                    int m, int n, int k, void* stream, int num_sms);
+
 /* Grouped (mixture-of-experts) forms of the FP8 GEMM: group g has its own weights rhs[g] ([n,k] e4m3) and scale table
  * rhs_scales[g] ([ceil(n/128)][k/128]); both arrays are contiguous over g. Arithmetic per row as above.
  * They fill in the reference's GemmType::GroupedContiguous / GroupedMasked and `int* grouped_layout` hooks

@@ -10,7 +10,7 @@ _lib = None
 
 SYMBOLS = ('yan_gemm_bf16_tn', 'yan_gemm_fp16_tn', 'yan_gemm_float_nt', 'yan_gemm_fp8_fp8_bf16_nt', 'yan_m_grouped_gemm_fp8_fp8_bf16_nt_contiguous',
            'yan_m_grouped_gemm_fp8_fp8_bf16_nt_masked', 'yan_per_token_cast_to_fp8', 'yan_per_block_cast_to_fp8',
-           'yan_gemm_select_tile', 'yan_gemm_fp8_fp8_bf16_nt_split_k', 'yan_gemm_select_split_k',
+           'yan_gemm_select_tile', 'yan_gemm_fp8_fp8_bf16_nt_split_k', 'yan_gemm_fp8_fp8_bf16_nt_static', 'yan_gemm_select_split_k',
            'yan_gemm_fp8_split_k_workspace_bytes', 'yan_gemm_fp8_split_k_counter_bytes', 'yan_gemm_version')
 
 
@@ -23,7 +23,7 @@ def load() -> ctypes.CDLL:
         vp, ci, ll = ctypes.c_void_p, ctypes.c_int, ctypes.c_longlong
         lib.yan_gemm_bf16_tn.argtypes = lib.yan_gemm_fp16_tn.argtypes = [ci, ci, ci, vp, vp, vp, vp]
         lib.yan_gemm_float_nt.argtypes = [ci, ci, ci, ctypes.c_float, vp, ci, vp, ci, ctypes.c_float, vp, ci, vp]
-        lib.yan_gemm_fp8_fp8_bf16_nt.argtypes = [vp, vp, ll, ll, vp, vp, vp, ci, ci, ci, vp, ci]
+        lib.yan_gemm_fp8_fp8_bf16_nt.argtypes = lib.yan_gemm_fp8_fp8_bf16_nt_static.argtypes = [vp, vp, ll, ll, vp, vp, vp, ci, ci, ci, vp, ci]
         lib.yan_gemm_select_tile.argtypes = [ci, ci, ci, ci, ci, ctypes.POINTER(ci), ctypes.POINTER(ci)]
         lib.yan_m_grouped_gemm_fp8_fp8_bf16_nt_contiguous.argtypes = [vp, vp, ll, ll, vp, vp, vp, vp, ci, ci, ci, ci, vp, ci]
         lib.yan_m_grouped_gemm_fp8_fp8_bf16_nt_masked.argtypes = [vp, vp, ll, ll, ll, vp, vp, vp, vp, ci, ci, ci, ci, ci, vp, ci]
@@ -81,6 +81,14 @@ def gemm_fp8_fp8_bf16_nt_split_k(lhs, rhs, out: torch.Tensor, workspace: torch.T
     return load().yan_gemm_fp8_fp8_bf16_nt_split_k(a8.data_ptr(), sa.data_ptr(), sa.stride(0), sa.stride(1), b8.data_ptr(),
                                                    sb.data_ptr(), out.data_ptr(), m, n, k, _stream_handle(), num_sms,
                                                    workspace.data_ptr(), workspace.numel() * workspace.element_size())
+
+
+def gemm_fp8_fp8_bf16_nt_static(lhs, rhs, out: torch.Tensor, num_sms: int = 0) -> int:
+    """The split-K GEMM on the library's own device array: nothing is allocated."""
+    (a8, sa), (b8, sb) = lhs, rhs
+    (m, k), n = a8.shape, b8.shape[0]
+    return load().yan_gemm_fp8_fp8_bf16_nt_static(a8.data_ptr(), sa.data_ptr(), sa.stride(0), sa.stride(1), b8.data_ptr(),
+                                                  sb.data_ptr(), out.data_ptr(), m, n, k, _stream_handle(), num_sms)
 
 
 def select_split_k(m: int, n: int, k: int, num_cus: int):

@@ -11,6 +11,11 @@
 
 #include <mutex>
 
+// Scratch of the entry point that allocates nothing (yan_gemm_fp8_fp8_bf16_nt_static): the split-K workspace as a device
+// array. Every GPU the library runs on holds its own copy, zero when the module is loaded, until the process ends; host
+// code reaches a GPU's copy through the address hipGetSymbolAddress returns with that GPU current, never through the name.
+static __device__ __align__(256) unsigned char scratch[yan::kSplitKWorkspaceBytes];
+
 namespace {
 
 struct TileCost { int bm, bn; double per_area; };
@@ -126,6 +131,21 @@ int dense(int m, int n, int k, const void* a, const void* b, void* c, void* stre
     return int(hipErrorInvalidValue);
 }
 
+void* static_scratch() {
+    constexpr int kMaxDevices = 64;
+    static std::mutex guard;
+    static void* address[kMaxDevices] = {};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
+    std::lock_guard<std::mutex> lock(guard);
+    if (!address[dev]) {
+        void* ptr = nullptr;
+        if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess) return nullptr;
+        address[dev] = ptr;
+    }
+    return address[dev];
+}
+
 // The plain FP8 GEMM. With a workspace, problems the split-K plan covers run split (a workspace too small for the plan is
 // an error); without one, and for every other problem, a workgroup per tile as before.
 int fp8_plain(const void* lhs, const float* lhs_scales, long long lhs_scales_stride_m, long long lhs_scales_stride_k,
@@ -198,6 +218,17 @@ int yan_gemm_fp8_fp8_bf16_nt_split_k(const void* lhs, const float* lhs_scales, l
     if (!workspace || workspace_bytes < 0) return int(hipErrorInvalidValue);
     return fp8_plain(lhs, lhs_scales, lhs_scales_stride_m, lhs_scales_stride_k, rhs, rhs_scales, out, m, n, k, stream, num_sms,
                      workspace, size_t(workspace_bytes));
+}
+
+// Same as yan_gemm_fp8_fp8_bf16_nt_split_k with the device array `scratch` for a workspace: no allocation anywhere on the
+// way. Calls on one GPU share that GPU's array: they must not overlap on the device.
+int yan_gemm_fp8_fp8_bf16_nt_static(const void* lhs, const float* lhs_scales, long long lhs_scales_stride_m,
+                                    long long lhs_scales_stride_k, const void* rhs, const float* rhs_scales, void* out,
+                                    int m, int n, int k, void* stream, int num_sms) {
+    void* workspace = static_scratch();
+    if (!workspace) return int(hipErrorInvalidValue);
+    return fp8_plain(lhs, lhs_scales, lhs_scales_stride_m, lhs_scales_stride_k, rhs, rhs_scales, out, m, n, k, stream, num_sms,
+                     workspace, yan::kSplitKWorkspaceBytes);
 }
 
 int yan_m_grouped_gemm_fp8_fp8_bf16_nt_contiguous(const void* lhs, const float* lhs_scales, long long lhs_scales_stride_m,
