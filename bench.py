@@ -290,9 +290,29 @@ def main():
         t_cold = yan.bench_kineto(decode, 'fp8_gemm', suppress_kineto_output=True, flush_l2=True)
         d = _sampled_fp8_diff(yan, harness, x8, sx, w8, sw, o)
         assert d < 1e-3, f'decode parity lost: calc_diff={d}'
+        # The Python entry spends longer on the host than the kernel on the device, so the launches above start on an idle
+        # GPU, which costs a kernel this short about 1 us. The same JIT kernels launched through their `launch` symbol with
+        # prepared arguments (3 us of host work per call, the launches queue up): the split-K plan the entry uses and the
+        # unsplit kernel it would use without one.
+        from yan_amd import jit
+        from yan_amd.jit_kernels import gemm as fp8_entry
+        stream, cus = torch.cuda.current_stream(), yan.get_num_sms()
+        name, keys, defs, smem, tmpl = fp8_entry.fp8_kernel_plan(mm, nn, kk, cus, True)
+        unsplit = jit.build(name, defs, jit.generate(fp8_entry.includes, defs, jit.cpp_format(tmpl, keys)))
+        t_unsplit = yan.bench_kineto(lambda: unsplit(x8, sx, w8, sw, o, mm, stream, cus, smem), 'fp8_gemm', suppress_kineto_output=True)
+        plan, t_split = fp8_entry.fp8_split_k_plan(mm, nn, kk, cus, True), None
+        if plan is not None:
+            name, keys, defs, tmpl = plan
+            split = jit.build(name, defs, jit.generate(fp8_entry.includes, defs, jit.cpp_format(tmpl, keys)))
+            workspace = fp8_entry.split_k_workspace(o.device, stream)
+            t_split = yan.bench_kineto(lambda: split(x8, sx, w8, sw, o, mm, stream, cus, smem, workspace, fp8_entry.SPLIT_K_WORKSPACE_BYTES),
+                                       'fp8_gemm', suppress_kineto_output=True)
         byt = _fp8_bytes(mm, nn, kk)
         extra['fp8_decode_64x4096x7168'] = {'kernel_us_warm': round(t_warm * 1e6, 2), 'kernel_us_cold': round(t_cold * 1e6, 2),
                                             'call_to_call_us': round(wall * 1e3, 2), 'algorithmic_bytes': byt,
+                                            'kernel_us_warm_queued_launches': round(t_split * 1e6, 2) if t_split else None,
+                                            'kernel_us_warm_queued_launches_unsplit': round(t_unsplit * 1e6, 2),
+                                            'split_k_plan': [plan[1][key] for key in ('BLOCK_M', 'BLOCK_N', 'SPLIT_K')] if plan else None,
                                             'gb_per_s_warm': round(byt / t_warm / 1e9, 1), 'gb_per_s_cold': round(byt / t_cold / 1e9, 1),
                                             'frac_of_hbm_peak_warm': round(byt / t_warm / 1e9 / PEAK_HBM_GBPS, 4),
                                             'frac_of_hbm_peak_cold': round(byt / t_cold / 1e9 / PEAK_HBM_GBPS, 4),

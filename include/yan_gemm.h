@@ -42,6 +42,18 @@ YAN_API int yan_gemm_bf16_tn(int m, int n, int k, const void* a, const void* b, 
 /* Same contraction for IEEE fp16 in / fp16 out, fp32 accumulate (the reference's dtype, cute_gemm.py:26). */
 YAN_API int yan_gemm_fp16_tn(int m, int n, int k, const void* a, const void* b, void* c, void* stream);
 
+/* The two dense GEMMs with K split over 2 to 4 workgroups per output tile where that pays: problems whose tiles would leave
+ * compute units idle and whose K is long (the smallest dense tile holds 64 weight rows, so 64 x 4096 x 7168 runs on 64
+ * workgroups; in four parts it runs on 256 and takes 16 us instead of 37). The parts leave fp32 partial sums in `workspace`;
+ * the part that arrives last adds them up in the order of their K ranges (results are repeatable to the bit) and stores the
+ * tile. Within the tolerance of the plain entry points, not bit-identical to them; every other problem runs exactly as
+ * through the plain entry points. `workspace` / `workspace_bytes`: as for yan_gemm_fp8_fp8_bf16_nt_split_k below (one
+ * workspace serves all three). The reference's dense launcher has no split (yan/include/gemm/cute_gemm.cuh:262-378). */
+YAN_API int yan_gemm_bf16_tn_split_k(int m, int n, int k, const void* a, const void* b, void* c, void* stream, void* workspace,
+                             long long workspace_bytes);
+YAN_API int yan_gemm_fp16_tn_split_k(int m, int n, int k, const void* a, const void* b, void* c, void* stream, void* workspace,
+                             long long workspace_bytes);
+
 /* c = alpha * a . b^T + beta * c in fp32 (fp32 MFMA accumulation).
  *   a  m x k with M contiguous: element (i, kk) at a[i + kk*lda];   b  n x k with N contiguous: b[j + kk*ldb];
  *   c  m x n row-major: c[i*ldc + j].  beta == 0 does not read c.
@@ -79,15 +91,15 @@ YAN_API int yan_gemm_fp8_fp8_bf16_nt(const void* lhs, const float* lhs_scales, l
  * their K ranges, so a result does not depend on which part that was, and stores the tile. Results are within the
  * tolerance of the plain entry point but not bit-identical to it (a different order of summation); every other problem
  * runs exactly as through the plain entry point.
- *   workspace        device memory of at least yan_gemm_fp8_split_k_workspace_bytes() bytes (16.0 MB), whose first
- *                    yan_gemm_fp8_split_k_counter_bytes() bytes (arrival counters) the caller zero-fills once, before the
+ *   workspace        device memory of at least yan_gemm_split_k_workspace_bytes() bytes (16.0 MB), whose first
+ *                    yan_gemm_split_k_counter_bytes() bytes (arrival counters) the caller zero-fills once, before the
  *                    first call; every call leaves them zero again, so one workspace serves calls of any shapes;
  *   workspace_bytes  its size; less than the problem's plan needs is hipErrorInvalidValue.
  * Calls that share a workspace must not overlap on the device (same stream, or otherwise ordered).
  * This is the `split` half of the reference's tile/split heuristics, which its template leaves to the caller's keys
  * (yan/jit_kernels/gemm.py:13-18); yan_gemm_select_split_k below says what a problem gets. */
-YAN_API long long yan_gemm_fp8_split_k_workspace_bytes(void);
-YAN_API long long yan_gemm_fp8_split_k_counter_bytes(void);
+YAN_API long long yan_gemm_split_k_workspace_bytes(void);
+YAN_API long long yan_gemm_split_k_counter_bytes(void);
 YAN_API int yan_gemm_fp8_fp8_bf16_nt_split_k(const void* lhs, const float* lhs_scales, long long lhs_scales_stride_m,
                                      long long lhs_scales_stride_k, const void* rhs, const float* rhs_scales, void* out,
                                      int m, int n, int k, void* stream, int num_sms, void* workspace,
@@ -95,7 +107,7 @@ YAN_API int yan_gemm_fp8_fp8_bf16_nt_split_k(const void* lhs, const float* lhs_s
 
 /* The split-K GEMM above for callers that cannot allocate or own a workspace (code under HIP graph capture, tight serving
  * loops, harnesses that forbid hipMalloc): the workspace is a device array inside the library, 16.0 MB
- * (yan_gemm_fp8_split_k_workspace_bytes()) on every GPU the library runs on, held until the process ends; the call
+ * (yan_gemm_split_k_workspace_bytes()) on every GPU the library runs on, held until the process ends; the call
  * allocates nothing and frees nothing. Same arguments, same plans and same bits as yan_gemm_fp8_fp8_bf16_nt_split_k. A problem
  * whose plan needed more than the array holds would return hipErrorInvalidValue without launching (no plan for up to 256
  * compute units does). Every call on a GPU uses that GPU's one array, on whatever stream or host thread: calls that
@@ -148,10 +160,10 @@ YAN_API int yan_per_block_cast_to_fp8(const void* w, int w_is_fp32, void* q, flo
  * (yan/jit_kernels/cute_gemm.py:41, yan/jit_kernels/gemm.py:13-16). Returns 0, or 1 for an unknown op. */
 YAN_API int yan_gemm_select_tile(int op, int m, int n, int k, int num_cus, int* block_m, int* block_n);
 
-/* Split-K plan of the plain FP8 GEMM on `num_cus` compute units: writes the tile and the number of parts, or
- * block_m = block_n = 0 and split_k = 1 when K is not split (then yan_gemm_select_tile names the tile). Host-only.
- * Returns 0, or 1 for a null pointer or num_cus <= 0. */
-YAN_API int yan_gemm_select_split_k(int m, int n, int k, int num_cus, int* block_m, int* block_n, int* split_k);
+/* Split-K plan of the dense 16-bit GEMM (op 0) or the plain FP8 GEMM (op 1) on `num_cus` compute units: writes the tile
+ * and the number of parts, or block_m = block_n = 0 and split_k = 1 when K is not split (then yan_gemm_select_tile names
+ * the tile). Host-only. Returns 0, or 1 for another op, a null pointer or num_cus <= 0. */
+YAN_API int yan_gemm_select_split_k(int op, int m, int n, int k, int num_cus, int* block_m, int* block_n, int* split_k);
 
 /* "yan-gemm gfx950 <n> dense + <n> fp32 + <n> fp8 tile variants + <n> weight-streaming fp8 variant + ...". */
 YAN_API const char* yan_gemm_version(void);

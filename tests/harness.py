@@ -212,6 +212,15 @@ FP8_SPLIT_K_PLAN_OF_SHAPE = {
     (64, 4096, 7168): (64, 64, 4), (128, 4096, 7168): (64, 128, 4),
 }
 FP8_SPLIT_K_SHAPES = [s for s in FP8_SPLIT_K_PLAN_OF_SHAPE if s not in ((64, 4096, 7168), (128, 4096, 7168))]
+# The same for the dense GEMMs: the three tiles split-K plans use, every factor, ragged m and n, n that is no multiple of 8,
+# a k tail (3080 = 48 k-tiles and 8 elements).
+DENSE_SPLIT_K_PLAN_OF_SHAPE = {
+    (33, 196, 2048): (64, 64, 2), (100, 196, 3080): (64, 64, 3), (65, 196, 4096): (64, 64, 4),
+    (129, 4100, 5632): (64, 128, 2), (200, 2112, 3072): (64, 128, 3), (129, 2112, 5120): (64, 128, 4),
+    (300, 4100, 4096): (128, 128, 2), (200, 4100, 3080): (128, 128, 3), (200, 3076, 5120): (128, 128, 4),
+    (64, 4096, 7168): (64, 64, 4), (256, 2048, 7168): (64, 128, 4),
+}
+DENSE_SPLIT_K_SHAPES = list(DENSE_SPLIT_K_PLAN_OF_SHAPE)
 # Grouped FP8 GEMMs: (rows per group, n, k, blocks of padding rows) and (groups, m_max, n, k, masked_m, expected_m).
 # Long groups on 256-row tiles whose two 128-row halves belong to different groups, or one of them to padding: a padding
 # block between the groups (negative entry) and one at the end; group 1 has 63 blocks, so it starts and the run ends on
@@ -288,11 +297,15 @@ def jit_kernels_in_use(num_cus: int = 256):
         kernels.setdefault((name, code), (name, arg_defs, code))
 
     # the last four: shapes only the benchmark's --also legs run
-    for m, n, k in DENSE_TEST_SHAPES + REFERENCE_DENSE_TEST_SHAPES + [(256, 512, 512), (4096, 5120, 5120), (2048, 7168, 7168), (4096, 7168, 16384), (8192, 8192, 9216)]:
+    for m, n, k in DENSE_TEST_SHAPES + REFERENCE_DENSE_TEST_SHAPES + DENSE_SPLIT_K_SHAPES + [(256, 512, 512), (4096, 5120, 5120), (2048, 7168, 7168), (4096, 7168, 16384), (8192, 8192, 9216)]:
         for dtype in (torch.bfloat16, torch.half):
             if m and n:
                 name, keys, arg_defs = bf16_gemm.dense_kernel_plan(m, n, k, dtype, num_cus)
                 add(name, arg_defs, bf16_gemm.includes, bf16_gemm.template, keys)
+                split = bf16_gemm.dense_split_k_plan(m, n, k, dtype, num_cus)
+                if split is not None:
+                    name, keys, arg_defs = split
+                    add(name, arg_defs, bf16_gemm.includes, bf16_gemm.split_k_template, keys)
     for m, n, k in REFERENCE_FLOAT_TEST_SHAPES + FLOAT_TEST_SHAPES + [(5120, 2048, 4096)]:
         name, keys, arg_defs = simple_gemm.float_kernel_plan(m, n, num_cus)
         add(name, arg_defs, simple_gemm.includes, simple_gemm.template, keys)

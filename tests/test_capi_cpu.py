@@ -24,7 +24,7 @@ def _declared(repo_root):
 
 def test_library_exports_every_declared_symbol(lib, repo_root):
     declared = _declared(repo_root)
-    assert declared == sorted(capi.SYMBOLS) and len(declared) == 15
+    assert declared == sorted(capi.SYMBOLS) and len(declared) == 17
     for name in declared:
         assert hasattr(lib, name), name
     out = subprocess.check_output(['nm', '-D', '--defined-only', os.path.join(repo_root, 'yan_amd', 'csrc', 'libyan_gemm.so')], text=True)
@@ -63,12 +63,15 @@ def test_version_and_tile_selection_match_python(lib):
                 for cus in (256, 64, 40, 8):
                     plan = capi.select_split_k(m, n, k, cus)
                     assert plan == heuristics.get_split_k_fp8_config(m, n, k, cus), (m, n, k, cus)
-                    plans += plan is not None
-    assert plans > 500
-    assert lib.yan_gemm_fp8_split_k_workspace_bytes() == yan.gemm.SPLIT_K_WORKSPACE_BYTES == 16 * 1024 + 256 * 128 * 128 * 4
-    assert lib.yan_gemm_fp8_split_k_counter_bytes() == yan.gemm.SPLIT_K_COUNTER_BYTES
+                    dense_plan = capi.select_split_k(m, n, k, cus, op=0)
+                    assert dense_plan == heuristics.get_split_k_dense_config(m, n, k, cus), (m, n, k, cus)
+                    plans += (plan is not None) + (dense_plan is not None)
+    assert plans > 1000
+    assert lib.yan_gemm_split_k_workspace_bytes() == yan.gemm.SPLIT_K_WORKSPACE_BYTES == 16 * 1024 + 256 * 128 * 128 * 4
+    assert lib.yan_gemm_split_k_counter_bytes() == yan.gemm.SPLIT_K_COUNTER_BYTES
     bm, bn = ctypes.c_int(), ctypes.c_int()
-    assert lib.yan_gemm_select_split_k(64, 4096, 7168, 0, ctypes.byref(bm), ctypes.byref(bn), ctypes.byref(bm)) == 1
+    assert lib.yan_gemm_select_split_k(1, 64, 4096, 7168, 0, ctypes.byref(bm), ctypes.byref(bn), ctypes.byref(bm)) == 1
+    assert lib.yan_gemm_select_split_k(2, 64, 4096, 7168, 256, ctypes.byref(bm), ctypes.byref(bn), ctypes.byref(bm)) == 1
     assert lib.yan_gemm_select_tile(7, 1, 1, 1, 256, ctypes.byref(bm), ctypes.byref(bn)) == 1
     assert lib.yan_gemm_select_tile(0, 1, 1, 1, 0, ctypes.byref(bm), ctypes.byref(bn)) == 1
 

@@ -146,6 +146,34 @@ def test_dense_weight_streaming_kernel_leaves_its_neighbours_alone(m, n, k):
     assert torch.equal(again, big[:m])
 
 
+@pytest.mark.parametrize('m,n,k', testing.DENSE_SPLIT_K_SHAPES)
+@pytest.mark.parametrize('dtype', [torch.bfloat16, torch.half])
+def test_dense_split_k_parity_vs_oracle(m, n, k, dtype):
+    """Problems whose K the dense entry points split over 2 to 4 workgroups per tile (the three tiles, every factor, ragged
+    edges, a k tail): parity against the oracle to the bar of the unsplit kernels, the same bits from the library's split-K
+    entry point, which writes nothing past row m, and arrival counters back at zero."""
+    from yan_amd.jit_kernels import bf16_gemm
+    plan = bf16_gemm.dense_split_k_plan(m, n, k, dtype, yan.get_num_sms())
+    assert plan is not None and (plan[1]['BLOCK_M'], plan[1]['BLOCK_N'], plan[1]['SPLIT_K']) == testing.DENSE_SPLIT_K_PLAN_OF_SHAPE[(m, n, k)]
+    _announce('dense split-k', dtype, m, n, k, plan[1]['BLOCK_M'], plan[1]['BLOCK_N'], plan[1]['SPLIT_K'])
+    a, b, c = testing.make_bf16_case(m, n, k, seed=42, device='cuda', dtype=dtype)
+    c.fill_(float('nan'))
+    (yan.gemm_bf16_tn if dtype == torch.bfloat16 else yan.gemm_fp16_tn)(a, b, c)
+    torch.cuda.synchronize()
+    got, ref = _np(c), oracle.gemm_bf16_tn_ref(_np(a), _np(b))
+    assert np.isfinite(got).all()
+    assert oracle.calc_diff(got, ref) < BF16_TOL
+    ulp = 2.0 ** (-7 if dtype == torch.bfloat16 else -10)
+    assert bool(np.all(np.abs(got - ref) <= np.abs(ref) * ulp + 1e-4 * np.sqrt(k)))
+    workspace = capi.split_k_workspace()
+    padded = torch.full((m + 3, n), 7.0, dtype=dtype, device='cuda')
+    assert capi.gemm_bf16_tn_split_k(a, b, padded, workspace) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(padded[:m], c) and bool((padded[m:] == 7.0).all())
+    counters = capi.load().yan_gemm_split_k_counter_bytes()
+    assert int(workspace[:counters].view(torch.int32).abs().sum()) == 0
+
+
 def test_dense_baseline_8192_cubed():
     """cfg2: rows sampled against the oracle, the whole matrix against a chunked fp32 matmul on the device."""
     m = n = k = 8192
@@ -498,7 +526,7 @@ def test_split_k_parity_vs_oracle(m, n, k, col_major):
     assert capi.gemm_fp8_fp8_bf16_nt_split_k((a8, sa), (b8, sb), padded, workspace) == 0
     torch.cuda.synchronize()
     assert torch.equal(padded[:m], out) and bool((padded[m:] == 7.0).all())
-    counters = capi.load().yan_gemm_fp8_split_k_counter_bytes()
+    counters = capi.load().yan_gemm_split_k_counter_bytes()
     assert int(workspace[:counters].view(torch.int32).abs().sum()) == 0
 
 
@@ -508,21 +536,34 @@ def test_split_k_launches_of_different_shapes_share_a_workspace():
     part that arrives last adds the parts up in the order of their K ranges, whichever it is)."""
     shapes = [(64, 4096, 7168), (33, 2112, 5376), (300, 4100, 4608), (129, 2112, 7168), (17, 196, 3584)]
     cases = [testing.make_fp8_case(*shape, seed=5 + i, device='cuda', gen_device='cuda') for i, shape in enumerate(shapes)]
-    firsts = []
+    dense_shapes = [(64, 4096, 7168), (200, 4100, 3080), (129, 2112, 5120)]        # the dense split-K kernels share it too
+    dense_cases = [testing.make_bf16_case(*shape, seed=15 + i, scale=shape[2] ** -0.5, device='cuda', gen_device='cuda') for i, shape in enumerate(dense_shapes)]
+    firsts, dense_firsts = [], []
     for (lhs, rhs, out) in cases:
         yan.gemm_fp8_fp8_bf16_nt(lhs, rhs, out)
         firsts.append(out.clone())
+    for (a, b, c) in dense_cases:
+        yan.gemm_bf16_tn(a, b, c)
+        dense_firsts.append(c.clone())
     for ((a8, sa), (b8, sb), out), first in zip(cases, firsts):
         assert float(yan.calc_diff(first.float(), testing.dequant_lhs(a8, sa) @ testing.dequant_rhs(b8, sb).t())) < 1e-5
+    for (a, b, c), first in zip(dense_cases, dense_firsts):
+        assert float(yan.calc_diff(first.float(), a.float() @ b.float().t())) < 1e-5
     flush = torch.empty(512 << 18, dtype=torch.int, device='cuda')
     for it in range(12):
         if it % 3 == 0:
             flush.zero_()
-        for (lhs, rhs, out) in cases:
+        for i, (lhs, rhs, out) in enumerate(cases):
             out.fill_(float('nan'))
             yan.gemm_fp8_fp8_bf16_nt(lhs, rhs, out)
+            if i < len(dense_cases):
+                a, b, c = dense_cases[i]
+                c.fill_(float('nan'))
+                yan.gemm_bf16_tn(a, b, c)
         for (_, _, out), first in zip(cases, firsts):
             assert torch.equal(out, first), it
+        for (_, _, c), first in zip(dense_cases, dense_firsts):
+            assert torch.equal(c, first), it
 
 
 def test_split_k_entry_point_checks_its_workspace():

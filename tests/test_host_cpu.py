@@ -87,6 +87,37 @@ def test_split_k_plans():
     assert gemm.fp8_split_k_plan(4096, 7168, 7168, 256) is None
 
 
+def test_dense_split_k_plans():
+    """The dense GEMMs split K by the same rule with their own tile numbers: plans fit one round and the workspace, leave each
+    part 16 k-tiles or more, and the shapes of the GPU suite get the plans the suite expects."""
+    import harness
+    plan = heuristics.get_split_k_dense_config
+    assert plan(64, 4096, 7168, 256) == (64, 64, 4) and plan(256, 7168, 16384, 256) == (128, 128, 2)
+    assert plan(256, 7168, 2048, 256) is None and plan(256, 24576, 1536, 256) is None and plan(8192, 8192, 8192, 256) is None
+    assert plan(16, 4096, 7168, 256) is None and plan(32, 4096, 7168, 256) is None          # the weight-streaming kernel's
+    for shape, expected in harness.DENSE_SPLIT_K_PLAN_OF_SHAPE.items():
+        assert plan(*shape, 256) == expected, shape
+    assert {(bm, bn) for bm, bn, _ in harness.DENSE_SPLIT_K_PLAN_OF_SHAPE.values()} == set(heuristics._DENSE_SPLIT_K_EXTRA_US)
+    assert {s for _, _, s in harness.DENSE_SPLIT_K_PLAN_OF_SHAPE.values()} == set(heuristics.DENSE_SPLIT_K_FACTORS)
+    assert set(heuristics._DENSE_SPLIT_K_TILE_US) == {t for t in heuristics._DENSE_TILES if heuristics.get_dense_num_stages(*t) > 2}
+    for m in (33, 64, 100, 129, 256, 300, 512, 1024):
+        for n in (196, 1536, 2112, 4096, 4100, 7168, 24576):
+            for k in (1536, 2048, 3080, 4608, 7168, 16384):
+                for cus in (256, 64, 8):
+                    p = plan(m, n, k, cus)
+                    if p is None:
+                        continue
+                    bm, bn, split = p
+                    slots = yan.ceil_div(yan.ceil_div(m, bm) * yan.ceil_div(n, bn), 8) * 8
+                    assert slots * split <= cus and yan.ceil_div(yan.ceil_div(k, 64), split) >= 16
+                    assert gemm.SPLIT_K_COUNTER_BYTES + slots * split * bm * bn * 4 <= gemm.SPLIT_K_WORKSPACE_BYTES
+                    assert slots * 4 * 4 <= gemm.SPLIT_K_COUNTER_BYTES
+    name, keys, defs = bf16_gemm.dense_split_k_plan(64, 4096, 7168, torch.half, 256)
+    assert name == 'gemm_fp16_tn_split_k' and keys['SPLIT_K'] == 4 and defs[-2:] == (('workspace', torch.uint8), ('workspace_bytes', int))
+    assert 'gemm_tn_split_k<BLOCK_M, BLOCK_N, kNumStages, kSplitK>' in bf16_gemm.split_k_template
+    assert bf16_gemm.dense_split_k_plan(8192, 8192, 8192, torch.bfloat16, 256) is None
+
+
 def test_fp8_shapes_of_the_gpu_suite_reach_every_tile_of_the_cost_table():
     import harness
     for shape, tile in harness.FP8_TILE_OF_SHAPE.items():

@@ -10,8 +10,8 @@ _lib = None
 
 SYMBOLS = ('yan_gemm_bf16_tn', 'yan_gemm_fp16_tn', 'yan_gemm_float_nt', 'yan_gemm_fp8_fp8_bf16_nt', 'yan_m_grouped_gemm_fp8_fp8_bf16_nt_contiguous',
            'yan_m_grouped_gemm_fp8_fp8_bf16_nt_masked', 'yan_per_token_cast_to_fp8', 'yan_per_block_cast_to_fp8',
-           'yan_gemm_select_tile', 'yan_gemm_fp8_fp8_bf16_nt_split_k', 'yan_gemm_fp8_fp8_bf16_nt_static', 'yan_gemm_select_split_k',
-           'yan_gemm_fp8_split_k_workspace_bytes', 'yan_gemm_fp8_split_k_counter_bytes', 'yan_gemm_version')
+           'yan_gemm_select_tile', 'yan_gemm_fp8_fp8_bf16_nt_split_k', 'yan_gemm_fp8_fp8_bf16_nt_static', 'yan_gemm_bf16_tn_split_k', 'yan_gemm_fp16_tn_split_k', 'yan_gemm_select_split_k',
+           'yan_gemm_split_k_workspace_bytes', 'yan_gemm_split_k_counter_bytes', 'yan_gemm_version')
 
 
 def load() -> ctypes.CDLL:
@@ -30,11 +30,12 @@ def load() -> ctypes.CDLL:
         lib.yan_per_token_cast_to_fp8.argtypes = [vp, ci, vp, vp, ll, ll, ci, ci, vp]
         lib.yan_per_block_cast_to_fp8.argtypes = [vp, ci, vp, vp, ci, ci, vp]
         lib.yan_gemm_fp8_fp8_bf16_nt_split_k.argtypes = [vp, vp, ll, ll, vp, vp, vp, ci, ci, ci, vp, ci, vp, ll]
-        lib.yan_gemm_select_split_k.argtypes = [ci, ci, ci, ci, ctypes.POINTER(ci), ctypes.POINTER(ci), ctypes.POINTER(ci)]
-        lib.yan_gemm_fp8_split_k_workspace_bytes.argtypes = lib.yan_gemm_fp8_split_k_counter_bytes.argtypes = []
+        lib.yan_gemm_select_split_k.argtypes = [ci, ci, ci, ci, ci, ctypes.POINTER(ci), ctypes.POINTER(ci), ctypes.POINTER(ci)]
+        lib.yan_gemm_bf16_tn_split_k.argtypes = lib.yan_gemm_fp16_tn_split_k.argtypes = [ci, ci, ci, vp, vp, vp, vp, vp, ll]
+        lib.yan_gemm_split_k_workspace_bytes.argtypes = lib.yan_gemm_split_k_counter_bytes.argtypes = []
         for name in SYMBOLS[:-1]:
             getattr(lib, name).restype = ci
-        lib.yan_gemm_fp8_split_k_workspace_bytes.restype = lib.yan_gemm_fp8_split_k_counter_bytes.restype = ll
+        lib.yan_gemm_split_k_workspace_bytes.restype = lib.yan_gemm_split_k_counter_bytes.restype = ll
         lib.yan_gemm_version.restype = ctypes.c_char_p
         _lib = lib
     return _lib
@@ -71,8 +72,8 @@ def gemm_fp8_fp8_bf16_nt(lhs, rhs, out: torch.Tensor, num_sms: int = 0) -> int:
 
 
 def split_k_workspace(device='cuda') -> torch.Tensor:
-    """A zero-filled workspace for `gemm_fp8_fp8_bf16_nt_split_k`, of the size the library asks for."""
-    return torch.zeros(load().yan_gemm_fp8_split_k_workspace_bytes(), dtype=torch.uint8, device=device)
+    """A zero-filled workspace for the split-K entry points, of the size the library asks for."""
+    return torch.zeros(load().yan_gemm_split_k_workspace_bytes(), dtype=torch.uint8, device=device)
 
 
 def gemm_fp8_fp8_bf16_nt_split_k(lhs, rhs, out: torch.Tensor, workspace: torch.Tensor, num_sms: int = 0) -> int:
@@ -91,10 +92,17 @@ def gemm_fp8_fp8_bf16_nt_static(lhs, rhs, out: torch.Tensor, num_sms: int = 0) -
                                                   sb.data_ptr(), out.data_ptr(), m, n, k, _stream_handle(), num_sms)
 
 
-def select_split_k(m: int, n: int, k: int, num_cus: int):
-    """(BLOCK_M, BLOCK_N, SPLIT_K) of the library's split-K plan, or None when K is not split."""
+def gemm_bf16_tn_split_k(a: torch.Tensor, b: torch.Tensor, c: torch.Tensor, workspace: torch.Tensor) -> int:
+    (m, k), n = a.shape, b.shape[0]
+    fn = load().yan_gemm_bf16_tn_split_k if a.dtype == torch.bfloat16 else load().yan_gemm_fp16_tn_split_k
+    return fn(m, n, k, a.data_ptr(), b.data_ptr(), c.data_ptr(), _stream_handle(), workspace.data_ptr(),
+              workspace.numel() * workspace.element_size())
+
+
+def select_split_k(m: int, n: int, k: int, num_cus: int, op: int = 1):
+    """(BLOCK_M, BLOCK_N, SPLIT_K) of the library's split-K plan (op 0: dense, 1: FP8), or None when K is not split."""
     bm, bn, split = ctypes.c_int(0), ctypes.c_int(0), ctypes.c_int(0)
-    assert load().yan_gemm_select_split_k(m, n, k, num_cus, ctypes.byref(bm), ctypes.byref(bn), ctypes.byref(split)) == 0
+    assert load().yan_gemm_select_split_k(op, m, n, k, num_cus, ctypes.byref(bm), ctypes.byref(bn), ctypes.byref(split)) == 0
     return (bm.value, bn.value, split.value) if split.value > 1 else None
 
 

@@ -92,6 +92,39 @@ bool pick_split_k(int m, int n, int k, int num_cus, int* bm, int* bn, int* split
     return best >= 0 && base - best >= 0.10 * (base + 3.5);
 }
 
+// Split-K plan of the dense 16-bit GEMM (get_split_k_dense_config in heuristics.py): false when K is not split.
+struct DenseSplitKTile { int bm, bn; double us_per_k_tile, extra_us; };      // extra < 0: not a tile plans use
+constexpr DenseSplitKTile kDenseSplitKTiles[] = {{64, 64, 0.248, 0.0}, {64, 128, 0.378, 1.0}, {128, 128, 0.51, 2.5}, {64, 192, 0.60, -1},
+                                                 {128, 192, 0.80, -1}, {128, 256, 0.94, -1}, {256, 128, 0.94, -1}};
+int dense_skinny_atoms(int m, int n, int k, int num_cus);
+
+bool pick_dense_split_k(int m, int n, int k, int num_cus, int* bm, int* bn, int* split_k) {
+    if (m <= 0 || n <= 0 || k <= 0 || dense_skinny_atoms(m, n, k, num_cus)) return false;
+    const int k_tiles = (k + 63) / 64;
+    int ubm = 0, ubn = 0;
+    pick(kDenseTiles, m, n, num_cus, &ubm, &ubn);
+    double unsplit_us = -1;
+    for (const DenseSplitKTile& t : kDenseSplitKTiles)
+        if (t.bm == ubm && t.bn == ubn) unsplit_us = t.us_per_k_tile;
+    if (unsplit_us < 0 || (long long)((m + ubm - 1) / ubm) * ((n + ubn - 1) / ubn) > num_cus) return false;
+    const double floor = double((long long)n * k * 2) / 6.0e6;
+    const double unsplit_time = k_tiles * unsplit_us;
+    const double base = unsplit_time > floor ? unsplit_time : floor;
+    double best = -1;
+    for (const DenseSplitKTile& t : kDenseSplitKTiles) {
+        if (t.extra_us < 0 || (t.bm > 64 && t.bm >= 2 * m)) continue;
+        const long long tiles = (long long)((m + t.bm - 1) / t.bm) * ((n + t.bn - 1) / t.bn);
+        for (const int s : kSplitKFactors) {
+            const int per_part = (k_tiles + s - 1) / s;
+            if ((tiles + 7) / 8 * 8 * s > (num_cus < 256 ? num_cus : 256) || per_part < 16) continue;
+            const double loop = per_part * t.us_per_k_tile + 0.5 + double(s * t.bm * t.bn * 4) / 1024 * 0.0125 + t.extra_us;
+            const double time = loop > floor ? loop : floor;
+            if (best < 0 || time < best) { best = time; *bm = t.bm; *bn = t.bn; *split_k = s; }
+        }
+    }
+    return best >= 0 && base - best >= 0.11 * (base + 3.5);
+}
+
 int device_cus() {
     static int cus = 0;
     if (cus == 0) {
@@ -110,8 +143,10 @@ int dense_skinny_atoms(int m, int n, int k, int num_cus) {
     return 0;
 }
 
+// With a workspace, problems the split-K plan covers run split (a workspace too small for the plan is an error); without
+// one, and for every other problem, a workgroup per tile.
 template <typename Atom, typename SkinnyAtom, typename Elem>
-int dense(int m, int n, int k, const void* a, const void* b, void* c, void* stream) {
+int dense(int m, int n, int k, const void* a, const void* b, void* c, void* stream, void* workspace = nullptr, size_t workspace_bytes = 0) {
     if (m == 0 || n == 0) return 0;
     if (m < 0 || n < 0) return int(hipErrorInvalidValue);
     hipStream_t s = static_cast<hipStream_t>(stream);
@@ -119,7 +154,16 @@ int dense(int m, int n, int k, const void* a, const void* b, void* c, void* stre
         if (atoms == 1) return int(yan::launch_dense_skinny<SkinnyAtom, Elem, 1, 8>(m, n, k, a, b, c, s));
         return int(yan::launch_dense_skinny<SkinnyAtom, Elem, 2, 8>(m, n, k, a, b, c, s));
     }
-    int bm = 0, bn = 0;
+    int bm = 0, bn = 0, split_k = 1;
+    if (workspace && pick_dense_split_k(m, n, k, device_cus(), &bm, &bn, &split_k)) {
+#define YAN_DENSE_SPLIT_K_CASE(BM, BN, S) \
+    if (bm == BM && bn == BN && split_k == S) return int(yan::launch_dense_split_k<Atom, Elem, BM, BN, S>(m, n, k, a, b, c, s, workspace, workspace_bytes));
+#define YAN_DENSE_SPLIT_K_TILE(BM, BN) YAN_DENSE_SPLIT_K_CASE(BM, BN, 2) YAN_DENSE_SPLIT_K_CASE(BM, BN, 3) YAN_DENSE_SPLIT_K_CASE(BM, BN, 4)
+        YAN_DENSE_SPLIT_K_TILE(64, 64) YAN_DENSE_SPLIT_K_TILE(64, 128) YAN_DENSE_SPLIT_K_TILE(128, 128)
+#undef YAN_DENSE_SPLIT_K_TILE
+#undef YAN_DENSE_SPLIT_K_CASE
+        return int(hipErrorInvalidValue);
+    }
     pick(kDenseTiles, m, n, device_cus(), &bm, &bn);
 #define YAN_DENSE_CASE(BM, BN) if (bm == BM && bn == BN) return int(yan::launch_dense<Atom, Elem, BM, BN>(m, n, k, a, b, c, s));
 #define YAN_DENSE_CASE_8W(BM, BN) if (bm == BM && bn == BN) return int(yan::launch_dense<Atom, Elem, BM, BN, 2>(m, n, k, a, b, c, s));
@@ -197,6 +241,18 @@ int yan_gemm_fp16_tn(int m, int n, int k, const void* a, const void* b, void* c,
     return dense<yan::MfmaF16_32x32x16, yan::MfmaF16_16x16x32, _Float16>(m, n, k, a, b, c, stream);
 }
 
+int yan_gemm_bf16_tn_split_k(int m, int n, int k, const void* a, const void* b, void* c, void* stream, void* workspace,
+                             long long workspace_bytes) {
+    if (!workspace || workspace_bytes < 0) return int(hipErrorInvalidValue);
+    return dense<yan::MfmaBF16_32x32x16, yan::MfmaBF16_16x16x32, __bf16>(m, n, k, a, b, c, stream, workspace, size_t(workspace_bytes));
+}
+
+int yan_gemm_fp16_tn_split_k(int m, int n, int k, const void* a, const void* b, void* c, void* stream, void* workspace,
+                             long long workspace_bytes) {
+    if (!workspace || workspace_bytes < 0) return int(hipErrorInvalidValue);
+    return dense<yan::MfmaF16_32x32x16, yan::MfmaF16_16x16x32, _Float16>(m, n, k, a, b, c, stream, workspace, size_t(workspace_bytes));
+}
+
 int yan_gemm_float_nt(int m, int n, int k, float alpha, const float* a, int lda, const float* b, int ldb, float beta,
                       float* c, int ldc, void* stream) {
     return int(gemm_nt(m, n, k, alpha, a, lda, b, ldb, beta, c, ldc, static_cast<hipStream_t>(stream), device_cus()));
@@ -209,8 +265,8 @@ int yan_gemm_fp8_fp8_bf16_nt(const void* lhs, const float* lhs_scales, long long
                      nullptr, 0);
 }
 
-long long yan_gemm_fp8_split_k_workspace_bytes(void) { return (long long)yan::kSplitKWorkspaceBytes; }
-long long yan_gemm_fp8_split_k_counter_bytes(void) { return (long long)yan::kSplitKCounterBytes; }
+long long yan_gemm_split_k_workspace_bytes(void) { return (long long)yan::kSplitKWorkspaceBytes; }
+long long yan_gemm_split_k_counter_bytes(void) { return (long long)yan::kSplitKCounterBytes; }
 
 int yan_gemm_fp8_fp8_bf16_nt_split_k(const void* lhs, const float* lhs_scales, long long lhs_scales_stride_m,
                                      long long lhs_scales_stride_k, const void* rhs, const float* rhs_scales, void* out,
@@ -306,12 +362,14 @@ int yan_gemm_select_tile(int op, int m, int n, int k, int num_cus, int* block_m,
     return 0;
 }
 
-int yan_gemm_select_split_k(int m, int n, int k, int num_cus, int* block_m, int* block_n, int* split_k) {
-    if (!block_m || !block_n || !split_k || num_cus <= 0) return 1;
-    if (!pick_split_k(m, n, k, num_cus, block_m, block_n, split_k)) { *block_m = *block_n = 0; *split_k = 1; }
+int yan_gemm_select_split_k(int op, int m, int n, int k, int num_cus, int* block_m, int* block_n, int* split_k) {
+    if (!block_m || !block_n || !split_k || num_cus <= 0 || (op != 0 && op != 1)) return 1;
+    const bool split = op == 0 ? pick_dense_split_k(m, n, k, num_cus, block_m, block_n, split_k)
+                               : pick_split_k(m, n, k, num_cus, block_m, block_n, split_k);
+    if (!split) { *block_m = *block_n = 0; *split_k = 1; }
     return 0;
 }
 
-const char* yan_gemm_version(void) { return "yan-gemm gfx950 11 dense + 2 weight-streaming dense + 7 fp32 + 10 fp8 tile variants + 15 split-K fp8 variants + 1 weight-streaming fp8 variant + 12 grouped fp8 variants + 4 quantiser kernels"; }
+const char* yan_gemm_version(void) { return "yan-gemm gfx950 11 dense + 18 split-K dense + 2 weight-streaming dense + 7 fp32 + 10 fp8 tile variants + 15 split-K fp8 variants + 1 weight-streaming fp8 variant + 12 grouped fp8 variants + 4 quantiser kernels"; }
 
 } // extern "C"

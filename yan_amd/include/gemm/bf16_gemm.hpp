@@ -15,6 +15,8 @@
 //     streaming: a ring of three to eight LDS stages, 4 waves, one per SIMD, each with a (BLOCK_N/WAVES_N) x
 //     (BLOCK_M/WAVES_M) slab of 32x32x16 MFMAs, up to 128 x 128 (256 accumulator registers, which the compiler keeps in
 //     AGPRs) (dense_gemm_body);
+//   * problems with long K and fewer ring tiles than compute units split K over SPLIT_K workgroups per tile, which meet in a
+//     caller-provided workspace (dense_gemm_split_k, dense_meet_partials; 64 x 4096 x 7168: 64 workgroups of 64 x 64 become 256);
 //   * B rows feed the MFMA row operand and A rows the column operand, so a lane's four consecutive accumulator
 //     registers are four consecutive n of one m: contiguous in C;
 //   * fp32 accumulators, round-to-nearest-even on the way out;
@@ -51,13 +53,65 @@ struct DenseTileConfig {
 
 // STAGES (3 ..): a ring of that many LDS stages with STAGES - 1 k-tiles in
 // flight, for the smaller tiles, which are picked when a problem is bound by streaming its operands.
-template <typename Atom, typename Elem, int BLOCK_M, int BLOCK_N, int STAGES>
+// Where the SPLIT_K parts of a dense tile meet: as fp8_meet_partials in fp8_gemm.hpp (sums written and read at device scope,
+// a counter per tile and wave, the last wave to arrive adds the parts up in the order of their K ranges and stores).
+template <int SPLIT_K, int NW, int TN, int TM, typename Acc>
+__device__ __forceinline__ bool
+dense_meet_partials(Acc (&acc)[TN][TM], float* __restrict__ partials, unsigned* __restrict__ counters, int tile_slot, int split, int wave, int lane) {
+    constexpr int kSc1 = 16;        // cache-policy bit sc1 of gfx950 buffer instructions: device scope
+    constexpr uint32_t VEC_BYTES = kWaveSize * 16, WAVE_BYTES = TN * TM * 4 * VEC_BYTES, PART_BYTES = NW * WAVE_BYTES;
+    const __amdgpu_buffer_rsrc_t parts = make_rsrc(partials + size_t(tile_slot) * (SPLIT_K * PART_BYTES / 4), SPLIT_K * PART_BYTES);
+    const uint32_t lane_off = uint32_t(wave) * WAVE_BYTES + lane * 16;
+#pragma unroll
+    for (int i = 0; i < TN; ++i)
+#pragma unroll
+        for (int j = 0; j < TM; ++j)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const f32x4 v = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
+                __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(i32x4, v), parts, lane_off + ((i * TM + j) * 4 + q) * VEC_BYTES,
+                                                       split * PART_BYTES, kSc1);
+            }
+    __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, kNoWaitLgkm));
+    asm volatile("" ::: "memory");
+    unsigned before = 0;
+    if (lane == 0) before = __hip_atomic_fetch_add(counters + tile_slot * NW + wave, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    before = __builtin_amdgcn_readfirstlane(before);
+    asm volatile("" ::: "memory");
+    if (before != SPLIT_K - 1) return false;
+#pragma unroll
+    for (int i = 0; i < TN; ++i)
+#pragma unroll
+        for (int j = 0; j < TM; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+#pragma unroll
+    for (int s = 0; s < SPLIT_K; ++s)
+#pragma unroll
+        for (int i = 0; i < TN; ++i)
+#pragma unroll
+            for (int j = 0; j < TM; ++j)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const f32x4 v = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(parts, lane_off + ((i * TM + j) * 4 + q) * VEC_BYTES,
+                                                                                                    s * PART_BYTES, kSc1));
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) acc[i][j][4 * q + r] += v[r];
+                }
+    if (lane == 0) __hip_atomic_store(counters + tile_slot * NW + wave, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return true;
+}
+
+template <typename Atom, typename Elem, int BLOCK_M, int BLOCK_N, int STAGES, int SPLIT_K = 1>
 __device__ __forceinline__ void
 dense_gemm_body(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, Elem* __restrict__ C,
-                int m, int n, int k, int bid) {
+                int m, int n, int k, int bid, float* __restrict__ partials = nullptr, unsigned* __restrict__ counters = nullptr) {
     using Cfg = DenseTileConfig<BLOCK_M, BLOCK_N>;
     constexpr int NW = Cfg::NUM_WAVES, TN = Cfg::WTN / 32, TM = Cfg::WTM / 32;
     static_assert(STAGES >= 3 && STAGES <= Cfg::MAX_STAGES, "a ring of three or more stages that fits the LDS");
+    // SPLIT_K > 1: launch slot `bid` is part `bid % SPLIT_K` of tile slot `bid / SPLIT_K`
+    [[maybe_unused]] int split = 0;
+    if constexpr (SPLIT_K > 1) { split = bid % SPLIT_K; bid /= SPLIT_K; }
 
     const XcdTileScheduler<> sched(m, n, BLOCK_M, BLOCK_N);
     const TileCoord tile = sched.tile_of(bid);
@@ -81,6 +135,14 @@ dense_gemm_body(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, El
     const int num_k_tiles = ceil_div(k_bytes, kRowBytes);
     const int tail_tile = (k_bytes % kRowBytes) ? num_k_tiles - 1 : -1;
     const uint32_t tail_a = stage_a.tail_voff(k_bytes % kRowBytes), tail_b = stage_b.tail_voff(k_bytes % kRowBytes);
+    // this part's k-tiles; copies past them keep the count of instructions in flight and move nothing
+    int kt_lo = 0, kt_hi = num_k_tiles;
+    if constexpr (SPLIT_K > 1) {
+        const int per = ceil_div(num_k_tiles, SPLIT_K);
+        kt_lo = min(split * per, num_k_tiles);
+        kt_hi = min(kt_lo + per, num_k_tiles);
+    }
+    const __amdgpu_buffer_rsrc_t rsrc_none = make_rsrc(A, 0);
     using StA = TileStager<BLOCK_M, NW>;
     using StB = TileStager<BLOCK_N, NW>;
     constexpr int NUM_COPIES = StA::PASSES + StB::PASSES;
@@ -88,8 +150,9 @@ dense_gemm_body(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, El
     // Copy number `d` (A passes first, then B passes) of k-tile `kt` into the given stage.
     auto copy_pass = [&](int d, int kt, uint8_t* la, uint8_t* lb) {
         const bool tail = kt == tail_tile;
-        if (d < StA::PASSES) stage_a.issue_pass_from(rsrc_a, la, kt * kRowBytes, wave, d, tail ? tail_a : stage_a.voff);
-        else stage_b.issue_pass_from(rsrc_b, lb, kt * kRowBytes, wave, d - StA::PASSES, tail ? tail_b : stage_b.voff);
+        const bool live = kt < kt_hi;
+        if (d < StA::PASSES) stage_a.issue_pass_from(live ? rsrc_a : rsrc_none, la, kt * kRowBytes, wave, d, tail ? tail_a : stage_a.voff);
+        else stage_b.issue_pass_from(live ? rsrc_b : rsrc_none, lb, kt * kRowBytes, wave, d - StA::PASSES, tail ? tail_b : stage_b.voff);
     };
 
     // Lane-constant LDS offsets of the four 16-deep K steps inside a 64-deep tile.
@@ -160,9 +223,9 @@ dense_gemm_body(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, El
 #pragma unroll
     for (int t = 0; t < STAGES - 1; ++t)
 #pragma unroll
-        for (int d = 0; d < NUM_COPIES; ++d) copy_pass(d, t, ring + t * STAGE_BYTES, ring + t * STAGE_BYTES + BLOCK_M * kRowBytes);
+        for (int d = 0; d < NUM_COPIES; ++d) copy_pass(d, kt_lo + t, ring + t * STAGE_BYTES, ring + t * STAGE_BYTES + BLOCK_M * kRowBytes);
     int st = 0;
-    for (int kt = 0; kt < num_k_tiles; ++kt) {
+    for (int kt = kt_lo; kt < kt_hi; ++kt) {
         __builtin_amdgcn_s_waitcnt(waitcnt_imm((STAGES - 2) * NUM_COPIES, kNoWaitLgkm));
         asm volatile("" ::: "memory");
         __builtin_amdgcn_s_barrier();
@@ -184,6 +247,14 @@ dense_gemm_body(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, El
     // stored with the non-temporal hint, so that it does not push the operand panels out of them.
     const bool stream_out = size_t(m) * n * sizeof(Elem) > (size_t(32) << 20);
     const __amdgpu_buffer_rsrc_t rsrc_c = make_out_rsrc(C + size_t(m0) * n + n0);
+    if constexpr (SPLIT_K > 1) {
+        // every wave has read the last k-tile before any wave's epilogue writes into that stage
+        __builtin_amdgcn_s_waitcnt(waitcnt_imm(kNoWaitVm, 0));
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        if (!dense_meet_partials<SPLIT_K, NW>(acc, partials, counters, bid, split, wave, lane)) return;
+    }
     constexpr int PITCH = Cfg::WTN * 2 + 16, REGION = 32 * PITCH;
     // lanes per row segment; rows one store instruction covers (a slab width that does not divide the wave leaves the last
     // lanes idle); store instructions per 32 rows
@@ -191,10 +262,12 @@ dense_gemm_body(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, El
     static_assert(NW * REGION <= STAGE_BYTES && STORES >= 1 && sizeof(Elem) == 2);
     if ((n % 8) == 0) {
         // every wave has read the last k-tile (a bare barrier: nothing here depends on the copies still under way)
-        __builtin_amdgcn_s_waitcnt(waitcnt_imm(kNoWaitVm, 0));
-        asm volatile("" ::: "memory");
-        __builtin_amdgcn_s_barrier();
-        asm volatile("" ::: "memory");
+        if constexpr (SPLIT_K == 1) {
+            __builtin_amdgcn_s_waitcnt(waitcnt_imm(kNoWaitVm, 0));
+            asm volatile("" ::: "memory");
+            __builtin_amdgcn_s_barrier();
+            asm volatile("" ::: "memory");
+        }
         uint8_t* region = ring + (st == 0 ? STAGES - 1 : st - 1) * STAGE_BYTES + wave * REGION;
         const int ml = lane % 32, r_in = lane / LANES_PER_ROW, c = lane % LANES_PER_ROW;
         const int n_in_tile = wn * Cfg::WTN + 8 * c;
@@ -512,12 +585,27 @@ dense_gemm_mfma(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, El
     dense_gemm_walk<Atom, Elem, BLOCK_M, BLOCK_N, STAGES>(A, B, C, m, n, k, num_slots);
 }
 
+// The ring tiles with K split SPLIT_K ways: launch slot s is part s % SPLIT_K of tile slot s / SPLIT_K.
+template <typename Atom, typename Elem, int BLOCK_M, int BLOCK_N, int STAGES, int SPLIT_K>
+__global__ void __launch_bounds__(4 * kWaveSize)
+dense_gemm_split_k(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, Elem* __restrict__ C, int m, int n, int k,
+                   float* __restrict__ partials, unsigned* __restrict__ counters) {
+    dense_gemm_body<Atom, Elem, BLOCK_M, BLOCK_N, STAGES, SPLIT_K>(A, B, C, m, n, k, int(blockIdx.x), partials, counters);
+}
+
 // The fp16 flavour under the name of the reference's kernel (yan/include/gemm/cute_gemm.cuh:20), so that profiler
 // filters written for it (tests/test_cute.py:35 looks for 'fp16_gemm_cute') keep finding it.
 template <int BLOCK_M, int BLOCK_N, int STAGES>
 __global__ void __launch_bounds__(4 * kWaveSize)
 fp16_gemm_cute(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, _Float16* __restrict__ C, int m, int n, int k, int num_slots) {
     dense_gemm_walk<MfmaF16_32x32x16, _Float16, BLOCK_M, BLOCK_N, STAGES>(A, B, C, m, n, k, num_slots);
+}
+
+template <int BLOCK_M, int BLOCK_N, int STAGES, int SPLIT_K>
+__global__ void __launch_bounds__(4 * kWaveSize)
+fp16_gemm_cute_split_k(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, _Float16* __restrict__ C, int m, int n, int k,
+                       float* __restrict__ partials, unsigned* __restrict__ counters) {
+    dense_gemm_body<MfmaF16_32x32x16, _Float16, BLOCK_M, BLOCK_N, STAGES, SPLIT_K>(A, B, C, m, n, k, int(blockIdx.x), partials, counters);
 }
 
 template <int BLOCK_M, int BLOCK_N>
@@ -575,6 +663,34 @@ inline hipError_t launch_dense(int m, int n, int k, const void* a, const void* b
     return hipGetLastError();
 }
 
+// K split SPLIT_K ways over as many workgroups per tile (ring tiles). `workspace`: device memory of at least
+// kSplitKCounterBytes + tile slots * SPLIT_K * BLOCK_M * BLOCK_N * 4 bytes: counters that are zero before the first launch and
+// after every launch, then the partial sums. Launches that share a workspace must not overlap (see fp8_gemm.hpp).
+template <typename Atom, typename Elem, int BLOCK_M, int BLOCK_N, int SPLIT_K, int STAGES = DenseTileConfig<BLOCK_M, BLOCK_N>::MAX_STAGES>
+inline hipError_t launch_dense_split_k(int m, int n, int k, const void* a, const void* b, void* c, hipStream_t stream,
+                                       void* workspace, size_t workspace_bytes) {
+    static_assert(SPLIT_K > 1 && !(BLOCK_M == 256 && STAGES == 2));
+    if (m == 0 || n == 0) return hipSuccess;
+    if (hipError_t e = check_dense_args(m, n, k, a, b, c, BLOCK_M, BLOCK_N); e != hipSuccess) return e;
+    if (!workspace) return hipErrorInvalidValue;
+    using Cfg = DenseTileConfig<BLOCK_M, BLOCK_N>;
+    const XcdTileScheduler<> sched(m, n, BLOCK_M, BLOCK_N);
+    const size_t slots = size_t(sched.grid_size());
+    if (slots * Cfg::NUM_WAVES * 4 > kSplitKCounterBytes) return hipErrorInvalidValue;
+    if (workspace_bytes < kSplitKCounterBytes + slots * SPLIT_K * BLOCK_M * BLOCK_N * 4) return hipErrorInvalidValue;
+    unsigned* counters = static_cast<unsigned*>(workspace);
+    float* partials = reinterpret_cast<float*>(static_cast<uint8_t*>(workspace) + kSplitKCounterBytes);
+    if constexpr (__is_same(Elem, _Float16))
+        hipLaunchKernelGGL((fp16_gemm_cute_split_k<BLOCK_M, BLOCK_N, STAGES, SPLIT_K>), dim3(int(slots) * SPLIT_K),
+                           dim3(Cfg::NUM_WAVES * kWaveSize), 0, stream, static_cast<const uint8_t*>(a),
+                           static_cast<const uint8_t*>(b), static_cast<Elem*>(c), m, n, k, partials, counters);
+    else
+        hipLaunchKernelGGL((dense_gemm_split_k<Atom, Elem, BLOCK_M, BLOCK_N, STAGES, SPLIT_K>), dim3(int(slots) * SPLIT_K),
+                           dim3(Cfg::NUM_WAVES * kWaveSize), 0, stream, static_cast<const uint8_t*>(a),
+                           static_cast<const uint8_t*>(b), static_cast<Elem*>(c), m, n, k, partials, counters);
+    return hipGetLastError();
+}
+
 } // namespace yan
 
 // bf16 in, fp32 accumulate, bf16 out. NUM_STAGES is the number of LDS stages (2 .. DenseTileConfig::MAX_STAGES; two
@@ -588,6 +704,18 @@ inline hipError_t gemm_tn(int m, int n, int k, const __hip_bfloat16* A, const __
 }
 
 // fp16 in, fp32 accumulate, fp16 out.
+template <int BLOCK_M, int BLOCK_N, int NUM_STAGES, int SPLIT_K>
+inline hipError_t gemm_tn_split_k(int m, int n, int k, const __hip_bfloat16* A, const __hip_bfloat16* B, __hip_bfloat16* C,
+                                  hipStream_t stream, void* workspace, size_t workspace_bytes) {
+    return yan::launch_dense_split_k<yan::MfmaBF16_32x32x16, __bf16, BLOCK_M, BLOCK_N, SPLIT_K, NUM_STAGES>(m, n, k, A, B, C, stream, workspace, workspace_bytes);
+}
+
+template <int BLOCK_M, int BLOCK_N, int NUM_STAGES, int SPLIT_K>
+inline hipError_t gemm_tn_split_k(int m, int n, int k, const __half* A, const __half* B, __half* C, hipStream_t stream,
+                                  void* workspace, size_t workspace_bytes) {
+    return yan::launch_dense_split_k<yan::MfmaF16_32x32x16, _Float16, BLOCK_M, BLOCK_N, SPLIT_K, NUM_STAGES>(m, n, k, A, B, C, stream, workspace, workspace_bytes);
+}
+
 template <int BLOCK_M, int BLOCK_N, int NUM_STAGES>
 inline hipError_t gemm_tn(int m, int n, int k, const __half* A, const __half* B, __half* C, hipStream_t stream, int num_sms = 0) {
     if constexpr (BLOCK_N == 16) return yan::launch_dense_skinny<yan::MfmaF16_16x16x32, _Float16, BLOCK_M / 16, 8>(m, n, k, A, B, C, stream);

@@ -222,10 +222,6 @@ fp8_store_slab(const f32x4 (&acc)[TN][TM], uint8_t* region, __amdgpu_buffer_rsrc
 // device scope (cache policy sc1: written through to memory, read from there), as the counter is; a device-scope fence
 // instead would write back and invalidate the whole L2 of the XCD once per wave (measured: 45-110 us for a 10 us GEMM).
 constexpr int kDeviceScope = 16;        // cache-policy bit sc1 of gfx950 buffer instructions
-// The arrival counters take the first kSplitKCounterBytes of a split-K workspace whatever the problem, so that launches of
-// different shapes can share one; the largest plan of the tile heuristics (256 workgroups of 128 x 128 partial sums)
-// fits kSplitKWorkspaceBytes.
-constexpr size_t kSplitKCounterBytes = 16 * 1024, kSplitKWorkspaceBytes = kSplitKCounterBytes + size_t(256) * 128 * 128 * 4;
 template <int SPLIT_K, int NW, int TN, int TM>
 __device__ __forceinline__ bool
 fp8_meet_partials(f32x4 (&acc)[TN][TM], float* __restrict__ partials, unsigned* __restrict__ counters, int tile_slot, int split, int wave, int lane) {

@@ -188,4 +188,9 @@ __host__ __device__ inline int capped_grid(int slots, int num_sms, int device_cu
     return num_sms >= kNumXCD ? num_sms / kNumXCD * kNumXCD : num_sms;
 }
 
+// Split-K workspaces (fp8_gemm.hpp, bf16_gemm.hpp): the arrival counters take the first kSplitKCounterBytes whatever the
+// problem, so that launches of different shapes and kernels can share a workspace; the largest plan of the tile heuristics
+// (256 workgroups of 128 x 128 partial sums) fits kSplitKWorkspaceBytes.
+constexpr size_t kSplitKCounterBytes = 16 * 1024, kSplitKWorkspaceBytes = kSplitKCounterBytes + size_t(256) * 128 * 128 * 4;
+
 } // namespace yan

@@ -12,7 +12,8 @@ import functools
 
 import torch
 
-from .heuristics import get_best_dense_config, get_dense_num_stages, get_dense_tile_space, get_skinny_dense_config, tuning_enabled
+from .heuristics import (get_best_dense_config, get_dense_num_stages, get_dense_tile_space, get_skinny_dense_config,
+                         get_split_k_dense_config, tuning_enabled)
 from .tuner import FrozenKeys, jit_tuner
 from .utils import get_num_sms, get_num_sms_cap
 
@@ -26,10 +27,37 @@ constexpr auto kNumSMs = {NUM_SMS};
 
 __return_code = static_cast<int>(gemm_tn<BLOCK_M, BLOCK_N, kNumStages>(m, n, k, A, B, C, stream, kNumSMs));
 """
+# K split over SPLIT_K workgroups per tile; the parts meet in `workspace` (launch_dense_split_k in gemm/bf16_gemm.hpp).
+split_k_template = """
+// Templated args from Python JIT call
+constexpr auto BLOCK_M = {BLOCK_M};
+constexpr auto BLOCK_N = {BLOCK_N};
+constexpr auto kNumStages = {NUM_STAGES};
+constexpr auto kSplitK = {SPLIT_K};
+
+__return_code = static_cast<int>(gemm_tn_split_k<BLOCK_M, BLOCK_N, kNumStages, kSplitK>(m, n, k, A, B, C, stream, workspace, workspace_bytes));
+"""
 
 
 def _arg_defs(dtype: torch.dtype):
     return (('m', int), ('n', int), ('k', int), ('A', dtype), ('B', dtype), ('C', dtype), ('stream', torch.cuda.Stream))
+
+
+def _split_k_arg_defs(dtype: torch.dtype):
+    return _arg_defs(dtype) + (('workspace', torch.uint8), ('workspace_bytes', int))
+
+
+@functools.lru_cache(maxsize=None)
+def dense_split_k_plan(m: int, n: int, k: int, dtype: torch.dtype, num_cus: int):
+    """(name, keys, arg_defs) of the split-K kernel a call with these sizes uses, or None when K is not split
+    (`get_split_k_dense_config`); needs no GPU."""
+    plan = get_split_k_dense_config(m, n, k, num_cus)
+    if plan is None:
+        return None
+    block_m, block_n, split_k = plan
+    name = 'gemm_bf16_tn_split_k' if dtype == torch.bfloat16 else 'gemm_fp16_tn_split_k'
+    keys = FrozenKeys({'BLOCK_M': block_m, 'BLOCK_N': block_n, 'NUM_STAGES': get_dense_num_stages(block_m, block_n), 'SPLIT_K': split_k})
+    return name, keys, _split_k_arg_defs(dtype)
 
 
 @functools.lru_cache(maxsize=None)
@@ -69,12 +97,19 @@ def _gemm_16bit_tn(a: torch.Tensor, b: torch.Tensor, c: torch.Tensor, dtype: tor
 
     stream = torch.cuda.current_stream()
     args = (m, n, k, a, b, c, stream)
+    code_template = template
     if tuning_enabled() and not get_skinny_dense_config(m, n, k, get_num_sms()):
         name, keys, space, arg_defs = dense_tuning_plan(m, n, k, dtype, get_num_sms(), get_num_sms_cap())
     else:
         (name, keys, arg_defs), space = dense_kernel_plan(m, n, k, dtype, get_num_sms(), get_num_sms_cap()), ()
+        split = dense_split_k_plan(m, n, k, dtype, get_num_sms())
+        if split is not None:
+            from .gemm import SPLIT_K_WORKSPACE_BYTES, split_k_workspace
+            name, keys, arg_defs = split
+            code_template = split_k_template
+            args += (split_k_workspace(c.device, stream), SPLIT_K_WORKSPACE_BYTES)
     runtime = jit_tuner.compile_and_tune(name=name, keys=keys, space=space, includes=includes,
-                                         arg_defs=arg_defs, template=template, args=args)
+                                         arg_defs=arg_defs, template=code_template, args=args)
     rc = runtime(*args)
     assert rc == 0, f'{name} failed with HIP error {rc}'
 

@@ -191,6 +191,50 @@ def get_split_k_fp8_config(m: int, n: int, k: int, num_cus: int) -> Optional[Tup
     return None
 
 
+# Split-K of the dense GEMM: microseconds per k-tile (64 deep) of a workgroup on a ring tile with the chip full (measured with
+# weights cycling through more matrices than the caches hold), for every tile the unsplit pick can be; the first three are
+# the tiles split-K plans use, with what their longer ring fill and larger partial sums add per launch.
+_DENSE_SPLIT_K_TILE_US = {(64, 64): 0.248, (64, 128): 0.378, (128, 128): 0.51, (64, 192): 0.60, (128, 192): 0.80, (128, 256): 0.94,
+                          (256, 128): 0.94}
+_DENSE_SPLIT_K_EXTRA_US = {(64, 64): 0.0, (64, 128): 1.0, (128, 128): 2.5}
+DENSE_SPLIT_K_FACTORS = (2, 3, 4)
+
+
+def get_split_k_dense_config(m: int, n: int, k: int, num_cus: int) -> Optional[Tuple[int, int, int]]:
+    """(BLOCK_M, BLOCK_N, SPLIT_K) when the dense 16-bit GEMM should split K over SPLIT_K workgroups per tile, else None.
+    The rule of `get_split_k_fp8_config` with the dense tiles' numbers: the smallest dense tile holds 64 weight rows, so
+    m = 64, n = 4096 puts 64 of 256 compute units to work and K = 7168 keeps each for 112 k-tiles; in four parts the same
+    tiles fill the chip. A plan fits one round (tile slots x SPLIT_K <= num_cus), leaves every part at least 16 k-tiles and
+    must beat the unsplit pick by 11 % of its modelled time plus 3.5 us. Measured (bf16, weights cycling, unsplit ->
+    plan): 64 x 4096 x 7168 37.1 -> 16.2 us, 256 x 2048 x 7168 34.2 -> 20.3, 256 x 5120 x 5120 44.7 -> 33.9,
+    256 x 7168 x 16384 113.4 -> 90.9, 512 x 4096 x 7168 53.4 -> 43.9 (hipBLASLt on the same operands: 22.7, 24.7, 49.6, 140.4, -);
+    over 54 shapes swept with every tile and factor the plan is the fastest measured or within 6 % of it (11 % in one case),
+    and over 118 shapes with a plan (m = 33..1024, 14 (n, k)) it takes 0.35 to 0.92 of the unsplit time, median 0.65. Same rule as
+    `pick_dense_split_k` in yan_amd/csrc/yan_gemm_capi.hip (a CPU test keeps the two in step)."""
+    if get_skinny_dense_config(m, n, k, num_cus) or m <= 0 or n <= 0 or k <= 0:
+        return None
+    k_tiles = ceil_div(k, 64)
+    unsplit = get_best_dense_config(m, n, k, num_cus)
+    if unsplit not in _DENSE_SPLIT_K_TILE_US or ceil_div(m, unsplit[0]) * ceil_div(n, unsplit[1]) > num_cus:
+        return None
+    floor = n * k * 2 / 6.0e6
+    base = max(k_tiles * _DENSE_SPLIT_K_TILE_US[unsplit], floor)
+    best, best_plan = None, None
+    for (bm, bn), extra in _DENSE_SPLIT_K_EXTRA_US.items():
+        if bm > 64 and bm >= 2 * m:
+            continue                # a tile more than twice as tall as the problem
+        tiles = ceil_div(m, bm) * ceil_div(n, bn)
+        for split in DENSE_SPLIT_K_FACTORS:
+            if ceil_div(tiles, 8) * 8 * split > min(num_cus, 256) or ceil_div(k_tiles, split) < 16:
+                continue
+            t = max(ceil_div(k_tiles, split) * _DENSE_SPLIT_K_TILE_US[(bm, bn)] + 0.5 + (split * bm * bn * 4) / 1024 * 0.0125 + extra, floor)
+            if best is None or t < best:
+                best, best_plan = t, (bm, bn, split)
+    if best is not None and base - best >= 0.11 * (base + 3.5):
+        return best_plan
+    return None
+
+
 # (BLOCK_M, BLOCK_N) -> cost per unit of tile area; tiles below 128 rows split K over their four waves.
 _FLOAT_TILES = {(256, 256): 1.00, (128, 256): 1.015, (128, 128): 1.03, (128, 64): 1.04, (64, 64): 1.13, (32, 64): 1.13, (32, 32): 1.25}
 
