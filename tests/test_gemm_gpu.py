@@ -138,7 +138,13 @@ def test_dense_weight_streaming_kernel_leaves_its_neighbours_alone(m, n, k):
     assert heuristics.get_dense_tile(m, n, k, yan.get_num_sms())[1] == 16
     a, b, _ = testing.make_bf16_case(m, n, k, seed=6, device='cuda')
     big = torch.full((m + 2, n), 7.0, dtype=torch.bfloat16, device='cuda')
-    yan.gemm_bf16_tn(a, b, big[:m])
+    # built from its plan: where K is long enough the public entry point prefers a split-K plan to the two-atom kernel
+    from yan_amd.jit_kernels import bf16_gemm
+    name, keys, defs = bf16_gemm.dense_kernel_plan(m, n, k, torch.bfloat16, yan.get_num_sms())
+    assert keys['BLOCK_N'] == 16
+    runtime = jit.build(name, defs, jit.generate(bf16_gemm.includes, defs, jit.cpp_format(bf16_gemm.template, keys)))
+    assert runtime(m, n, k, a, b, big[:m], torch.cuda.current_stream()) == 0
+    torch.cuda.synchronize()
     assert bool((big[m:] == 7.0).all())
     assert oracle.calc_diff(_np(big[:m]), oracle.gemm_bf16_tn_ref(_np(a), _np(b))) < BF16_TOL
     again = torch.empty(m, n, dtype=torch.bfloat16, device='cuda')

@@ -99,7 +99,7 @@ constexpr DenseSplitKTile kDenseSplitKTiles[] = {{64, 64, 0.248, 0.0}, {64, 128,
 int dense_skinny_atoms(int m, int n, int k, int num_cus);
 
 bool pick_dense_split_k(int m, int n, int k, int num_cus, int* bm, int* bn, int* split_k) {
-    if (m <= 0 || n <= 0 || k <= 0 || dense_skinny_atoms(m, n, k, num_cus)) return false;
+    if (m <= 0 || n <= 0 || k <= 0 || (m <= 16 && dense_skinny_atoms(m, n, k, num_cus))) return false;
     const int k_tiles = (k + 63) / 64;
     int ubm = 0, ubn = 0;
     pick(kDenseTiles, m, n, num_cus, &ubm, &ubn);
@@ -150,11 +150,9 @@ int dense(int m, int n, int k, const void* a, const void* b, void* c, void* stre
     if (m == 0 || n == 0) return 0;
     if (m < 0 || n < 0) return int(hipErrorInvalidValue);
     hipStream_t s = static_cast<hipStream_t>(stream);
-    if (const int atoms = dense_skinny_atoms(m, n, k, device_cus())) {
-        if (atoms == 1) return int(yan::launch_dense_skinny<SkinnyAtom, Elem, 1, 8>(m, n, k, a, b, c, s));
-        return int(yan::launch_dense_skinny<SkinnyAtom, Elem, 2, 8>(m, n, k, a, b, c, s));
-    }
     int bm = 0, bn = 0, split_k = 1;
+    // a split-K plan goes before the two-atom weight-streaming kernel (pick_dense_split_k makes none up to 16 rows where the
+    // one-atom kernel runs)
     if (workspace && pick_dense_split_k(m, n, k, device_cus(), &bm, &bn, &split_k)) {
 #define YAN_DENSE_SPLIT_K_CASE(BM, BN, S) \
     if (bm == BM && bn == BN && split_k == S) return int(yan::launch_dense_split_k<Atom, Elem, BM, BN, S>(m, n, k, a, b, c, s, workspace, workspace_bytes));
@@ -163,6 +161,10 @@ int dense(int m, int n, int k, const void* a, const void* b, void* c, void* stre
 #undef YAN_DENSE_SPLIT_K_TILE
 #undef YAN_DENSE_SPLIT_K_CASE
         return int(hipErrorInvalidValue);
+    }
+    if (const int atoms = dense_skinny_atoms(m, n, k, device_cus())) {
+        if (atoms == 1) return int(yan::launch_dense_skinny<SkinnyAtom, Elem, 1, 8>(m, n, k, a, b, c, s));
+        return int(yan::launch_dense_skinny<SkinnyAtom, Elem, 2, 8>(m, n, k, a, b, c, s));
     }
     pick(kDenseTiles, m, n, device_cus(), &bm, &bn);
 #define YAN_DENSE_CASE(BM, BN) if (bm == BM && bn == BN) return int(yan::launch_dense<Atom, Elem, BM, BN>(m, n, k, a, b, c, s));

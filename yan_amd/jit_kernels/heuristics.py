@@ -210,9 +210,12 @@ def get_split_k_dense_config(m: int, n: int, k: int, num_cus: int) -> Optional[T
     256 x 7168 x 16384 113.4 -> 90.9, 512 x 4096 x 7168 53.4 -> 43.9 (hipBLASLt on the same operands: 22.7, 24.7, 49.6, 140.4, -);
     over 54 shapes swept with every tile and factor the plan is the fastest measured or within 6 % of it (11 % in one case),
     and over 118 shapes with a plan (m = 33..1024, 14 (n, k)) it takes 0.35 to 0.92 of the unsplit time, median 0.65. Same rule as
-    `pick_dense_split_k` in yan_amd/csrc/yan_gemm_capi.hip (a CPU test keeps the two in step)."""
-    if get_skinny_dense_config(m, n, k, num_cus) or m <= 0 or n <= 0 or k <= 0:
-        return None
+    `pick_dense_split_k` in yan_amd/csrc/yan_gemm_capi.hip (a CPU test keeps the two in step). A plan goes before the
+    two-atom weight-streaming kernel (17 to 32 rows; n = 4096, k = 7168: 21.1 - 25.2 us against 14.8 - 14.9 for 64 x 64 tiles
+    in four parts), which therefore runs only where no plan exists or no workspace is at hand (the C library's plain entry
+    points); up to 16 rows the one-atom kernel stays (14.5 - 18.2 us against 14.7 - 14.8, and ahead on longer K)."""
+    if m <= 0 or n <= 0 or k <= 0 or (m <= 16 and get_skinny_dense_config(m, n, k, num_cus)):
+        return None         # up to 16 rows the weight-streaming kernel is as fast or faster; from 17 rows a plan goes first
     k_tiles = ceil_div(k, 64)
     unsplit = get_best_dense_config(m, n, k, num_cus)
     if unsplit not in _DENSE_SPLIT_K_TILE_US or ceil_div(m, unsplit[0]) * ceil_div(n, unsplit[1]) > num_cus:
