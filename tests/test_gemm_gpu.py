@@ -1097,6 +1097,41 @@ def test_entry_points_replay_correctly_from_a_captured_graph():
         assert float(replayed['fp8'].float().abs().sum()) > 0 and float(replayed['masked'][1, 40:].float().abs().sum()) == 0
 
 
+def test_split_k_replays_correctly_from_a_captured_graph():
+    """Split-K launches captured into a graph: the workspace of the capture stream is made during the capture (a torch
+    allocation and a fill kernel, both legal there) and every replay, with new inputs and eager split-K work on the other
+    stream's workspace in between, gives the bits of an eager run."""
+    _announce('split-k graph replay')
+    (a8, sa), (b8, sb), out8 = testing.make_fp8_case(33, 2112, 5376, seed=8, device='cuda', gen_device='cuda')
+    a, b, c = testing.make_bf16_case(100, 196, 3080, seed=9, scale=0.02, device='cuda', gen_device='cuda')
+    assert yan.gemm.fp8_split_k_plan(33, 2112, 5376, yan.get_num_sms(), False) is not None
+
+    def chain():
+        yan.gemm_fp8_fp8_bf16_nt((a8, sa), (b8, sb), out8)
+        yan.gemm_bf16_tn(a, b, c)
+
+    chain()                                                # loads the kernels
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        chain()
+    g = torch.Generator(device='cuda').manual_seed(5)
+    for rep in range(3):
+        a.copy_((torch.randn(a.shape, device='cuda', generator=g) * 0.02).bfloat16())
+        a8.copy_(torch.randn(a8.shape, device='cuda', generator=g).to(torch.float8_e4m3fn))
+        out8.zero_()
+        c.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        replayed = (out8.clone(), c.clone())
+        out8.zero_()
+        c.zero_()
+        chain()
+        torch.cuda.synchronize()
+        assert torch.equal(replayed[0], out8) and torch.equal(replayed[1], c), rep
+        assert float(out8.float().abs().sum()) > 0 and float(c.float().abs().sum()) > 0
+
+
 def test_capi_seeded_random_shapes_against_device_references():
     """Breadth: 240 seeded random shapes through the C entries (every tile variant, ragged edges, k tails, leading
     dimensions), each against an fp32 / fp64 product of the same operands on the device. The oracle-based tests above
