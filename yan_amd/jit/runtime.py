@@ -49,9 +49,13 @@ class Runtime:
             if isinstance(arg, torch.Tensor):
                 assert arg.dtype == dtype, f'Expected tensor dtype `{dtype}` for `{name}`, got `{arg.dtype}`'
                 cargs.append(arg.data_ptr())
+            elif dtype is torch.cuda.Stream:
+                # a Stream object, or its bare hipStream_t handle as an int (on ROCm `cuda_stream` is that handle)
+                assert isinstance(arg, (torch.cuda.Stream, int)), f'Expected a stream for `{name}`, got `{type(arg)}`'
+                cargs.append(arg if isinstance(arg, int) else arg.cuda_stream)
             else:
                 assert isinstance(arg, dtype), f'Expected built-in type `{dtype}` for `{name}`, got `{type(arg)}`'
-                cargs.append(arg.cuda_stream if dtype is torch.cuda.Stream else arg)     # on ROCm the hipStream_t handle
+                cargs.append(arg)
         rc = ctypes.c_int(0)
         self._launch(*cargs, rc)
         return rc.value

@@ -15,7 +15,7 @@ import torch
 from .heuristics import (get_best_dense_config, get_dense_num_stages, get_dense_tile_space, get_skinny_dense_config,
                          get_split_k_dense_config, tuning_enabled)
 from .tuner import FrozenKeys, jit_tuner
-from .utils import get_num_sms, get_num_sms_cap
+from .utils import current_raw_stream, get_num_sms, get_num_sms_cap
 
 includes = ('"gemm/bf16_gemm.hpp"', )
 template = """
@@ -95,7 +95,7 @@ def _gemm_16bit_tn(a: torch.Tensor, b: torch.Tensor, c: torch.Tensor, dtype: tor
     if m == 0 or n == 0:
         return
 
-    stream = torch.cuda.current_stream()
+    stream = current_raw_stream()
     args = (m, n, k, a, b, c, stream)
     code_template = template
     if tuning_enabled() and not get_skinny_dense_config(m, n, k, get_num_sms()):

@@ -14,7 +14,7 @@ from typing import Tuple
 import torch
 
 from .tuner import FrozenKeys, jit_tuner
-from .utils import ceil_div
+from .utils import ceil_div, current_raw_stream
 
 includes = ('"gemm/fp8_cast.hpp"', )
 
@@ -70,7 +70,7 @@ def per_token_cast_to_fp8(x: torch.Tensor, col_major_scales: bool = False) -> Tu
     if m == 0 or k == 0:
         return q, scales
     name, keys, arg_defs, template = cast_kernel_plan('per_token', x.dtype)
-    args = (x, q, scales, scales.stride(0), scales.stride(1), m, k, torch.cuda.current_stream())
+    args = (x, q, scales, scales.stride(0), scales.stride(1), m, k, current_raw_stream())
     runtime = jit_tuner.compile_and_tune(name=name, keys=keys, space=(), includes=includes, arg_defs=arg_defs,
                                          template=template, args=args)
     rc = runtime(*args)
@@ -88,7 +88,7 @@ def per_block_cast_to_fp8(w: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
     if n == 0 or k == 0:
         return q, scales
     name, keys, arg_defs, template = cast_kernel_plan('per_block', w.dtype)
-    args = (w, q, scales, n, k, torch.cuda.current_stream())
+    args = (w, q, scales, n, k, current_raw_stream())
     runtime = jit_tuner.compile_and_tune(name=name, keys=keys, space=(), includes=includes, arg_defs=arg_defs,
                                          template=template, args=args)
     rc = runtime(*args)

@@ -18,7 +18,7 @@ import torch
 from .heuristics import (get_best_fp8_config, get_fp8_num_stages, get_fp8_tile_space, get_skinny_fp8_config,
                          get_split_k_fp8_config, tuning_enabled)
 from .tuner import FrozenKeys, jit_tuner
-from .utils import get_num_sms, ceil_div, get_col_major_tensor
+from .utils import current_raw_stream, get_num_sms, ceil_div, get_col_major_tensor
 
 # C++ code templates
 includes = ('"gemm/fp8_gemm.hpp"', '"gemm/fp8_gemm_skinny.hpp"')
@@ -91,11 +91,11 @@ SPLIT_K_WORKSPACE_BYTES = SPLIT_K_COUNTER_BYTES + 256 * 128 * 128 * 4
 _split_k_workspaces = {}
 
 
-def split_k_workspace(device: torch.device, stream: torch.cuda.Stream) -> torch.Tensor:
-    """The workspace split-K launches on `stream` share: one per device and stream, made (and zeroed, on the current
-    stream) at the first call and kept. Launches on one stream run one after the other, which is what sharing needs; the
+def split_k_workspace(device: torch.device, stream) -> torch.Tensor:
+    """The workspace split-K launches on `stream` (a Stream or its bare handle) share: one per device and stream, made (and
+    zeroed, on the current stream) at the first call and kept. Launches on one stream run one after the other, which is what sharing needs; the
     counters at its start are zero again after every launch."""
-    key = (device.index, stream.cuda_stream)
+    key = (device.index, stream if isinstance(stream, int) else stream.cuda_stream)
     workspace = _split_k_workspaces.get(key)
     if workspace is None:
         workspace = torch.zeros(SPLIT_K_WORKSPACE_BYTES, dtype=torch.uint8, device=device)
@@ -184,7 +184,7 @@ def gemm_fp8_fp8_bf16_nt(lhs: Tuple[torch.Tensor, torch.Tensor],
     stride_m, stride_k = lhs_scales.stride()
     token_contiguous = (m == 1 or stride_m == 1) and (lhs_scales.size(1) == 1 or stride_k == m)
     name, keys, defs, smem_size, code_template = fp8_kernel_plan(m, n, k, num_sms, token_contiguous)
-    stream = torch.cuda.current_stream()
+    stream = current_raw_stream()
     args = (lhs, lhs_scales, rhs, rhs_scales, out, m, stream, num_sms, smem_size)
     space = ()
     if tuning_enabled():

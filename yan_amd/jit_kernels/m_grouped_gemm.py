@@ -15,7 +15,7 @@ import torch
 from .gemm import includes
 from .heuristics import get_best_grouped_fp8_config, get_fp8_num_stages
 from .tuner import FrozenKeys, jit_tuner
-from .utils import ceil_div, get_m_alignment_for_contiguous_layout, get_num_sms
+from .utils import ceil_div, current_raw_stream, get_m_alignment_for_contiguous_layout, get_num_sms
 
 template = """
 using namespace yan;
@@ -65,7 +65,7 @@ def _launch(gemm_type, num_groups, plan_m, m, n, k, lhs, lhs_scales, rhs, rhs_sc
     # `strides`: the three strides of the activation scales, then expected_m (masked layout; 0 otherwise)
     num_sms = get_num_sms()
     name, keys, defs, smem_size = grouped_kernel_plan(gemm_type, num_groups, plan_m, n, k, num_sms)
-    args = (lhs, lhs_scales, rhs, rhs_scales, out, layout, m, torch.cuda.current_stream(), num_sms, smem_size, *strides)
+    args = (lhs, lhs_scales, rhs, rhs_scales, out, layout, m, current_raw_stream(), num_sms, smem_size, *strides)
     runtime = jit_tuner.compile_and_tune(name=name, keys=keys, space=(), includes=includes,
                                          arg_defs=defs, template=template, args=args)
     rc = runtime(*args)

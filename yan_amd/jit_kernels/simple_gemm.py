@@ -13,7 +13,7 @@ import torch
 
 from .heuristics import get_best_float_config
 from .tuner import FrozenKeys, jit_tuner
-from .utils import get_num_sms
+from .utils import current_raw_stream, get_num_sms
 
 includes = ('"gemm/simple_gemm.hpp"', )
 template = """
@@ -71,7 +71,7 @@ def gemm_float_nt(a: torch.Tensor, b: torch.Tensor, c: torch.Tensor,
         return
 
     ldA, ldB, ldC = _leading_dim(a), _leading_dim(b), n
-    stream = torch.cuda.current_stream()
+    stream = current_raw_stream()
     args = (m, n, k, float(alpha), a, ldA, b, ldB, float(beta), c, ldC, stream)
     name, keys, defs = float_kernel_plan(m, n, get_num_sms())
     runtime = jit_tuner.compile_and_tune(name=name, keys=keys, space=(), includes=includes,

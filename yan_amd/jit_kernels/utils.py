@@ -5,10 +5,25 @@
 import torch
 
 _num_sms = None
+_cu_count = None
 
 
 def _device_cu_count() -> int:
-    return torch.cuda.get_device_properties(device='cuda').multi_processor_count
+    # asked once: the query costs several microseconds, as much as the host side of a whole GEMM call
+    global _cu_count
+    if _cu_count is None:
+        _cu_count = torch.cuda.get_device_properties(device='cuda').multi_processor_count
+    return _cu_count
+
+
+def current_raw_stream() -> int:
+    """The hipStream_t handle of the current stream of the current device as an int. `torch.cuda.current_stream()` builds
+    a Stream object around it and costs 3-4 us per call, a third of the host side of a decode-shape GEMM; the JIT
+    runtime takes the bare handle wherever an argument is declared a `torch.cuda.Stream`."""
+    try:
+        return torch._C._cuda_getCurrentRawStream(torch.cuda.current_device())
+    except AttributeError:          # a torch without the raw accessor
+        return torch.cuda.current_stream().cuda_stream
 
 
 def set_num_sms(num_sms: int) -> None:
