@@ -94,7 +94,8 @@ def test_dense_split_k_plans():
     plan = heuristics.get_split_k_dense_config
     assert plan(64, 4096, 7168, 256) == (64, 64, 4) and plan(256, 7168, 16384, 256) == (128, 128, 2)
     assert plan(256, 7168, 2048, 256) is None and plan(256, 24576, 1536, 256) is None and plan(8192, 8192, 8192, 256) is None
-    assert plan(16, 4096, 7168, 256) is None and plan(17, 4096, 7168, 256) == (64, 64, 4)   # up to 16 rows: the weight-streaming kernel's
+    assert plan(7, 4096, 7168, 256) is None and plan(16, 4096, 16384, 256) is None          # the one-atom weight-streaming kernel's
+    assert plan(8, 4096, 7168, 256) == (64, 64, 4) and plan(17, 4096, 16384, 256) == (64, 64, 4)
     for shape, expected in harness.DENSE_SPLIT_K_PLAN_OF_SHAPE.items():
         assert plan(*shape, 256) == expected, shape
     assert {(bm, bn) for bm, bn, _ in harness.DENSE_SPLIT_K_PLAN_OF_SHAPE.values()} == set(heuristics._DENSE_SPLIT_K_EXTRA_US)

@@ -99,7 +99,7 @@ constexpr DenseSplitKTile kDenseSplitKTiles[] = {{64, 64, 0.248, 0.0}, {64, 128,
 int dense_skinny_atoms(int m, int n, int k, int num_cus);
 
 bool pick_dense_split_k(int m, int n, int k, int num_cus, int* bm, int* bn, int* split_k) {
-    if (m <= 0 || n <= 0 || k <= 0 || (m <= 16 && dense_skinny_atoms(m, n, k, num_cus))) return false;
+    if (m <= 0 || n <= 0 || k <= 0 || ((m < 8 || (m <= 16 && k > 8192)) && dense_skinny_atoms(m, n, k, num_cus))) return false;
     const int k_tiles = (k + 63) / 64;
     int ubm = 0, ubn = 0;
     pick(kDenseTiles, m, n, num_cus, &ubm, &ubn);
@@ -151,8 +151,8 @@ int dense(int m, int n, int k, const void* a, const void* b, void* c, void* stre
     if (m < 0 || n < 0) return int(hipErrorInvalidValue);
     hipStream_t s = static_cast<hipStream_t>(stream);
     int bm = 0, bn = 0, split_k = 1;
-    // a split-K plan goes before the two-atom weight-streaming kernel (pick_dense_split_k makes none up to 16 rows where the
-    // one-atom kernel runs)
+    // a split-K plan goes before the weight-streaming kernels (pick_dense_split_k makes none where the one-atom kernel is the
+    // faster: below 8 rows, and up to 16 rows on K beyond 8192)
     if (workspace && pick_dense_split_k(m, n, k, device_cus(), &bm, &bn, &split_k)) {
 #define YAN_DENSE_SPLIT_K_CASE(BM, BN, S) \
     if (bm == BM && bn == BN && split_k == S) return int(yan::launch_dense_split_k<Atom, Elem, BM, BN, S>(m, n, k, a, b, c, s, workspace, workspace_bytes));

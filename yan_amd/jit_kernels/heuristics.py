@@ -213,9 +213,11 @@ def get_split_k_dense_config(m: int, n: int, k: int, num_cus: int) -> Optional[T
     `pick_dense_split_k` in yan_amd/csrc/yan_gemm_capi.hip (a CPU test keeps the two in step). A plan goes before the
     two-atom weight-streaming kernel (17 to 32 rows; n = 4096, k = 7168: 21.1 - 25.2 us against 14.8 - 14.9 for 64 x 64 tiles
     in four parts), which therefore runs only where no plan exists or no workspace is at hand (the C library's plain entry
-    points); up to 16 rows the one-atom kernel stays (14.5 - 18.2 us against 14.7 - 14.8, and ahead on longer K)."""
-    if m <= 0 or n <= 0 or k <= 0 or (m <= 16 and get_skinny_dense_config(m, n, k, num_cus)):
-        return None         # up to 16 rows the weight-streaming kernel is as fast or faster; from 17 rows a plan goes first
+    points), and before the one-atom kernel from 8 rows on K up to 8192 (m = 8: 15.8 against 14.7 us, m = 16: 18.2 against 14.8;
+    n = 2048: 15.0 / 17.5 against 12.3 / 12.4); below 8 rows and on longer K that kernel stays (m = 1: 14.5 against 14.7;
+    k = 16384, m = 8: 28.9 against 31.0)."""
+    if m <= 0 or n <= 0 or k <= 0 or ((m < 8 or (m <= 16 and k > 8192)) and get_skinny_dense_config(m, n, k, num_cus)):
+        return None         # a handful of rows, or up to 16 on a long K: the one-atom weight-streaming kernel is as fast or faster
     k_tiles = ceil_div(k, 64)
     unsplit = get_best_dense_config(m, n, k, num_cus)
     if unsplit not in _DENSE_SPLIT_K_TILE_US or ceil_div(m, unsplit[0]) * ceil_div(n, unsplit[1]) > num_cus:
