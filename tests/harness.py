@@ -209,9 +209,9 @@ FP8_SPLIT_K_PLAN_OF_SHAPE = {
     (100, 2112, 5376): (64, 64, 3), (65, 1536, 7168): (64, 64, 4),
     (200, 3076, 3584): (64, 128, 2), (100, 4100, 5376): (64, 128, 3), (129, 2112, 7168): (64, 128, 4),
     (300, 4100, 4608): (128, 128, 2), (200, 4100, 5376): (128, 128, 3), (129, 4096, 7168): (128, 128, 4),
-    (64, 4096, 7168): (64, 64, 4), (128, 4096, 7168): (64, 128, 4),
+    (64, 4096, 7168): (64, 64, 4), (128, 4096, 7168): (64, 128, 4), (5, 2052, 3712): (32, 32, 2), (1, 4096, 7168): (32, 32, 2),
 }
-FP8_SPLIT_K_SHAPES = [s for s in FP8_SPLIT_K_PLAN_OF_SHAPE if s not in ((64, 4096, 7168), (128, 4096, 7168))]
+FP8_SPLIT_K_SHAPES = [s for s in FP8_SPLIT_K_PLAN_OF_SHAPE if s not in ((64, 4096, 7168), (128, 4096, 7168), (1, 4096, 7168))]
 # The same for the dense GEMMs: the three tiles split-K plans use, every factor, ragged m and n, n that is no multiple of 8,
 # a k tail (3080 = 48 k-tiles and 8 elements), a dozen rows (where a plan goes before the weight-streaming kernel).
 DENSE_SPLIT_K_PLAN_OF_SHAPE = {

@@ -61,7 +61,8 @@ def test_split_k_plans():
     assert plan(256, 7168, 7168, 256) == (128, 128, 2) and plan(128, 7168, 16384, 256) == (128, 128, 4)
     # short K, a weight matrix that takes as long to stream as to multiply, work for every compute unit, few rows
     assert plan(64, 7168, 2048, 256) is None and plan(64, 16384, 7168, 256) is None and plan(4096, 7168, 7168, 256) is None
-    assert plan(16, 4096, 7168, 256) is None and plan(0, 4096, 7168, 256) is None
+    assert plan(16, 4096, 2048, 256) is None and plan(0, 4096, 7168, 256) is None
+    assert plan(16, 4096, 7168, 256) == (32, 32, 2) and plan(1, 2112, 7168, 256) == (32, 32, 3)      # before the weight-streaming kernel
     for shape, expected in harness.FP8_SPLIT_K_PLAN_OF_SHAPE.items():
         assert plan(*shape, 256) == expected, shape
     assert {(bm, bn) for bm, bn, _ in harness.FP8_SPLIT_K_PLAN_OF_SHAPE.values()} == set(heuristics._FP8_SPLIT_K_TILE_US)

@@ -66,7 +66,7 @@ constexpr SplitKTile kSplitKTiles[] = {{32, 32, 0.133}, {64, 32, 0.192}, {64, 64
 constexpr int kSplitKFactors[] = {2, 3, 4};
 
 bool pick_split_k(int m, int n, int k, int num_cus, int* bm, int* bn, int* split_k) {
-    if (m <= 0 || n <= 0 || k <= 0 || skinny_atoms(m, n, num_cus)) return false;
+    if (m <= 0 || n <= 0 || k <= 0) return false;
     const int k_tiles = k / 128;
     int ubm = 0, ubn = 0;
     pick(kFp8Tiles, m, n, num_cus, &ubm, &ubn);
@@ -205,10 +205,8 @@ int fp8_plain(const void* lhs, const float* lhs_scales, long long lhs_scales_str
     const int cus = (num_sms > 0 && num_sms < device_cus()) ? num_sms : device_cus();
     hipStream_t s = static_cast<hipStream_t>(stream);
     __hip_bfloat16* o = static_cast<__hip_bfloat16*>(out);
-    if (skinny_atoms(m, n, cus))
-        return int(yan::launch_fp8_skinny<0, 0, 1, 8>(o, lhs, lhs_scales, int(lhs_scales_stride_m), int(lhs_scales_stride_k), rhs,
-                                                      rhs_scales, m, n, k, s));
     int bm = 0, bn = 0, split_k = 1;
+    // a split-K plan goes before the weight-streaming kernel
     if (workspace && pick_split_k(m, n, k, cus, &bm, &bn, &split_k)) {
 #define YAN_SPLIT_K_CASE(BM, BN, S)                                                                                  \
     if (bm == BM && bn == BN && split_k == S)                                                                        \
@@ -220,6 +218,9 @@ int fp8_plain(const void* lhs, const float* lhs_scales, long long lhs_scales_str
 #undef YAN_SPLIT_K_CASE
         return int(hipErrorInvalidValue);
     }
+    if (skinny_atoms(m, n, cus))
+        return int(yan::launch_fp8_skinny<0, 0, 1, 8>(o, lhs, lhs_scales, int(lhs_scales_stride_m), int(lhs_scales_stride_k), rhs,
+                                                      rhs_scales, m, n, k, s));
     pick(kFp8Tiles, m, n, cus, &bm, &bn);
 #define YAN_FP8_CASE(BM, BN)                                                                                         \
     if (bm == BM && bn == BN)                                                                                        \

@@ -165,8 +165,11 @@ def get_split_k_fp8_config(m: int, n: int, k: int, num_cus: int) -> Optional[Tup
     k = 1536..16384) swept with every tile and factor, weights cycling through more matrices than the caches hold, the
     plan taken is the fastest measured or within 1 % of it wherever one is taken: 13 to 38 % faster than unsplit
     (64 x 4096 x 7168: 64 x 64 tiles in four parts; 32 x 2112 x 7168: 32 x 32 in three); k = 2048 and n = 16384 or more
-    stay unsplit. Same rule as `pick_split_k` in yan_amd/csrc/yan_gemm_capi.hip (a CPU test keeps the two in step)."""
-    if get_skinny_fp8_config(m, n, k, num_cus) or m <= 0 or n <= 0:
+    stay unsplit. A plan also goes before the weight-streaming kernel of up to 16 rows (32 x 32 tiles in two to four parts
+    against that kernel, m = 1..16: n = 4096, k = 7168: 9.7 - 9.8 against 10.7 - 12.2 us; n = 2048: 8.4 against 10.1 - 11.8; level
+    at k = 4096 and at k = 16384 below 8 rows), which runs where no plan exists or no workspace is at hand. Same rule as
+    `pick_split_k` in yan_amd/csrc/yan_gemm_capi.hip (a CPU test keeps the two in step)."""
+    if m <= 0 or n <= 0:
         return None
     k_tiles = k // 128
     unsplit = get_best_fp8_config(m, n, k, num_cus)
