@@ -6,7 +6,8 @@
 //     (reference: yan/include/gemm/scheduler.cuh:39-41, num_blocks = ceil(m/BLOCK_M) * ceil(N/BLOCK_N));
 //   * under every compute-unit cap, the walk b, b + grid, b + 2 grid, ... of capped_grid() workgroups covers every slot
 //     exactly once and, for grids that are multiples of 8, never leaves the XCD residue b % 8;
-//   * the masked layout's slot numbering (MaskedSlots) visits every (group, tile) once, likely tile rows first;
+//   * the masked layout's slot numbering (MaskedSlots) visits every (group, tile) once, likely tile rows first, and bands
+//     fitted to the height of a group lose no tile and keep a patch inside one group;
 //   * the same holds in region order (operand rows long enough that the problem outgrows the memory-side cache), whose
 //     choice of region is pinned for a few measured shapes.
 #include "gemm/scheduler.hpp"
@@ -71,6 +72,28 @@ int main() {
                 }
             }
     }
+    // bands fitted to the tile-rows of a group (grouped layouts): still every tile exactly once, and with aligned groups the
+    // 32 consecutive tiles of a patch stay inside one group
+    for (int rows_per_group : {1, 2, 3, 4, 5, 8, 11})
+        for (int groups : {1, 4, 9})
+            for (int tn : {1, 7, 16, 40}) {
+                const int bm = 256, bn = 256, tm = rows_per_group * groups, m = tm * bm, n = (tn - 1) * bn + 1;
+                yan::XcdTileScheduler<> sched(m, n, bm, bn);
+                sched.fit_bands_to_groups(rows_per_group);
+                CHECK(sched.band_height == (rows_per_group < 8 ? rows_per_group : 8));
+                std::vector<int> seen(size_t(tm) * tn, 0);
+                for (int bid = 0; bid < sched.grid_size(); ++bid) {
+                    const yan::TileCoord t = sched.tile_of(bid);
+                    if (t.valid) { CHECK(t.m_idx >= 0 && t.m_idx < tm && t.n_idx >= 0 && t.n_idx < tn); ++seen[size_t(t.m_idx) * tn + t.n_idx]; }
+                }
+                for (int v : seen) CHECK(v == 1);
+                if (rows_per_group <= 8 && 32 % rows_per_group == 0 && tn % (32 / rows_per_group) == 0)
+                    for (int t0 = 0; t0 + 32 <= sched.total; t0 += 32) {
+                        const int g0 = sched.band_tile(t0).m_idx / rows_per_group;
+                        for (int t = t0; t < t0 + 32; ++t) CHECK(sched.band_tile(t).m_idx / rows_per_group == g0);
+                    }
+                ++cases;
+            }
     // the masked layout's slot numbering: every (group, tile) exactly once, the tile rows below expected_m before the others
     for (int groups : {1, 3, 8, 17})
         for (int tm = 1; tm <= 9; tm += (tm < 3 ? 1 : 3))

@@ -293,7 +293,9 @@ fp8_gemm_tile(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_sca
     [[maybe_unused]] const int tile_slot = bid;
 
     // a plain GEMM whose operands outgrow the memory-side cache walks its tiles in region order (scheduler.hpp)
-    const XcdTileScheduler<> sched(m, N, BLOCK_M, BLOCK_N, kGemmType == GemmType::Normal ? (long long)K : 0);
+    XcdTileScheduler<> sched(m, N, BLOCK_M, BLOCK_N, kGemmType == GemmType::Normal ? (long long)K : 0);
+    // contiguous groups of equal size start on band boundaries when the bands are as tall as a group (or divide one)
+    if constexpr (kGemmType == GemmType::GroupedContiguous) sched.fit_bands_to_groups(sched.tiles_m / max(num_groups, 1));
     TileCoord tile;
     if constexpr (kGemmType == GemmType::GroupedMasked) {
         int group;

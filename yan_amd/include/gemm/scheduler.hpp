@@ -39,6 +39,7 @@ struct XcdTileScheduler {
     static constexpr long long kCacheBytes = 256ll << 20;
 
     int  tiles_m, tiles_n, total, per_xcd;
+    int  band_height;                     // tile-rows of a band: GROUP_M, or fewer when the caller's groups hold fewer (below)
     int  region_rows, region_cols;        // 0: band order
     bool rows_outer;                      // region order: all column blocks of a row block before the next row block
 
@@ -47,6 +48,7 @@ struct XcdTileScheduler {
         tiles_n = ceil_div(n, block_n);
         total   = tiles_m * tiles_n;
         per_xcd = ceil_div(total, kNumXCD);
+        band_height = GROUP_M;
         region_rows = region_cols = 0;
         rows_outer = true;
         const long long panel_a = row_bytes * block_m, panel_b = row_bytes * block_n;
@@ -80,11 +82,19 @@ struct XcdTileScheduler {
         return band_tile(t);
     }
 
+    // Grouped layouts: the rows are `groups` stacked problems with their own weights. Bands no taller than a group keep the
+    // 32 consecutive tiles an XCD runs at once inside one group where groups are aligned: h x (32 / h) tiles share h
+    // activation panels and 32 / h weight panels of one group, instead of 8 and 4 per group touched (4 groups of 4 tile-rows:
+    // 12 panels instead of 16).
+    __host__ __device__ void fit_bands_to_groups(int tile_rows_per_group) {
+        band_height = tile_rows_per_group < 1 ? 1 : (tile_rows_per_group < GROUP_M ? tile_rows_per_group : GROUP_M);
+    }
+
     // Tile number t of the band-order sequence.
     __host__ __device__ TileCoord band_tile(int t) const {
-        const int band      = GROUP_M * tiles_n;
-        const int first_m   = (t / band) * GROUP_M;
-        const int band_rows = (tiles_m - first_m) < GROUP_M ? (tiles_m - first_m) : GROUP_M;
+        const int band      = band_height * tiles_n;
+        const int first_m   = (t / band) * band_height;
+        const int band_rows = (tiles_m - first_m) < band_height ? (tiles_m - first_m) : band_height;
         const int in_band   = t % band;
         return {first_m + in_band % band_rows, in_band / band_rows, true};
     }
@@ -143,8 +153,8 @@ struct XcdTileScheduler {
 
 // Slot numbering of the masked layout. Only the first masked_m[g] rows of a group exist, and the caller's `expected_m`
 // says how many that usually is: the tile rows below it come first, all groups' stacked along m into one grid whose
-// patches of 8 x 4 tiles are dealt out to the XCDs in turn (the 32 tiles an XCD runs at once lie in one or two groups and
-// share weight panels through its L2; consecutive patches go to different XCDs, so a group with few rows or none does not
+// patches of 32 tiles (8 x 4, or as tall as a group where groups hold fewer tile-rows) are dealt out to the XCDs in turn (the
+// 32 tiles an XCD runs at once share weight panels through its L2; consecutive patches go to different XCDs, so a group with few rows or none does not
 // leave one XCD idle), the tile rows above it afterwards in a second grid of the same kind. A workgroup whose tile does not exist leaves at once, but
 // it still takes a compute unit to start: numbered group by group, existing and empty tiles alternate and the existing
 // ones start in ever smaller waves as the empty ones get out of their way (8 groups x 128 rows of which 64 exist: 58 us
@@ -160,6 +170,8 @@ struct MaskedSlots {
         likely_rows = likely_rows < tiles_m ? likely_rows : tiles_m;
         likely = XcdTileScheduler<>(num_groups * likely_rows * block_m, n, block_m, block_n);
         rest   = XcdTileScheduler<>(num_groups * (tiles_m - likely_rows) * block_m, n, block_m, block_n);
+        likely.fit_bands_to_groups(likely_rows);
+        rest.fit_bands_to_groups(tiles_m - likely_rows);
         likely_slots = likely.grid_size();
     }
 
