@@ -325,10 +325,13 @@ fp8_gemm_tile(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_sca
             if (g0 < 0) return;
             pass_group[0] = g0;
         } else {
-            num_passes = 0;
-            if (g0 >= 0) { pass_group[0] = g0; pass_hi[0] = m0 + 128; num_passes = 1; }
-            if (g1 >= 0) { pass_group[num_passes] = g1; pass_lo[num_passes] = m0 + 128; ++num_passes; }
-            if (num_passes == 0) return;
+            // constant indices only: an index computed at run time would put these arrays into scratch memory
+            const bool first = g0 >= 0, second = g1 >= 0;
+            if (!first && !second) return;
+            if (first) { pass_group[0] = g0; pass_hi[0] = m0 + 128; }
+            if (second && first)  { pass_group[1] = g1; pass_lo[1] = m0 + 128; }
+            if (second && !first) { pass_group[0] = g1; pass_lo[0] = m0 + 128; }
+            num_passes = int(first) + int(second);
         }
     }
     const uint8_t* const rhs_all = rhs;
@@ -417,7 +420,12 @@ fp8_gemm_tile(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_sca
     constexpr bool kStagedEpilogue = Cfg::WTN >= 32;
     [[maybe_unused]] uint8_t* epi_a = nullptr;
     [[maybe_unused]] uint8_t* epi_b = nullptr;
-    for (int pass = 0; pass < (kGemmType == GemmType::GroupedContiguous ? num_passes : 1); ++pass) {
+    // The second pass is a copy of the code, not a trip round a loop: as a loop with a run-time count even a single pass ran
+    // 10 % slower (the compiler keeps less of the main loop's state where it was).
+    constexpr int kMaxPasses = kTwoHalves ? 2 : 1;
+#pragma unroll
+    for (int pass = 0; pass < kMaxPasses; ++pass) {
+    if (kTwoHalves && pass >= num_passes) break;
     if constexpr (kGemmType == GemmType::GroupedContiguous) {
         rhs        = rhs_all + size_t(pass_group[pass]) * N * K;
         rhs_scales = rhs_scales_all + size_t(pass_group[pass]) * NUM_N_BLOCKS * NUM_K_BLOCKS;
