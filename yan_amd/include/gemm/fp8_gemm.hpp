@@ -829,6 +829,14 @@ fp8_gemm_kernel(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_s
             return;
         }
     }
+    // A workgroup per slot (no cap): the tile without a loop around it. Inside the loop below the same code runs 2 to 14 %
+    // slower on the ring tiles even for a single trip (64 x 7168 x 2048 on 64 x 32 tiles: 6.0 against 5.2 us).
+    if (int(gridDim.x) >= num_slots) {
+        fp8_gemm_tile<SHAPE_N, SHAPE_K, BLOCK_M, BLOCK_N, kGemmType, STAGES>(lhs, lhs_scales, rhs, rhs_scales, out, m, n_rt, k_rt,
+                                                                             sa_stride_m, sa_stride_k, grouped_layout, sa_stride_g,
+                                                                             int(blockIdx.x), num_groups, expected_m, two_stages);
+        return;
+    }
     for (int slot = blockIdx.x; slot < num_slots; slot += gridDim.x) {
         fp8_gemm_tile<SHAPE_N, SHAPE_K, BLOCK_M, BLOCK_N, kGemmType, STAGES>(lhs, lhs_scales, rhs, rhs_scales, out, m, n_rt, k_rt,
                                                                              sa_stride_m, sa_stride_k, grouped_layout, sa_stride_g,
