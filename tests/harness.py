@@ -202,14 +202,14 @@ FP8_SIDE_SHAPES = [(1024, 4096, 7168), (8192, 4096, 7168), (200, 384, 512), (115
                    (256, 200, 128), (256, 512, 512)]
 # Problems the split-K plan covers on 256 compute units, with the (BLOCK_M, BLOCK_N, SPLIT_K) it makes (a CPU test keeps this
 # true): every ring tile, every factor, ragged m and n, n that is no multiple of 8 (direct stores), K ranges of unequal
-# length (29 k-tiles in 2 parts, 43 and 56 in 3).
+# length (49 k-tiles in 2 parts, 43 and 56 in 3).
 FP8_SPLIT_K_PLAN_OF_SHAPE = {
-    (17, 196, 3584): (32, 32, 2), (33, 196, 5504): (32, 32, 3), (64, 196, 7168): (32, 32, 4), (31, 516, 3712): (32, 32, 2),
+    (17, 3076, 6272): (32, 32, 2), (33, 196, 5504): (32, 32, 3), (64, 196, 7168): (32, 32, 4), (31, 3588, 6272): (32, 32, 2),
     (33, 2112, 5376): (64, 32, 3), (50, 1536, 7168): (64, 32, 4), (64, 2112, 7168): (64, 32, 3),
     (100, 2112, 5376): (64, 64, 3), (65, 1536, 7168): (64, 64, 4),
-    (200, 3076, 3584): (64, 128, 2), (100, 4100, 5376): (64, 128, 3), (129, 2112, 7168): (64, 128, 4),
-    (300, 4100, 4608): (128, 128, 2), (200, 4100, 5376): (128, 128, 3), (129, 4096, 7168): (128, 128, 4),
-    (64, 4096, 7168): (64, 64, 4), (128, 4096, 7168): (64, 128, 4), (5, 2052, 3712): (32, 32, 2), (1, 4096, 7168): (32, 32, 2),
+    (200, 3076, 6144): (64, 128, 2), (100, 4100, 5376): (64, 128, 3), (129, 2112, 7168): (64, 128, 4),
+    (300, 4100, 6144): (128, 128, 2), (200, 4100, 5376): (128, 128, 3), (129, 4096, 7168): (128, 128, 4),
+    (64, 4096, 7168): (64, 64, 4), (128, 4096, 7168): (64, 128, 4), (5, 3076, 6144): (32, 32, 2), (1, 4096, 7168): (32, 32, 2),
 }
 FP8_SPLIT_K_SHAPES = [s for s in FP8_SPLIT_K_PLAN_OF_SHAPE if s not in ((64, 4096, 7168), (128, 4096, 7168), (1, 4096, 7168))]
 # The same for the dense GEMMs: the three tiles split-K plans use, every factor, ragged m and n, n that is no multiple of 8,

@@ -53,7 +53,7 @@ def test_tile_heuristics_fill_256_cus():
 
 def test_split_k_plans():
     """K is split when the unsplit tiles leave the chip short of work and K is long; every plan fits one round of
-    workgroups and the workspace, leaves each part 14 k-tiles or more, and the shapes of the GPU suite get the plans the
+    workgroups and the workspace, leaves each part 14 k-tiles or more (24 of two), and the shapes of the GPU suite get the plans the
     suite expects (every ring tile, every factor)."""
     import harness
     plan = heuristics.get_split_k_fp8_config
@@ -76,7 +76,7 @@ def test_split_k_plans():
                         continue
                     bm, bn, split = p
                     slots = yan.ceil_div(yan.ceil_div(m, bm) * yan.ceil_div(n, bn), 8) * 8
-                    assert slots * split <= cus and yan.ceil_div(k // 128, split) >= 14
+                    assert slots * split <= cus and yan.ceil_div(k // 128, split) >= (24 if split == 2 else 14)
                     assert gemm.SPLIT_K_COUNTER_BYTES + slots * split * bm * bn * 4 <= gemm.SPLIT_K_WORKSPACE_BYTES
                     assert slots * 8 * 4 <= gemm.SPLIT_K_COUNTER_BYTES
                     assert heuristics.get_fp8_num_stages(bm, bn) > 2          # a ring tile

@@ -61,8 +61,9 @@ int skinny_atoms(int m, int n, int num_cus) {
 }
 
 // Split-K plan of the plain FP8 GEMM (get_split_k_fp8_config in heuristics.py): false when K is not split.
-struct SplitKTile { int bm, bn; double us_per_k_tile; };
-constexpr SplitKTile kSplitKTiles[] = {{32, 32, 0.133}, {64, 32, 0.192}, {64, 64, 0.296}, {64, 128, 0.395}, {128, 128, 0.51}};
+struct SplitKTile { int bm, bn; double us_per_k_tile, unsplit_us_per_k_tile; };
+constexpr SplitKTile kSplitKTiles[] = {{32, 32, 0.133, 0.117}, {64, 32, 0.192, 0.169}, {64, 64, 0.296, 0.275}, {64, 128, 0.395, 0.375},
+                                       {128, 128, 0.51, 0.497}};
 constexpr int kSplitKFactors[] = {2, 3, 4};
 
 bool pick_split_k(int m, int n, int k, int num_cus, int* bm, int* bn, int* split_k) {
@@ -72,7 +73,7 @@ bool pick_split_k(int m, int n, int k, int num_cus, int* bm, int* bn, int* split
     pick(kFp8Tiles, m, n, num_cus, &ubm, &ubn);
     double unsplit_us = -1;
     for (const SplitKTile& t : kSplitKTiles)
-        if (t.bm == ubm && t.bn == ubn) unsplit_us = t.us_per_k_tile;
+        if (t.bm == ubm && t.bn == ubn) unsplit_us = t.unsplit_us_per_k_tile;
     if (unsplit_us < 0 || (long long)((m + ubm - 1) / ubm) * ((n + ubn - 1) / ubn) > num_cus) return false;
     const double floor = double((long long)n * k) / 6.0e6;
     const double unsplit_time = k_tiles * unsplit_us;
@@ -83,7 +84,7 @@ bool pick_split_k(int m, int n, int k, int num_cus, int* bm, int* bn, int* split
         const long long tiles = (long long)((m + t.bm - 1) / t.bm) * ((n + t.bn - 1) / t.bn);
         for (const int s : kSplitKFactors) {
             const int per_part = (k_tiles + s - 1) / s;
-            if ((tiles + 7) / 8 * 8 * s > (num_cus < 256 ? num_cus : 256) || per_part < 14) continue;
+            if ((tiles + 7) / 8 * 8 * s > (num_cus < 256 ? num_cus : 256) || per_part < (s == 2 ? 24 : 14)) continue;
             const double loop = per_part * t.us_per_k_tile + 0.5 + double(s * t.bm * t.bn * 4) / 1024 * 0.0125;
             const double time = loop > floor ? loop : floor;
             if (best < 0 || time < best) { best = time; *bm = t.bm; *bn = t.bn; *split_k = s; }

@@ -149,6 +149,9 @@ def get_fp8_tile(m: int, n: int, k: int, num_cus: int) -> Tuple[int, int]:
 # (measured: m x 4096 x 7168, sizes at run time, 56 k-tiles, one round of workgroups). Only used to weigh split-K plans
 # against the unsplit pick of the cost table above.
 _FP8_SPLIT_K_TILE_US = {(32, 32): 0.133, (64, 32): 0.192, (64, 64): 0.296, (64, 128): 0.395, (128, 128): 0.51}
+# The same for the unsplit kernel, which pulls its weights with fewer workgroups at a time and, a workgroup per tile, runs
+# without a loop around the tile: 0.88 to 0.975 of the figures above.
+_FP8_UNSPLIT_TILE_US = {(32, 32): 0.117, (64, 32): 0.169, (64, 64): 0.275, (64, 128): 0.375, (128, 128): 0.497}
 FP8_SPLIT_K_FACTORS = (2, 3, 4)
 
 
@@ -160,12 +163,12 @@ def get_split_k_fp8_config(m: int, n: int, k: int, num_cus: int) -> Optional[Tup
     a larger tile on as many workgroups pulls fewer bytes per output; the price is a round trip of the partial sums
     through memory, paid by the part that arrives last. Modelled time of a plan: k-tiles per part x the tile's time per
     k-tile + 0.5 us + 12.5 ns per KB of partial sums the last part reads, never less than streaming the weights at 6 TB/s.
-    A plan is taken when it fits one round (tile slots x SPLIT_K <= num_cus), leaves every part at least 14 k-tiles and beats
-    the unsplit pick by a tenth of its modelled time plus 3.5 us of launch. On 36 shapes (m = 32..256, n = 1536..24576,
+    A plan is taken when it fits one round (tile slots x SPLIT_K <= num_cus), leaves every part at least 14 k-tiles (24 when there are only two parts) and beats
+    the unsplit pick (its own, slightly lower time per k-tile) by a tenth of its modelled time plus 3.5 us of launch. On 36 shapes (m = 32..256, n = 1536..24576,
     k = 1536..16384) swept with every tile and factor, weights cycling through more matrices than the caches hold, the
-    plan taken is the fastest measured or within 1 % of it wherever one is taken: 13 to 38 % faster than unsplit
-    (64 x 4096 x 7168: 64 x 64 tiles in four parts; 32 x 2112 x 7168: 32 x 32 in three); k = 2048 and n = 16384 or more
-    stay unsplit. A plan also goes before the weight-streaming kernel of up to 16 rows (32 x 32 tiles in two to four parts
+    plan taken is the fastest measured or within 1 % of it wherever one is taken (64 x 4096 x 7168: 64 x 64 tiles in four
+    parts; 32 x 2112 x 7168: 32 x 32 in three); over 80 shapes with a plan (m = 17..1024, 13 (n, k)) it takes 0.47 to 1.04 of the
+    unsplit time, median 0.83; k up to about 5000 in two parts, k = 2048 and n = 16384 or more stay unsplit. A plan also goes before the weight-streaming kernel of up to 16 rows (32 x 32 tiles in two to four parts
     against that kernel, m = 1..16: n = 4096, k = 7168: 9.7 - 9.8 against 10.7 - 12.2 us; n = 2048: 8.4 against 10.1 - 11.8; level
     at k = 4096 and at k = 16384 below 8 rows), which runs where no plan exists or no workspace is at hand. Same rule as
     `pick_split_k` in yan_amd/csrc/yan_gemm_capi.hip (a CPU test keeps the two in step)."""
@@ -176,7 +179,7 @@ def get_split_k_fp8_config(m: int, n: int, k: int, num_cus: int) -> Optional[Tup
     if unsplit not in _FP8_SPLIT_K_TILE_US or ceil_div(m, unsplit[0]) * ceil_div(n, unsplit[1]) > num_cus:
         return None
     floor = n * k / 6.0e6
-    base = max(k_tiles * _FP8_SPLIT_K_TILE_US[unsplit], floor)
+    base = max(k_tiles * _FP8_UNSPLIT_TILE_US[unsplit], floor)
     best, best_plan = None, None
     for (bm, bn), per_k_tile in _FP8_SPLIT_K_TILE_US.items():
         if bm > 32 and bm >= 2 * m:
@@ -184,7 +187,8 @@ def get_split_k_fp8_config(m: int, n: int, k: int, num_cus: int) -> Optional[Tup
         tiles = ceil_div(m, bm) * ceil_div(n, bn)
         for split in FP8_SPLIT_K_FACTORS:
             # a workgroup per part of every tile slot (tiles rounded up to the 8 XCDs); 256 also bounds the workspace
-            if ceil_div(tiles, 8) * 8 * split > min(num_cus, 256) or ceil_div(k_tiles, split) < 14:
+            # two parts save half the k-tiles at most: they pay from 24 k-tiles per part on, three and four from 14
+            if ceil_div(tiles, 8) * 8 * split > min(num_cus, 256) or ceil_div(k_tiles, split) < (24 if split == 2 else 14):
                 continue
             t = max(ceil_div(k_tiles, split) * per_k_tile + 0.5 + (split * bm * bn * 4) / 1024 * 0.0125, floor)
             if best is None or t < best:
