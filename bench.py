@@ -332,6 +332,26 @@ def main():
         del x8, sx, w8, sw, o
 
     if args.also:
+        # bf16 with few rows and long K, where the entry point splits K: a decode-like shape and the m = 256 shapes of the
+        # reference's own dense test with k >= 5120 (tests/test_cute.py), next to torch.matmul (hipBLASLt). Both sides cycle
+        # through copies of the weights that together exceed the caches, as a model's layers do.
+        from yan_amd.jit_kernels.heuristics import get_split_k_dense_config
+        for mm, nn, kk in ((64, 4096, 7168), (256, 2048, 7168), (256, 5120, 5120), (256, 7168, 16384)):
+            a, b, c = harness.make_bf16_case(mm, nn, kk, seed=42, scale=kk ** -0.5, device='cuda', gen_device='cuda')
+            weights = [b.clone() for _ in range(min(40, max(2, (600 << 20) // (nn * kk * 2))))]
+            def cycle(fn):
+                def run():
+                    for w in weights:
+                        fn(w)
+                return run
+            per = len(weights)
+            ms, _ = _event_time_ms(cycle(lambda w: yan.gemm_bf16_tn(a, w, c)), 8, 2, 4)
+            ms_t, _ = _event_time_ms(cycle(lambda w: torch.matmul(a, w.t(), out=c)), 8, 2, 4)
+            plan = get_split_k_dense_config(mm, nn, kk, yan.get_num_sms())
+            extra[f'bf16_{mm}x{nn}x{kk}_cycling_weights'] = {'us': round(ms * 1e3 / per, 2), 'torch_hipblaslt_us': round(ms_t * 1e3 / per, 2),
+                                                            'hipblaslt_over_this': round(ms_t / ms, 3), 'split_k_plan': list(plan) if plan else None,
+                                                            'weight_copies': per}
+            del a, b, c, weights
         # bf16 shapes whose tiles do not fill whole rounds of 256 compute units at 256 x 256, next to torch.matmul (hipBLASLt)
         for mm, nn, kk in ((4096, 5120, 5120), (2048, 7168, 7168), (4096, 7168, 16384), (8192, 8192, 9216)):
             a, b, c = harness.make_bf16_case(mm, nn, kk, seed=42, scale=kk ** -0.5, device='cuda', gen_device='cuda')
