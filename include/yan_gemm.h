@@ -13,7 +13,8 @@
  *
  * Conventions shared by every entry point:
  *   - all matrices are row-major with the K dimension contiguous ("TN"/"NT": both operands K-major);
- *   - pointers are device pointers owned by the caller; nothing is allocated, freed or retained;
+ *   - pointers are device pointers owned by the caller; nothing is allocated, freed or retained (the split-K entry points
+ *     work in a caller-owned workspace, or, for the one that says so, in a device array the library holds);
  *   - work is enqueued on `stream` (a hipStream_t, NULL for the default stream) and NOT synchronised;
  *   - the return value is a hipError_t as int: 0 on success, hipErrorInvalidValue (1) for sizes the kernels do
  *     not take (they never fault on a bad size), or whatever the launch reported;

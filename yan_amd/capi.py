@@ -42,7 +42,8 @@ def load() -> ctypes.CDLL:
 
 
 def _stream_handle():
-    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    from .jit_kernels.utils import current_raw_stream
+    return ctypes.c_void_p(current_raw_stream())
 
 
 def gemm_bf16_tn(a: torch.Tensor, b: torch.Tensor, c: torch.Tensor) -> int:
