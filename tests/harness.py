@@ -213,12 +213,14 @@ FP8_SPLIT_K_PLAN_OF_SHAPE = {
 }
 FP8_SPLIT_K_SHAPES = [s for s in FP8_SPLIT_K_PLAN_OF_SHAPE if s not in ((64, 4096, 7168), (128, 4096, 7168), (1, 4096, 7168))]
 # The same for the dense GEMMs: the three tiles split-K plans use, every factor, ragged m and n, n that is no multiple of 8,
-# a k tail (3080 = 48 k-tiles and 8 elements), a dozen rows (where a plan goes before the weight-streaming kernel).
+# k tails (3080 = 48 k-tiles and 8 elements, 7176), a dozen rows (where a plan goes before the weight-streaming kernel), six and
+# eight parts.
 DENSE_SPLIT_K_PLAN_OF_SHAPE = {
     (33, 196, 2048): (64, 64, 2), (100, 196, 3080): (64, 64, 3), (65, 196, 4096): (64, 64, 4),
     (129, 4100, 5632): (64, 128, 2), (200, 2112, 3072): (64, 128, 3), (129, 2112, 5120): (64, 128, 4),
     (300, 4100, 4096): (128, 128, 2), (200, 4100, 3080): (128, 128, 3), (200, 3076, 5120): (128, 128, 4),
     (64, 4096, 7168): (64, 64, 4), (256, 2048, 7168): (64, 128, 4), (12, 2052, 4096): (64, 64, 4),
+    (20, 580, 7176): (64, 64, 6), (50, 1028, 16384): (64, 64, 8),
 }
 DENSE_SPLIT_K_SHAPES = list(DENSE_SPLIT_K_PLAN_OF_SHAPE)
 # Grouped FP8 GEMMs: (rows per group, n, k, blocks of padding rows) and (groups, m_max, n, k, masked_m, expected_m).

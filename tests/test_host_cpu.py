@@ -101,6 +101,7 @@ def test_dense_split_k_plans():
         assert plan(*shape, 256) == expected, shape
     assert {(bm, bn) for bm, bn, _ in harness.DENSE_SPLIT_K_PLAN_OF_SHAPE.values()} == set(heuristics._DENSE_SPLIT_K_EXTRA_US)
     assert {s for _, _, s in harness.DENSE_SPLIT_K_PLAN_OF_SHAPE.values()} == set(heuristics.DENSE_SPLIT_K_FACTORS)
+    assert all((bm, bn) == (64, 64) for bm, bn, s in harness.DENSE_SPLIT_K_PLAN_OF_SHAPE.values() if s > 4)
     assert set(heuristics._DENSE_SPLIT_K_TILE_US) == {t for t in heuristics._DENSE_TILES if heuristics.get_dense_num_stages(*t) > 2}
     for m in (33, 64, 100, 129, 256, 300, 512, 1024):
         for n in (196, 1536, 2112, 4096, 4100, 7168, 24576):

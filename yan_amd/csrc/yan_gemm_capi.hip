@@ -97,6 +97,7 @@ bool pick_split_k(int m, int n, int k, int num_cus, int* bm, int* bn, int* split
 struct DenseSplitKTile { int bm, bn; double us_per_k_tile, extra_us; };      // extra < 0: not a tile plans use
 constexpr DenseSplitKTile kDenseSplitKTiles[] = {{64, 64, 0.248, 0.0}, {64, 128, 0.378, 1.0}, {128, 128, 0.51, 2.5}, {64, 192, 0.60, -1},
                                                  {128, 192, 0.80, -1}, {128, 256, 0.94, -1}, {256, 128, 0.94, -1}};
+constexpr int kDenseSplitKFactors[] = {2, 3, 4, 6, 8};       // six and eight parts on 64 x 64 tiles only
 int dense_skinny_atoms(int m, int n, int k, int num_cus);
 
 bool pick_dense_split_k(int m, int n, int k, int num_cus, int* bm, int* bn, int* split_k) {
@@ -115,7 +116,8 @@ bool pick_dense_split_k(int m, int n, int k, int num_cus, int* bm, int* bn, int*
     for (const DenseSplitKTile& t : kDenseSplitKTiles) {
         if (t.extra_us < 0 || (t.bm > 64 && t.bm >= 2 * m)) continue;
         const long long tiles = (long long)((m + t.bm - 1) / t.bm) * ((n + t.bn - 1) / t.bn);
-        for (const int s : kSplitKFactors) {
+        for (const int s : kDenseSplitKFactors) {
+            if (s > 4 && !(t.bm == 64 && t.bn == 64)) continue;
             const int per_part = (k_tiles + s - 1) / s;
             if ((tiles + 7) / 8 * 8 * s > (num_cus < 256 ? num_cus : 256) || per_part < 16) continue;
             const double loop = per_part * t.us_per_k_tile + 0.5 + double(s * t.bm * t.bn * 4) / 1024 * 0.0125 + t.extra_us;
@@ -159,6 +161,7 @@ int dense(int m, int n, int k, const void* a, const void* b, void* c, void* stre
     if (bm == BM && bn == BN && split_k == S) return int(yan::launch_dense_split_k<Atom, Elem, BM, BN, S>(m, n, k, a, b, c, s, workspace, workspace_bytes));
 #define YAN_DENSE_SPLIT_K_TILE(BM, BN) YAN_DENSE_SPLIT_K_CASE(BM, BN, 2) YAN_DENSE_SPLIT_K_CASE(BM, BN, 3) YAN_DENSE_SPLIT_K_CASE(BM, BN, 4)
         YAN_DENSE_SPLIT_K_TILE(64, 64) YAN_DENSE_SPLIT_K_TILE(64, 128) YAN_DENSE_SPLIT_K_TILE(128, 128)
+        YAN_DENSE_SPLIT_K_CASE(64, 64, 6) YAN_DENSE_SPLIT_K_CASE(64, 64, 8)
 #undef YAN_DENSE_SPLIT_K_TILE
 #undef YAN_DENSE_SPLIT_K_CASE
         return int(hipErrorInvalidValue);
@@ -374,6 +377,6 @@ int yan_gemm_select_split_k(int op, int m, int n, int k, int num_cus, int* block
     return 0;
 }
 
-const char* yan_gemm_version(void) { return "yan-gemm gfx950 11 dense + 18 split-K dense + 2 weight-streaming dense + 7 fp32 + 10 fp8 tile variants + 15 split-K fp8 variants + 1 weight-streaming fp8 variant + 12 grouped fp8 variants + 4 quantiser kernels"; }
+const char* yan_gemm_version(void) { return "yan-gemm gfx950 11 dense + 22 split-K dense + 2 weight-streaming dense + 7 fp32 + 10 fp8 tile variants + 15 split-K fp8 variants + 1 weight-streaming fp8 variant + 12 grouped fp8 variants + 4 quantiser kernels"; }
 
 } // extern "C"

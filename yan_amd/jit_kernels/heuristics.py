@@ -204,7 +204,7 @@ def get_split_k_fp8_config(m: int, n: int, k: int, num_cus: int) -> Optional[Tup
 _DENSE_SPLIT_K_TILE_US = {(64, 64): 0.248, (64, 128): 0.378, (128, 128): 0.51, (64, 192): 0.60, (128, 192): 0.80, (128, 256): 0.94,
                           (256, 128): 0.94}
 _DENSE_SPLIT_K_EXTRA_US = {(64, 64): 0.0, (64, 128): 1.0, (128, 128): 2.5}
-DENSE_SPLIT_K_FACTORS = (2, 3, 4)
+DENSE_SPLIT_K_FACTORS = (2, 3, 4, 6, 8)         # six and eight parts on 64 x 64 tiles only (few weight rows, long K)
 
 
 def get_split_k_dense_config(m: int, n: int, k: int, num_cus: int) -> Optional[Tuple[int, int, int]]:
@@ -214,7 +214,8 @@ def get_split_k_dense_config(m: int, n: int, k: int, num_cus: int) -> Optional[T
     tiles fill the chip. A plan fits one round (tile slots x SPLIT_K <= num_cus), leaves every part at least 16 k-tiles and
     must beat the unsplit pick by 11 % of its modelled time plus 3.5 us. Measured (bf16, weights cycling, unsplit ->
     plan): 64 x 4096 x 7168 37.1 -> 16.2 us, 256 x 2048 x 7168 34.2 -> 20.3, 256 x 5120 x 5120 44.7 -> 33.9,
-    256 x 7168 x 16384 113.4 -> 90.9, 512 x 4096 x 7168 53.4 -> 43.9 (hipBLASLt on the same operands: 22.7, 24.7, 49.6, 140.4, -);
+    64 x 2048 x 7168 36.1 -> 12.8 (six parts; four: 14.5), 64 x 1024 x 16384 69.3 -> 16.5 (eight parts; four: 24.1),
+    256 x 7168 x 16384 113.4 -> 90.9, 512 x 4096 x 7168 53.4 -> 43.9 (hipBLASLt on the first five and the 256-row shapes: 22.7, 24.7, 49.6, 140.4);
     over 54 shapes swept with every tile and factor the plan is the fastest measured or within 6 % of it (11 % in one case),
     and over 118 shapes with a plan (m = 33..1024, 14 (n, k)) it takes 0.35 to 0.92 of the unsplit time, median 0.65. Same rule as
     `pick_dense_split_k` in yan_amd/csrc/yan_gemm_capi.hip (a CPU test keeps the two in step). A plan goes before the
@@ -237,6 +238,8 @@ def get_split_k_dense_config(m: int, n: int, k: int, num_cus: int) -> Optional[T
             continue                # a tile more than twice as tall as the problem
         tiles = ceil_div(m, bm) * ceil_div(n, bn)
         for split in DENSE_SPLIT_K_FACTORS:
+            if split > 4 and (bm, bn) != (64, 64):
+                continue            # the last part of a larger tile would hold more partial sums than it has registers for
             if ceil_div(tiles, 8) * 8 * split > min(num_cus, 256) or ceil_div(k_tiles, split) < 16:
                 continue
             t = max(ceil_div(k_tiles, split) * _DENSE_SPLIT_K_TILE_US[(bm, bn)] + 0.5 + (split * bm * bn * 4) / 1024 * 0.0125 + extra, floor)
