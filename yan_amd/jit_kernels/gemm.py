@@ -98,6 +98,8 @@ def split_k_workspace(device: torch.device, stream) -> torch.Tensor:
     key = (device.index, stream if isinstance(stream, int) else stream.cuda_stream)
     workspace = _split_k_workspaces.get(key)
     if workspace is None:
+        if len(_split_k_workspaces) >= 64:      # streams come and go: the oldest workspace returns to torch's allocator,
+            _split_k_workspaces.pop(next(iter(_split_k_workspaces)))      # which hands it out again in stream order
         workspace = torch.zeros(SPLIT_K_WORKSPACE_BYTES, dtype=torch.uint8, device=device)
         _split_k_workspaces[key] = workspace
     return workspace
