@@ -573,6 +573,11 @@ dense_gemm_mfma_8w(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
 template <typename Atom, typename Elem, int BLOCK_M, int BLOCK_N, int STAGES>
 __device__ __forceinline__ void
 dense_gemm_walk(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, Elem* __restrict__ C, int m, int n, int k, int num_slots) {
+    // a workgroup per tile (no cap): the tile without a loop around it (up to 2 % faster than one trip round the loop below)
+    if (int(gridDim.x) >= num_slots) {
+        dense_gemm_body<Atom, Elem, BLOCK_M, BLOCK_N, STAGES>(A, B, C, m, n, k, int(blockIdx.x));
+        return;
+    }
     for (int slot = blockIdx.x; slot < num_slots; slot += gridDim.x) {
         dense_gemm_body<Atom, Elem, BLOCK_M, BLOCK_N, STAGES>(A, B, C, m, n, k, slot);
         if (slot + int(gridDim.x) < num_slots) __syncthreads();
