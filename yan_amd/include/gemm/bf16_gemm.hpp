@@ -53,53 +53,27 @@ struct DenseTileConfig {
 
 // STAGES (3 ..): a ring of that many LDS stages with STAGES - 1 k-tiles in
 // flight, for the smaller tiles, which are picked when a problem is bound by streaming its operands.
-// Where the SPLIT_K parts of a dense tile meet: as fp8_meet_partials in fp8_gemm.hpp (sums written and read at device scope,
-// a counter per tile and wave, the last wave to arrive adds the parts up in the order of their K ranges and stores).
+// Where the SPLIT_K parts of a dense tile meet (meet_partials in tile_io.hpp): the wave's TN x TM atoms of 16 sums each, as
+// four 16-byte vectors per atom.
+template <typename Acc>
+struct AccQuarter {         // registers 4q .. 4q+3 of an accumulator, readable and writable as one f32x4
+    Acc& acc;
+    int  q;
+    __device__ __forceinline__ operator f32x4() const { return f32x4{acc[4 * q], acc[4 * q + 1], acc[4 * q + 2], acc[4 * q + 3]}; }
+    __device__ __forceinline__ void operator=(f32x4 v) const {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) acc[4 * q + r] = v[r];
+    }
+    __device__ __forceinline__ void operator+=(f32x4 v) const {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) acc[4 * q + r] += v[r];
+    }
+};
 template <int SPLIT_K, int NW, int TN, int TM, typename Acc>
 __device__ __forceinline__ bool
 dense_meet_partials(Acc (&acc)[TN][TM], float* __restrict__ partials, unsigned* __restrict__ counters, int tile_slot, int split, int wave, int lane) {
-    constexpr int kSc1 = 16;        // cache-policy bit sc1 of gfx950 buffer instructions: device scope
-    constexpr uint32_t VEC_BYTES = kWaveSize * 16, WAVE_BYTES = TN * TM * 4 * VEC_BYTES, PART_BYTES = NW * WAVE_BYTES;
-    const __amdgpu_buffer_rsrc_t parts = make_rsrc(partials + size_t(tile_slot) * (SPLIT_K * PART_BYTES / 4), SPLIT_K * PART_BYTES);
-    const uint32_t lane_off = uint32_t(wave) * WAVE_BYTES + lane * 16;
-#pragma unroll
-    for (int i = 0; i < TN; ++i)
-#pragma unroll
-        for (int j = 0; j < TM; ++j)
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const f32x4 v = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
-                __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(i32x4, v), parts, lane_off + ((i * TM + j) * 4 + q) * VEC_BYTES,
-                                                       split * PART_BYTES, kSc1);
-            }
-    __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, kNoWaitLgkm));
-    asm volatile("" ::: "memory");
-    unsigned before = 0;
-    if (lane == 0) before = __hip_atomic_fetch_add(counters + tile_slot * NW + wave, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    before = __builtin_amdgcn_readfirstlane(before);
-    asm volatile("" ::: "memory");
-    if (before != SPLIT_K - 1) return false;
-#pragma unroll
-    for (int i = 0; i < TN; ++i)
-#pragma unroll
-        for (int j = 0; j < TM; ++j)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
-#pragma unroll
-    for (int s = 0; s < SPLIT_K; ++s)
-#pragma unroll
-        for (int i = 0; i < TN; ++i)
-#pragma unroll
-            for (int j = 0; j < TM; ++j)
-#pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    const f32x4 v = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(parts, lane_off + ((i * TM + j) * 4 + q) * VEC_BYTES,
-                                                                                                    s * PART_BYTES, kSc1));
-#pragma unroll
-                    for (int r = 0; r < 4; ++r) acc[i][j][4 * q + r] += v[r];
-                }
-    if (lane == 0) __hip_atomic_store(counters + tile_slot * NW + wave, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    return true;
+    return meet_partials<SPLIT_K, NW, TN * TM * 4>([&](int v) { return AccQuarter<Acc>{acc[(v / 4) / TM][(v / 4) % TM], v % 4}; }, partials, counters,
+                                                   tile_slot, split, wave, lane);
 }
 
 template <typename Atom, typename Elem, int BLOCK_M, int BLOCK_N, int STAGES, int SPLIT_K = 1>

@@ -214,48 +214,11 @@ fp8_store_slab(const f32x4 (&acc)[TN][TM], uint8_t* region, __amdgpu_buffer_rsrc
 // GroupedMasked:     lhs [G, m, K], out [G, m, N], rhs as above; only the first grouped_layout[g] rows of group g
 //                    are computed; lhs_scales of group g start at g * sa_stride_g floats. Slots are numbered by
 //                    MaskedSlots: the tile rows below `expected_m` of all groups first.
-// Where the SPLIT_K parts of a tile meet. Wave w of every part leaves its sums in `partials` (laid out as the registers
-// are: part, wave, atom, lane) and counts itself in at counters[tile * NW + w]; the wave that arrives last adds the parts
-// up in the order of their K ranges, whichever it was itself, puts the counter back to zero for the next launch and
-// returns true: it stores the tile. The counters must be zero before the first launch.
-// The parts run on different XCDs, whose L2s do not see each other's lines. The sums are therefore written and read at
-// device scope (cache policy sc1: written through to memory, read from there), as the counter is; a device-scope fence
-// instead would write back and invalidate the whole L2 of the XCD once per wave (measured: 45-110 us for a 10 us GEMM).
-constexpr int kDeviceScope = 16;        // cache-policy bit sc1 of gfx950 buffer instructions
+// Where the SPLIT_K parts of a tile meet (meet_partials in tile_io.hpp): the wave's TN x TM atoms of four sums each.
 template <int SPLIT_K, int NW, int TN, int TM>
 __device__ __forceinline__ bool
 fp8_meet_partials(f32x4 (&acc)[TN][TM], float* __restrict__ partials, unsigned* __restrict__ counters, int tile_slot, int split, int wave, int lane) {
-    constexpr uint32_t ATOM_BYTES = kWaveSize * 16, WAVE_BYTES = TN * TM * ATOM_BYTES, PART_BYTES = NW * WAVE_BYTES;
-    const __amdgpu_buffer_rsrc_t parts = make_rsrc(partials + size_t(tile_slot) * (SPLIT_K * PART_BYTES / 4), SPLIT_K * PART_BYTES);
-    const uint32_t lane_off = uint32_t(wave) * WAVE_BYTES + lane * 16;
-#pragma unroll
-    for (int i = 0; i < TN; ++i)
-#pragma unroll
-        for (int j = 0; j < TM; ++j)
-            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(i32x4, acc[i][j]), parts, lane_off + (i * TM + j) * ATOM_BYTES,
-                                                   split * PART_BYTES, kDeviceScope);
-    // the sums have reached memory before the count is taken
-    __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, kNoWaitLgkm));
-    asm volatile("" ::: "memory");
-    unsigned before = 0;
-    if (lane == 0) before = __hip_atomic_fetch_add(counters + tile_slot * NW + wave, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    before = __builtin_amdgcn_readfirstlane(before);
-    asm volatile("" ::: "memory");
-    if (before != SPLIT_K - 1) return false;
-#pragma unroll
-    for (int i = 0; i < TN; ++i)
-#pragma unroll
-        for (int j = 0; j < TM; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int s = 0; s < SPLIT_K; ++s)
-#pragma unroll
-        for (int i = 0; i < TN; ++i)
-#pragma unroll
-            for (int j = 0; j < TM; ++j)
-                acc[i][j] += __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(parts, lane_off + (i * TM + j) * ATOM_BYTES,
-                                                                                             s * PART_BYTES, kDeviceScope));
-    if (lane == 0) __hip_atomic_store(counters + tile_slot * NW + wave, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    return true;
+    return meet_partials<SPLIT_K, NW, TN * TM>([&](int v) -> f32x4& { return acc[v / TM][v % TM]; }, partials, counters, tile_slot, split, wave, lane);
 }
 
 // STAGES: 2 = two LDS stages with the next k-tile's scales in registers; 3.. = a ring of that many stages.

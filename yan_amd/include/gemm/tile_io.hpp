@@ -122,6 +122,43 @@ struct TileStager {
     }
 };
 
+// Where the SPLIT_K parts of a split-K tile meet (fp8_gemm.hpp, bf16_gemm.hpp). Wave w of every part leaves its VECS
+// 16-byte vectors of sums in `partials` (laid out as the registers are: part, wave, vector, lane) and counts itself in at
+// counters[tile * NW + w]; the wave that arrives last adds the parts up in the order of their K ranges, whichever it was
+// itself, puts the counter back to zero for the next launch and returns true: it stores the tile. The counters must be zero
+// before the first launch. `sums(v)` is a reference to vector v of the caller's accumulators.
+// The parts run on different XCDs, whose L2s do not see each other's lines. The sums are therefore written and read at
+// device scope (cache policy sc1: written through to memory, read from there), as the counter is; a device-scope fence
+// instead would write back and invalidate the whole L2 of the XCD once per wave (measured: 45-110 us for a 10 us GEMM).
+template <int SPLIT_K, int NW, int VECS, typename Sums>
+__device__ __forceinline__ bool
+meet_partials(Sums&& sums, float* __restrict__ partials, unsigned* __restrict__ counters, int tile_slot, int split, int wave, int lane) {
+    constexpr int kDeviceScope = 16;        // cache-policy bit sc1 of gfx950 buffer instructions
+    constexpr uint32_t VEC_BYTES = kWaveSize * 16, WAVE_BYTES = VECS * VEC_BYTES, PART_BYTES = NW * WAVE_BYTES;
+    const __amdgpu_buffer_rsrc_t parts = make_rsrc(partials + size_t(tile_slot) * (SPLIT_K * PART_BYTES / 4), SPLIT_K * PART_BYTES);
+    const uint32_t lane_off = uint32_t(wave) * WAVE_BYTES + lane * 16;
+#pragma unroll
+    for (int v = 0; v < VECS; ++v)
+        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(i32x4, f32x4(sums(v))), parts, lane_off + v * VEC_BYTES, split * PART_BYTES, kDeviceScope);
+    // the sums have reached memory before the count is taken
+    __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, kNoWaitLgkm));
+    asm volatile("" ::: "memory");
+    unsigned before = 0;
+    if (lane == 0) before = __hip_atomic_fetch_add(counters + tile_slot * NW + wave, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    before = __builtin_amdgcn_readfirstlane(before);
+    asm volatile("" ::: "memory");
+    if (before != SPLIT_K - 1) return false;
+#pragma unroll
+    for (int v = 0; v < VECS; ++v) sums(v) = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int s = 0; s < SPLIT_K; ++s)
+#pragma unroll
+        for (int v = 0; v < VECS; ++v)
+            sums(v) += __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(parts, lane_off + v * VEC_BYTES, s * PART_BYTES, kDeviceScope));
+    if (lane == 0) __hip_atomic_store(counters + tile_slot * NW + wave, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return true;
+}
+
 // Byte offset, relative to the first row of an R-row atom that starts at a multiple of 16 tile rows, of logical
 // chunk `chunk` of the row this lane owns.
 template <int R>
