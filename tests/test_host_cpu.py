@@ -51,6 +51,23 @@ def test_tile_heuristics_fill_256_cus():
     assert ranked == sorted(ranked) and len(ranked) == len(heuristics._FP8_TILES)
 
 
+def test_activation_scales_are_relaid_only_where_it_pays():
+    """Large problems get token-contiguous activation scales (same values), small ones and scales that already are
+    token-contiguous pass through untouched."""
+    from yan_amd.jit_kernels.utils import scales_for_kernel, SCALE_RELAYOUT_MIN_FLOP
+    rows = torch.arange(512 * 56, dtype=torch.float32).reshape(512, 56)
+    assert scales_for_kernel(rows, SCALE_RELAYOUT_MIN_FLOP / 2) is rows
+    big = scales_for_kernel(rows, SCALE_RELAYOUT_MIN_FLOP)
+    assert big.stride() == (1, 512) and torch.equal(big, rows)
+    assert scales_for_kernel(big, 1e15) is big
+    one_block = rows[:, :1]
+    assert scales_for_kernel(one_block, 1e15) is one_block
+    batched = torch.arange(3 * 64 * 8, dtype=torch.float32).reshape(3, 64, 8)
+    relaid = scales_for_kernel(batched, 1e15)
+    assert relaid.stride() == (64 * 8, 1, 64) and torch.equal(relaid, batched)
+    assert scales_for_kernel(relaid, 1e15) is relaid
+
+
 def test_split_k_plans():
     """K is split when the unsplit tiles leave the chip short of work and K is long; every plan fits one round of
     workgroups and the workspace, leaves each part 14 k-tiles or more (24 of two), and the shapes of the GPU suite get the plans the

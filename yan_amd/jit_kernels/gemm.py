@@ -18,7 +18,7 @@ import torch
 from .heuristics import (get_best_fp8_config, get_fp8_num_stages, get_fp8_tile_space, get_skinny_fp8_config,
                          get_split_k_fp8_config, tuning_enabled)
 from .tuner import FrozenKeys, jit_tuner
-from .utils import current_raw_stream, get_num_sms, ceil_div, get_col_major_tensor
+from .utils import current_raw_stream, get_num_sms, ceil_div, get_col_major_tensor, scales_for_kernel
 
 # C++ code templates
 includes = ('"gemm/fp8_gemm.hpp"', '"gemm/fp8_gemm_skinny.hpp"')
@@ -183,6 +183,7 @@ def gemm_fp8_fp8_bf16_nt(lhs: Tuple[torch.Tensor, torch.Tensor],
         return
 
     num_sms = get_num_sms()
+    lhs_scales = scales_for_kernel(lhs_scales, 2.0 * m * n * k)
     stride_m, stride_k = lhs_scales.stride()
     token_contiguous = (m == 1 or stride_m == 1) and (lhs_scales.size(1) == 1 or stride_k == m)
     name, keys, defs, smem_size, code_template = fp8_kernel_plan(m, n, k, num_sms, token_contiguous)

@@ -15,7 +15,7 @@ import torch
 from .gemm import includes
 from .heuristics import get_best_grouped_fp8_config, get_fp8_num_stages
 from .tuner import FrozenKeys, jit_tuner
-from .utils import ceil_div, current_raw_stream, get_m_alignment_for_contiguous_layout, get_num_sms
+from .utils import ceil_div, current_raw_stream, get_m_alignment_for_contiguous_layout, get_num_sms, scales_for_kernel
 
 template = """
 using namespace yan;
@@ -105,6 +105,7 @@ def m_grouped_gemm_fp8_fp8_bf16_nt_contiguous(lhs: Tuple[torch.Tensor, torch.Ten
 
     if m == 0:
         return
+    lhs_scales = scales_for_kernel(lhs_scales, 2.0 * m * n * k)
     _launch('GroupedContiguous', num_groups, m, m, n, k, lhs, lhs_scales, rhs, rhs_scales, out, m_indices,
             (lhs_scales.stride(0), lhs_scales.stride(1), 0, 0))
 
@@ -142,5 +143,6 @@ def m_grouped_gemm_fp8_fp8_bf16_nt_masked(lhs: Tuple[torch.Tensor, torch.Tensor]
 
     if m == 0 or num_groups == 0:
         return
+    lhs_scales = scales_for_kernel(lhs_scales, 2.0 * num_groups * min(expected_m, m) * n * k)
     _launch('GroupedMasked', num_groups, min(expected_m, m), m, n, k, lhs, lhs_scales, rhs, rhs_scales, out, masked_m,
             (lhs_scales.stride(1), lhs_scales.stride(2), lhs_scales.stride(0), min(expected_m, m)))
