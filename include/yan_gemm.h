@@ -70,6 +70,8 @@ YAN_API int yan_gemm_float_nt(int m, int n, int k, float alpha, const float* a, 
  *   lhs        e4m3 (OCP, max 448) [m,k] row-major
  *   lhs_scales fp32, element (i,kb) at lhs_scales[i*lhs_scales_stride_m + kb*lhs_scales_stride_k]
  *              (row-major: strides (k/128, 1); token-contiguous as DeepGEMM callers pass it: (1, m))
+ *              Both give the same bits. Large problems (256-row tiles) run 13-18 % faster on token-contiguous scales:
+ *              a wave reads one scale per lane and k-tile, in the row-major layout a cache line each.
  *   rhs        e4m3 [n,k] row-major;  rhs_scales fp32 [ceil(n/128)][k/128] row-major
  *   out        bf16 [m,n] row-major
  * Requires k % 128 == 0, n % 4 == 0; m arbitrary; (m rounded up to the tile's rows, at most 256) * k < 2^31 bytes, same
