@@ -393,6 +393,18 @@ def main():
         extra['fp8_grouped_masked_4x1024x4096x7168'] = {'us': round(ms * 1e3, 1), 'tflops': round(fl / ms / 1e9, 1),
                                                         'frac_of_fp8_peak': round(fl / ms / 1e9 / PEAK_FP8_TFLOPS, 4)}
         del x8, sx, w8, sw, o
+        # the masked layout at decode sizes: 32 groups holding 8 rows each of 64; 940 MB of weights, more than the caches
+        # hold, so every launch streams them from HBM
+        groups, held = 32, 8
+        (x8, sx), (w8, sw), o, mm_ = harness.make_grouped_masked_case(groups, 64, nn, kk, (held,) * groups, seed=42, device='cuda', gen_device='cuda')
+        sx = yan.get_col_major_tensor(sx)
+        t = yan.bench_kineto(lambda: yan.m_grouped_gemm_fp8_fp8_bf16_nt_masked((x8, sx), (w8, sw), o, mm_, held), 'fp8_gemm',
+                             suppress_kineto_output=True)
+        byt = groups * (nn * kk + 4 * ((nn + 127) // 128) * (kk // 128) + held * (kk + 4 * (kk // 128)) + held * nn * 2)
+        extra['fp8_grouped_masked_decode_32x8x4096x7168'] = {'kernel_us': round(t * 1e6, 1), 'algorithmic_bytes': byt,
+                                                             'gb_per_s': round(byt / t / 1e9, 1),
+                                                             'frac_of_hbm_peak': round(byt / t / 1e9 / PEAK_HBM_GBPS, 4)}
+        del x8, sx, w8, sw, o
         # quantisers in front of the GEMM (HBM-bound): cfg3's activations per token, its weights per block, from bf16
         mm, nn, kk = harness.BASELINE_FP8['cfg3']
         xs = torch.randn(mm, kk, device='cuda').bfloat16()
