@@ -228,8 +228,11 @@ DENSE_SPLIT_K_SHAPES = list(DENSE_SPLIT_K_PLAN_OF_SHAPE)
 # block between the groups (negative entry) and one at the end; group 1 has 63 blocks, so it starts and the run ends on
 # odd multiples of 128. The test also runs the rows rotated by one block, which moves every boundary by 128 rows.
 GROUPED_TWO_PASS_CASE = ((8192, -128, 8064, 8192, 8192), 4096, 1024, 1)
+# Sixteen groups of nine blocks: every other boundary falls in the middle of a 256-row tile, and the 73 tile rows are more
+# than the 64 a wave looks at at once when it works out which rows hold two groups (those go first in the launch order).
+GROUPED_TWO_GROUP_ROWS_FIRST_CASE = ((1152,) * 16, 512, 512, 1)
 GROUPED_CONTIGUOUS_TEST_CASES = [
-    GROUPED_TWO_PASS_CASE,
+    GROUPED_TWO_PASS_CASE, GROUPED_TWO_GROUP_ROWS_FIRST_CASE,
     ((100, 128, 1, 300), 320, 384, 1), ((128, 128), 4096, 1024, 0), ((129,), 200, 128, 2),
     ((1024, 1024, 1024, 1024), 4096, 7168, 0), ((8192, 8192, 8192, 8192), 4096, 7168, 0),
     # long groups whose boundaries fall in the middle of 256-row tiles (two-pass tiles), with a trailing padding block

@@ -8,6 +8,8 @@
 //     exactly once and, for grids that are multiples of 8, never leaves the XCD residue b % 8;
 //   * the masked layout's slot numbering (MaskedSlots) visits every (group, tile) once, likely tile rows first, and bands
 //     fitted to the height of a group lose no tile and keep a patch inside one group;
+//   * the contiguous layout's slot numbering on 256-row tiles (ContiguousSlots) visits every tile once within the launched
+//     slots for any number of two-group rows, and deals those rows' tiles evenly to the XCDs, first in each;
 //   * the same holds in region order (operand rows long enough that the problem outgrows the memory-side cache), whose
 //     choice of region is pinned for a few measured shapes.
 #include "gemm/scheduler.hpp"
@@ -115,6 +117,35 @@ int main() {
                         else CHECK(!rest_seen);
                     }
                     for (int v : seen) CHECK(v == 1);
+                    ++cases;
+                }
+    // the contiguous layout's slot numbering on 256-row tiles (ContiguousSlots): every (row position, column) once within the
+    // slots the host launches, whatever number of two-group rows the device finds; those rows' tiles come first in every
+    // XCD's slots and no XCD gets two more of them than another
+    for (int tm : {1, 2, 7, 8, 32, 33, 73, 128})
+        for (int tn : {1, 2, 16, 28, 33})
+            for (int groups : {1, 4, 16})
+                for (int two : {0, 1, 2, 7, 8, 31, 64, 127}) {
+                    if (two > tm) continue;
+                    const int bm = 256, bn = 256, m = (tm - 1) * bm + 129, n = (tn - 1) * bn + 1;
+                    const yan::ContiguousSlots slots(m, n, bm, bn, groups, two);
+                    const long long num_slots = yan::ContiguousSlots::num_slots(m, n, bm, bn);
+                    CHECK(num_slots % yan::kNumXCD == 0 && num_slots <= (long long)tm * tn + 2 * yan::kNumXCD);
+                    std::vector<int> seen(size_t(tm) * tn, 0);
+                    int first_of_xcd[yan::kNumXCD] = {0};
+                    bool other_seen[yan::kNumXCD] = {false};
+                    for (int s = 0; s < num_slots; ++s) {
+                        const yan::TileCoord t = slots.tile_of(s);
+                        if (!t.valid) continue;
+                        CHECK(t.m_idx >= 0 && t.m_idx < tm && t.n_idx >= 0 && t.n_idx < tn);
+                        ++seen[size_t(t.m_idx) * tn + t.n_idx];
+                        if (two == 0) continue;
+                        const int x = s % yan::kNumXCD;
+                        if (t.m_idx < two) { CHECK(!other_seen[x]); ++first_of_xcd[x]; }
+                        else other_seen[x] = true;
+                    }
+                    for (int v : seen) CHECK(v == 1);
+                    for (int x = 0; x < yan::kNumXCD; ++x) CHECK(first_of_xcd[x] - first_of_xcd[yan::kNumXCD - 1] <= 1 && first_of_xcd[x] >= first_of_xcd[yan::kNumXCD - 1]);
                     ++cases;
                 }
     // what the traffic model picks for shapes that were measured (bf16, 256 x 256 tiles)

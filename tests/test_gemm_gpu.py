@@ -939,6 +939,13 @@ def test_grouped_contiguous_parity(rows, n, k, pad_blocks):
         assert bool(((halves[:, 0] != halves[:, 1]) & (halves >= 0).all(1)).any())      # two groups in one tile
         assert bool(((halves[:, 0] < 0) & (halves[:, 1] >= 0)).any())                   # padding, then a group
         assert bool(((halves[:, 0] >= 0) & (halves[:, 1] < 0)).any())                   # a group, then padding
+    if rows == testing.GROUPED_TWO_GROUP_ROWS_FIRST_CASE[0]:
+        from yan_amd.jit_kernels.m_grouped_gemm import grouped_kernel_plan
+        assert grouped_kernel_plan('GroupedContiguous', len(group_rows), m, n, k, 256)[1]['BLOCK_M'] == 256
+        blocks = idx.view(-1, 128)[:, 0]
+        halves = blocks[:len(blocks) // 2 * 2].view(-1, 2)
+        two = ((halves[:, 0] != halves[:, 1]) & (halves >= 0).all(1)).nonzero().flatten()
+        assert len(two) == 8 and int(two.min()) < 64 <= int(two.max()) and (m + 255) // 256 > 64
     a8d, sad, b8d, sbd, idxd = a8.cuda(), sa.cuda(), b8.cuda(), sb.cuda(), idx.cuda()
     got = out.cuda()
     assert yan.m_grouped_gemm_fp8_fp8_bf16_nt_contiguous((a8d, sad), (b8d, sbd), got, idxd) is None

@@ -221,6 +221,47 @@ fp8_meet_partials(f32x4 (&acc)[TN][TM], float* __restrict__ partials, unsigned* 
     return meet_partials<SPLIT_K, NW, TN * TM>([&](int v) -> f32x4& { return acc[v / TM][v % TM]; }, partials, counters, tile_slot, split, wave, lane);
 }
 
+// Contiguous groups on 256-row tiles: which tile rows hold two groups (they go first in the launch order, ContiguousSlots in
+// scheduler.hpp) is in `grouped_layout`, on the device; every wave works it out for itself, 64 tile rows at a time with a
+// row per lane. Bit `lane` of the result: tile row 64 * chunk + lane has a group in either half, and not the same.
+__device__ __forceinline__ unsigned long long
+two_group_rows_of_chunk(const int* __restrict__ grouped_layout, int m, int tiles_m, int chunk, int lane) {
+    const int row = chunk * kWaveSize + lane, m0 = row * 256;
+    bool yes = false;
+    if (row < tiles_m && m0 + 128 < m) {
+        const int g0 = grouped_layout[m0], g1 = grouped_layout[m0 + 128];
+        yes = g0 >= 0 && g1 >= 0 && g0 != g1;
+    }
+    return __ballot(yes);
+}
+
+__device__ __forceinline__ int
+count_two_group_rows(const int* __restrict__ grouped_layout, int m, int tiles_m, int lane) {
+    int count = 0;
+    for (int c = 0; c < ceil_div(tiles_m, kWaveSize); ++c) count += __popcll(two_group_rows_of_chunk(grouped_layout, m, tiles_m, c, lane));
+    return count;
+}
+
+// The tile row at position `pos` of the order "two-group rows first, then the others, either kind ascending". Wave-uniform.
+__device__ __forceinline__ int
+contiguous_row_at(const int* __restrict__ grouped_layout, int m, int tiles_m, int count, int pos, int lane) {
+    const bool among_two = pos < count;
+    int rank = among_two ? pos : pos - count;
+    for (int c = 0; c < ceil_div(tiles_m, kWaveSize); ++c) {
+        const int rows_here = min(kWaveSize, tiles_m - c * kWaveSize);
+        const unsigned long long all = rows_here == 64 ? ~0ull : ((1ull << rows_here) - 1);
+        const unsigned long long two = two_group_rows_of_chunk(grouped_layout, m, tiles_m, c, lane), mask = among_two ? two : (~two & all);
+        const int here = __popcll(mask);
+        if (rank < here) {
+            const bool mine = ((mask >> lane) & 1) && __popcll(mask & ((1ull << lane) - 1)) == rank;
+            const unsigned long long found = __ballot(mine);
+            return found ? c * kWaveSize + __ffsll((long long)found) - 1 : pos;
+        }
+        rank -= here;
+    }
+    return pos;         // not reached: pos < tiles_m
+}
+
 // STAGES: 2 = two LDS stages with the next k-tile's scales in registers; 3.. = a ring of that many stages.
 // One output tile (one slot of the launch: `bid` is what blockIdx.x would be with a workgroup per slot).
 template <int SHAPE_N, int SHAPE_K, int BLOCK_M, int BLOCK_N, GemmType kGemmType, int STAGES, int SPLIT_K = 1>
@@ -269,6 +310,10 @@ fp8_gemm_tile(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_sca
         rhs        += size_t(group) * N * K;
         rhs_scales += size_t(group) * NUM_N_BLOCKS * NUM_K_BLOCKS;
         m = min(m, grouped_layout[group]);        // rows of this group that exist; tiles past them leave at once
+    } else if constexpr (kGemmType == GemmType::GroupedContiguous && BLOCK_M == 256) {
+        const int two_group_rows = count_two_group_rows(grouped_layout, m, sched.tiles_m, get_lane_id());
+        tile = ContiguousSlots(m, N, BLOCK_M, BLOCK_N, num_groups, two_group_rows).tile_of(bid);
+        if (tile.valid && two_group_rows) tile.m_idx = contiguous_row_at(grouped_layout, m, sched.tiles_m, two_group_rows, tile.m_idx, get_lane_id());
     } else {
         tile = sched.tile_of(bid);
     }
@@ -407,11 +452,36 @@ fp8_gemm_tile(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_sca
     stage_a.issue(rsrc_a, lds_a0, 0, wave);
     stage_b.issue(rsrc_b, lds_b0, 0, wave);
     load_scales(0);
-    for (int kb = 0; kb + 1 < NUM_K_BLOCKS; kb += 2) {
-        k_step(kb, lds_a0, lds_b0, lds_a1, lds_b1);
-        k_step(kb + 1, lds_a1, lds_b1, lds_a0, lds_b0);
+    // A pass over one 128-row half of a 256-row tile: the waves whose slabs lie in the other half have nothing to multiply.
+    // They run a loop of their own with the same barriers and their share of the copies, which leaves the matrix cores half
+    // a tile per k-tile (a SIMD holds one wave of either half).
+    bool other_half = false;
+    if constexpr (kTwoHalves) {
+        static_assert(128 % Cfg::WTM == 0, "a wave's slab lies in one half of the tile");
+        other_half = num_passes == 2 && (m_slab < pass_lo[pass] || m_slab >= pass_hi[pass]);
     }
-    if (NUM_K_BLOCKS % 2 == 1) k_step(NUM_K_BLOCKS - 1, lds_a0, lds_b0, lds_a1, lds_b1);
+    if (kTwoHalves && other_half) {
+        auto copy_step = [&](int kb, uint8_t* a_nxt, uint8_t* b_nxt) {
+            wait_for_copies();
+            __syncthreads();
+#pragma unroll
+            for (int d = 0; d < NUM_COPIES; ++d) {
+                if (d < StA::PASSES) stage_a.issue_pass(rsrc_a, a_nxt, (kb + 1) * kRowBytes, wave, d);
+                else stage_b.issue_pass(rsrc_b, b_nxt, (kb + 1) * kRowBytes, wave, d - StA::PASSES);
+            }
+        };
+        for (int kb = 0; kb + 1 < NUM_K_BLOCKS; kb += 2) {
+            copy_step(kb, lds_a1, lds_b1);
+            copy_step(kb + 1, lds_a0, lds_b0);
+        }
+        if (NUM_K_BLOCKS % 2 == 1) copy_step(NUM_K_BLOCKS - 1, lds_a1, lds_b1);
+    } else {
+        for (int kb = 0; kb + 1 < NUM_K_BLOCKS; kb += 2) {
+            k_step(kb, lds_a0, lds_b0, lds_a1, lds_b1);
+            k_step(kb + 1, lds_a1, lds_b1, lds_a0, lds_b0);
+        }
+        if (NUM_K_BLOCKS % 2 == 1) k_step(NUM_K_BLOCKS - 1, lds_a0, lds_b0, lds_a1, lds_b1);
+    }
     epi_a = (NUM_K_BLOCKS % 2 == 1) ? lds_a0 : lds_a1;
     epi_b = (NUM_K_BLOCKS % 2 == 1) ? lds_b0 : lds_b1;
     } else {
@@ -867,7 +937,7 @@ public:
         const XcdTileScheduler<> sched(m, n, BLOCK_M, BLOCK_N);
         const uint64_t slots = kGemmType == GemmType::GroupedMasked
                                    ? uint64_t(MaskedSlots(num_groups, m, n, BLOCK_M, BLOCK_N, expected_m).num_slots())
-                                   : uint64_t(sched.grid_size());
+                                   : (BLOCK_M == 256 ? uint64_t(ContiguousSlots::num_slots(m, n, BLOCK_M, BLOCK_N)) : uint64_t(sched.grid_size()));
         if (slots >= kOutOfRange) return hipErrorInvalidValue;
         const int grid = capped_grid(int(slots), num_sms, device_cu_count());
         hipLaunchKernelGGL((fp8_gemm_kernel<SHAPE_N, SHAPE_K, BLOCK_M, BLOCK_N, kGemmType, int(kNumStages)>), dim3(grid),

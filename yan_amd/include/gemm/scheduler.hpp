@@ -189,6 +189,47 @@ struct MaskedSlots {
     }
 };
 
+// Slot numbering of the contiguous layout on 256-row tiles. A tile row whose two 128-row halves belong to two groups makes
+// two passes over K and takes about half as long again as the others; started last, one of them ends alone after everyone
+// else. `two_group_rows` of the `tiles_m` rows are of that kind (the kernel counts them in the caller's layout; the host
+// does not know them and launches `num_slots()` workgroups whatever their number). Their tiles come first in every XCD's
+// share of the slots and are dealt to the XCDs one by one, so that every XCD gets as many (an XCD runs its own slots, and
+// a patch of 32 slow tiles would fall to one of them); the other rows follow in band order dealt out in patches of 32.
+// `tile_of` names rows by position: positions below `two_group_rows` are the two-group rows, the others follow, either
+// kind in ascending order. With no such row the order is the plain one (a contiguous range of the band order per XCD).
+struct ContiguousSlots {
+    XcdTileScheduler<> all, rest;
+    int two_group_rows, first_tiles;
+
+    __host__ __device__ ContiguousSlots(int m, int n, int block_m, int block_n, int num_groups, int two_group_rows_)
+        : all(m, n, block_m, block_n), rest(0, 0, block_m, block_n), two_group_rows(two_group_rows_) {
+        all.fit_bands_to_groups(all.tiles_m / (num_groups > 0 ? num_groups : 1));
+        rest = XcdTileScheduler<>((all.tiles_m - two_group_rows) * block_m, n, block_m, block_n);
+        rest.band_height = all.band_height;
+        first_tiles = two_group_rows * all.tiles_n;
+    }
+
+    // one slot per XCD more than the tiles need: the two kinds of rows are rounded up to whole slots per XCD separately
+    __host__ __device__ static long long num_slots(int m, int n, int block_m, int block_n) {
+        return (long long)XcdTileScheduler<>(m, n, block_m, block_n).grid_size() + kNumXCD;
+    }
+
+    __host__ __device__ TileCoord tile_of(int slot) const {
+        if (two_group_rows == 0) return slot < all.grid_size() ? all.tile_of(slot) : TileCoord{0, 0, false};
+        const int x = slot % kNumXCD, q = slot / kNumXCD;
+        const int mine = first_tiles > x ? (first_tiles - x + kNumXCD - 1) / kNumXCD : 0;      // two-group tiles of this XCD
+        if (q < mine) {
+            const int t = q * kNumXCD + x;
+            return {t / all.tiles_n, t % all.tiles_n, true};
+        }
+        const int s = (q - mine) * kNumXCD + x;
+        if (s >= rest.grid_size()) return {0, 0, false};
+        TileCoord t = rest.dealt_band_tile_of(s);
+        t.m_idx += two_group_rows;
+        return t;
+    }
+};
+
 // Workgroups to launch for `slots` units of work (tiles, or groups x tiles) under the caller's compute-unit cap, the
 // `num_sms` of the reference's persistent kernels (yan/include/gemm/fp8_gemm.cuh:40 launches num_sms blocks,
 // yan/jit_kernels/utils.py:6-29 holds the cap). No cap (0, or at least `device_cus`): one workgroup per slot, and the
