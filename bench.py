@@ -386,6 +386,17 @@ def main():
         fl = 2.0 * sum(rows) * nn * kk
         extra['fp8_grouped_contiguous_4x8192x4096x7168'] = {'us': round(ms * 1e3, 1), 'tflops': round(fl / ms / 1e9, 1),
                                                             'frac_of_fp8_peak': round(fl / ms / 1e9 / PEAK_FP8_TFLOPS, 4)}
+        del x8, sx, w8, sw, o, idx
+        # groups whose boundaries fall in the middle of 256-row tiles (every other one): 8 groups of 896 and 1152 rows, next to
+        # 8 groups of 1024 rows
+        for label, rows in (('8x896_1152', (896, 1152) * 4), ('8x1024', (1024,) * 8)):
+            (x8, sx), (w8, sw), o, idx = harness.make_grouped_contiguous_case(rows, nn, kk, seed=42, device='cuda', gen_device='cuda')
+            sx = yan.get_col_major_tensor(sx)
+            ms, _ = _event_time_ms(lambda: yan.m_grouped_gemm_fp8_fp8_bf16_nt_contiguous((x8, sx), (w8, sw), o, idx), 30, 5, 150)
+            fl = 2.0 * sum(rows) * nn * kk
+            extra[f'fp8_grouped_contiguous_{label}x4096x7168'] = {'us': round(ms * 1e3, 1), 'tflops': round(fl / ms / 1e9, 1),
+                                                                 'frac_of_fp8_peak': round(fl / ms / 1e9 / PEAK_FP8_TFLOPS, 4)}
+            del x8, sx, w8, sw, o, idx
         (x8, sx), (w8, sw), o, mm_ = harness.make_grouped_masked_case(4, 1024, nn, kk, (1024,) * 4, seed=42, device='cuda', gen_device='cuda')
         sx = yan.get_col_major_tensor(sx)
         ms, _ = _event_time_ms(lambda: yan.m_grouped_gemm_fp8_fp8_bf16_nt_masked((x8, sx), (w8, sw), o, mm_, 1024), 50, 5, 600)
