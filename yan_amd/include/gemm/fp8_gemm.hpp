@@ -406,6 +406,10 @@ fp8_gemm_tile(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_sca
     using StB = TileStager<BLOCK_N, NW>;
     constexpr int NUM_COPIES = StA::PASSES + StB::PASSES, SPREAD_ROWS = TN >= 2 ? TN / 2 : 1;
     float sa_cur[TM], sb_cur[NB];
+    // A pass over one 128-row half of a 256-row tile does not fetch the other half of the activation tile: the copy passes of
+    // those rows (the first or the second half of them) go through the empty descriptor and move zeros.
+    [[maybe_unused]] __amdgpu_buffer_rsrc_t rsrc_a_half[2] = {rsrc_a, rsrc_a};
+    static_assert(!kTwoHalves || StA::PASSES % 2 == 0);
     auto k_step = [&](int kb, const uint8_t* a_cur, const uint8_t* b_cur, uint8_t* a_nxt, uint8_t* b_nxt) {
 #pragma unroll
         for (int j = 0; j < TM; ++j) sa_cur[j] = sa_next[j];
@@ -418,7 +422,7 @@ fp8_gemm_tile(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_sca
 #pragma unroll
             for (int d = 0; d < NUM_COPIES; ++d) {
                 if (d * SPREAD_ROWS / NUM_COPIES != row) continue;
-                if (d < StA::PASSES) stage_a.issue_pass(rsrc_a, a_nxt, (kb + 1) * kRowBytes, wave, d);
+                if (d < StA::PASSES) stage_a.issue_pass(kTwoHalves ? rsrc_a_half[d * 2 / StA::PASSES] : rsrc_a, a_nxt, (kb + 1) * kRowBytes, wave, d);
                 else stage_b.issue_pass(rsrc_b, b_nxt, (kb + 1) * kRowBytes, wave, d - StA::PASSES);
             }
         });
@@ -439,6 +443,11 @@ fp8_gemm_tile(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_sca
         rhs_scales = rhs_scales_all + size_t(pass_group[pass]) * NUM_N_BLOCKS * NUM_K_BLOCKS;
         rsrc_b     = make_rsrc(rhs, uint32_t(N) * K);
         if (pass) __syncthreads();        // every wave has read the last k-tile of the previous pass
+        if constexpr (kTwoHalves) {
+            const bool half_pass = num_passes == 2;
+            rsrc_a_half[0] = half_pass && pass_lo[pass] != m0 ? rsrc_none : rsrc_a;
+            rsrc_a_half[1] = half_pass && pass_hi[pass] == m0 + 128 ? rsrc_none : rsrc_a;
+        }
     }
 #pragma unroll
     for (int i = 0; i < TN; ++i)
@@ -466,7 +475,7 @@ fp8_gemm_tile(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_sca
             __syncthreads();
 #pragma unroll
             for (int d = 0; d < NUM_COPIES; ++d) {
-                if (d < StA::PASSES) stage_a.issue_pass(rsrc_a, a_nxt, (kb + 1) * kRowBytes, wave, d);
+                if (d < StA::PASSES) stage_a.issue_pass(rsrc_a_half[d * 2 / StA::PASSES], a_nxt, (kb + 1) * kRowBytes, wave, d);
                 else stage_b.issue_pass(rsrc_b, b_nxt, (kb + 1) * kRowBytes, wave, d - StA::PASSES);
             }
         };
