@@ -355,6 +355,13 @@ def jit_kernels_in_use(num_cus: int = 256):
     for groups, m_max, n, k, _, expected_m in GROUPED_MASKED_TEST_CASES:
         name, keys, arg_defs, _ = m_grouped_gemm.grouped_kernel_plan('GroupedMasked', groups, min(expected_m, m_max), n, k, num_cus)
         add(name, arg_defs, m_grouped_gemm.includes, m_grouped_gemm.template, keys)
+    # the grouped layouts under the compute-unit cap: tiles chosen for NUM_SMS_CAP units
+    rows, n, k, pad_blocks = GROUPED_TWO_GROUP_ROWS_FIRST_CASE
+    name, keys, arg_defs, _ = m_grouped_gemm.grouped_kernel_plan('GroupedContiguous', len(rows), sum(rows) + 128 * pad_blocks, n, k, NUM_SMS_CAP)
+    add(name, arg_defs, m_grouped_gemm.includes, m_grouped_gemm.template, keys)
+    groups, m_max, n, k, _, expected_m = GROUPED_MASKED_TEST_CASES[6]
+    name, keys, arg_defs, _ = m_grouped_gemm.grouped_kernel_plan('GroupedMasked', groups, min(expected_m, m_max), n, k, NUM_SMS_CAP)
+    add(name, arg_defs, m_grouped_gemm.includes, m_grouped_gemm.template, keys)
     return list(kernels.values())
 
 

@@ -699,6 +699,37 @@ def test_num_sms_caps_the_workgroups_without_changing_a_bit(m, n, k):
         yan.set_num_sms(full)
 
 
+def test_grouped_layouts_under_a_compute_unit_cap_give_the_same_bits():
+    """Both grouped layouts with `set_num_sms(64)`: 64 workgroups walk the slots, several tiles each (for the contiguous
+    layout on 256-row tiles the slots of `ContiguousSlots`, two-group rows first), and write the bits of the uncapped
+    launch."""
+    from yan_amd.jit_kernels.m_grouped_gemm import grouped_kernel_plan
+    cap, full = testing.NUM_SMS_CAP, yan.get_num_sms()
+    rows, n, k, pad_blocks = testing.GROUPED_TWO_GROUP_ROWS_FIRST_CASE
+    _announce('grouped contiguous under a cap', rows, n, k, cap)
+    (a8, sa), (b8, sb), out, idx = testing.make_grouped_contiguous_case(rows, n, k, seed=5, padding_blocks=pad_blocks)
+    a8, sa, b8, sb, idx = a8.cuda(), sa.cuda(), b8.cuda(), sb.cuda(), idx.cuda()
+    assert grouped_kernel_plan('GroupedContiguous', len(rows), a8.size(0), n, k, cap)[1]['BLOCK_M'] == 256
+    groups, m_max, n2, k2, masked, expected_m = testing.GROUPED_MASKED_TEST_CASES[6]
+    (x8, sx), (w8, sw), out2, mm = testing.make_grouped_masked_case(groups, m_max, n2, k2, masked, seed=6)
+    x8, sx, w8, sw, mm = x8.cuda(), sx.cuda(), w8.cuda(), sw.cuda(), mm.cuda()
+    results = {}
+    try:
+        for cus in (full, cap):
+            yan.set_num_sms(cus)
+            got, got2 = out.cuda(), out2.cuda()
+            yan.m_grouped_gemm_fp8_fp8_bf16_nt_contiguous((a8, sa), (b8, sb), got, idx)
+            _announce('grouped masked under a cap', groups, m_max, n2, k2, cus)
+            yan.m_grouped_gemm_fp8_fp8_bf16_nt_masked((x8, sx), (w8, sw), got2, mm, expected_m)
+            torch.cuda.synchronize()
+            results[cus] = (got, got2)
+    finally:
+        yan.set_num_sms(full)
+    assert torch.equal(results[cap][0], results[full][0])
+    assert torch.equal(results[cap][1], results[full][1])
+    assert bool((results[full][0][idx >= 0] != -7.0).any())
+
+
 @pytest.mark.parametrize('cap', testing.ODD_CAP_CASE[1])
 def test_walks_under_a_cap_that_is_no_multiple_of_the_xcds_reach_every_tile(cap):
     """18 tiles of 256 x 256 leave an empty slot at the end of six of the eight XCDs' ranges; 3 or 5 persistent workgroups
