@@ -327,8 +327,9 @@ def jit_kernels_in_use(num_cus: int = 256):
             name, keys, arg_defs = bf16_gemm.dense_kernel_plan(m, n, k, torch.bfloat16, cus, cap)
             add(name, arg_defs, bf16_gemm.includes, bf16_gemm.template, keys)
         for cus in (num_cus, NUM_SMS_CAP):
-            name, keys, arg_defs, _, code_template = gemm.fp8_kernel_plan(m, n, k, cus, False)
-            add(name, arg_defs, gemm.includes, code_template, keys)
+            for token_contiguous in (False, True):      # row-major scales of a large problem reach the kernel token-contiguous
+                name, keys, arg_defs, _, code_template = gemm.fp8_kernel_plan(m, n, k, cus, token_contiguous)
+                add(name, arg_defs, gemm.includes, code_template, keys)
     for block_m, block_n, (m, n, k) in FP8_EXPLICIT_TILE_CASES:
         name, keys, arg_defs, code_template = fp8_explicit_tile_plan(block_m, block_n, n, k)
         add(name, arg_defs, gemm.includes, code_template, keys)

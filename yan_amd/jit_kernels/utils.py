@@ -69,10 +69,11 @@ def get_col_major_tensor(x: torch.Tensor) -> torch.Tensor:
     return batched if x.dim() == 3 else batched.squeeze(0)
 
 
-# From this much arithmetic on (about 50 us of kernel time) a GEMM whose activation scales are not token-contiguous gets a
-# token-contiguous copy of them first: the 256-row tiles read a scale per lane and k-tile, which in the row-major layout is a
-# cache line per lane (4096 x 4096 x 7168: 110 us against 96 us), and the copy costs about 5 us.
-SCALE_RELAYOUT_MIN_FLOP = 1.2e11
+# From this much arithmetic on (about 40 us of kernel time) a GEMM whose activation scales are not token-contiguous gets a
+# token-contiguous copy of them first: the kernels read a scale per lane and k-tile, which in the row-major layout is a
+# cache line per lane (4096 x 4096 x 7168: 110 us against 96 us; 1024 x 4096 x 7168: 46.9 against 41.8), and the copy costs
+# about 3 us on the device. Below it the copy costs as much as it saves (512 x 7168 x 4096: 25.8 against 24.0 us).
+SCALE_RELAYOUT_MIN_FLOP = 6e10
 
 
 def scales_for_kernel(scales: torch.Tensor, flop: float) -> torch.Tensor:
