@@ -304,7 +304,7 @@ def main():
         if plan is not None:
             name, keys, defs, tmpl = plan
             split = jit.build(name, defs, jit.generate(fp8_entry.includes, defs, jit.cpp_format(tmpl, keys)))
-            workspace = fp8_entry.split_k_workspace(o.device, stream)
+            workspace, _ = fp8_entry.split_k_workspace(o.device, stream.cuda_stream)
             t_split = yan.bench_kineto(lambda: split(x8, sx, w8, sw, o, mm, stream, cus, smem, workspace, fp8_entry.SPLIT_K_WORKSPACE_BYTES),
                                        'fp8_gemm', suppress_kineto_output=True)
         # Weights from HBM, everything else warm, as a model's layers present them: every launch takes the next of enough copies

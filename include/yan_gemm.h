@@ -120,6 +120,14 @@ YAN_API int yan_gemm_fp8_fp8_bf16_nt_static(const void* lhs, const float* lhs_sc
                                     long long lhs_scales_stride_k, const void* rhs, const float* rhs_scales, void* out,
                                     int m, int n, int k, void* stream, int num_sms);
 
+/* Puts the arrival counters of a split-K workspace back to zero, on `stream` (a small fill kernel, so the call may be
+ * captured into a graph). `workspace` NULL names the library's own array, the one yan_gemm_fp8_fp8_bf16_nt_static uses on
+ * the current GPU. The counters are zero after every split-K launch that ran to its end, so an ordinary caller needs this
+ * once at most (instead of zero-filling a fresh workspace itself). Call it before reusing a workspace after anything that
+ * may have left a launch half done: a split-K call that returned non-zero, calls that overlapped on one workspace, a
+ * device reset. Partial sums need no clearing. It has no counterpart in the reference (its kernels keep no state). */
+YAN_API int yan_gemm_split_k_reset(void* workspace, void* stream);
+
 /* Grouped (mixture-of-experts) forms of the FP8 GEMM: group g has its own weights rhs[g] ([n,k] e4m3) and scale table
  * rhs_scales[g] ([ceil(n/128)][k/128]); both arrays are contiguous over g. Arithmetic per row as above.
  * They fill in the reference's GemmType::GroupedContiguous / GroupedMasked and `int* grouped_layout` hooks

@@ -24,7 +24,7 @@ def _declared(repo_root):
 
 def test_library_exports_every_declared_symbol(lib, repo_root):
     declared = _declared(repo_root)
-    assert declared == sorted(capi.SYMBOLS) and len(declared) == 17
+    assert declared == sorted(capi.SYMBOLS) and len(declared) == 18
     for name in declared:
         assert hasattr(lib, name), name
     out = subprocess.check_output(['nm', '-D', '--defined-only', os.path.join(repo_root, 'yan_amd', 'csrc', 'libyan_gemm.so')], text=True)

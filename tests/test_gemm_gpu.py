@@ -1170,6 +1170,78 @@ def test_split_k_replays_correctly_from_a_captured_graph():
         assert float(out8.float().abs().sum()) > 0 and float(c.float().abs().sum()) > 0
 
 
+def test_two_graphs_with_split_k_launches_do_not_share_a_workspace():
+    """Two graphs captured one after the other, each with split-K launches: every capture gets a workspace of its own,
+    zeroed by a node of its own graph, so the second graph replays correctly before the first has ever run, the two may be
+    replayed on different streams at the same time, and eager launches in between use yet another workspace."""
+    from yan_amd.jit_kernels import split_k
+    _announce('two split-k graphs')
+    (a8, sa), (b8, sb), out_1 = testing.make_fp8_case(33, 2112, 5376, seed=18, device='cuda', gen_device='cuda')
+    (c8, sc), (d8, sd), out_2 = testing.make_fp8_case(64, 4096, 7168, seed=19, device='cuda', gen_device='cuda')
+    assert yan.gemm.fp8_split_k_plan(33, 2112, 5376, yan.get_num_sms(), False) is not None
+    assert yan.gemm.fp8_split_k_plan(64, 4096, 7168, yan.get_num_sms(), False) is not None
+    yan.gemm_fp8_fp8_bf16_nt((a8, sa), (b8, sb), out_1)
+    yan.gemm_fp8_fp8_bf16_nt((c8, sc), (d8, sd), out_2)
+    torch.cuda.synchronize()
+    want_1, want_2 = out_1.clone(), out_2.clone()
+    captures_before = len(split_k._book.captures)
+    graph_1, graph_2 = torch.cuda.CUDAGraph(), torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph_1):
+        yan.gemm_fp8_fp8_bf16_nt((a8, sa), (b8, sb), out_1)
+        yan.gemm_fp8_fp8_bf16_nt((c8, sc), (d8, sd), out_2)
+    with torch.cuda.graph(graph_2):
+        yan.gemm_fp8_fp8_bf16_nt((c8, sc), (d8, sd), out_2)
+        yan.gemm_fp8_fp8_bf16_nt((a8, sa), (b8, sb), out_1)
+    assert len(split_k._book.captures) == captures_before + 2
+    ws = list(split_k._book.captures.values())[-2:]
+    assert ws[0].data_ptr() != ws[1].data_ptr()
+    assert all(w.data_ptr() != e.data_ptr() for w in ws for e in split_k._book.eager.values())
+    for first, second in ((graph_2, graph_1), (graph_1, graph_2), (graph_2, graph_2)):
+        for graph in (first, second):
+            out_1.zero_()
+            out_2.zero_()
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(out_1, want_1) and torch.equal(out_2, want_2)
+            yan.gemm_fp8_fp8_bf16_nt((a8, sa), (b8, sb), out_1)            # eager, on the stream's own workspace
+    # a graph heals itself: counters left dirty by whatever ran before are zeroed by the graph's own first node
+    ws[1][:split_k.SPLIT_K_COUNTER_BYTES].fill_(3)
+    out_1.zero_()
+    out_2.zero_()
+    graph_2.replay()
+    torch.cuda.synchronize()
+    assert torch.equal(out_1, want_1) and torch.equal(out_2, want_2)
+
+
+def test_a_workspace_whose_launch_failed_is_cleared_before_its_next_use(monkeypatch):
+    """The entry points clear the arrival counters of a workspace after a launch on it reported an error: counters that
+    are not zero would make the next launch store tiles early or never. With split-K switched off (YAN_SPLIT_K=0) the
+    entry keeps no state and gives the bits of the unsplit kernel."""
+    from yan_amd.jit_kernels import split_k
+    _announce('suspect split-k workspace')
+    (a8, sa), (b8, sb), out = testing.make_fp8_case(64, 4096, 7168, seed=20, device='cuda', gen_device='cuda')
+    yan.gemm_fp8_fp8_bf16_nt((a8, sa), (b8, sb), out)
+    torch.cuda.synchronize()
+    want = out.clone()
+    workspace, token = split_k.split_k_workspace(out.device, yan.jit_kernels.utils.current_raw_stream())
+    assert int(workspace[:split_k.SPLIT_K_COUNTER_BYTES].max()) == 0           # zero after a launch that ran to its end
+    workspace[:split_k.SPLIT_K_COUNTER_BYTES].fill_(1)
+    split_k.split_k_launch_failed(token)
+    out.zero_()
+    yan.gemm_fp8_fp8_bf16_nt((a8, sa), (b8, sb), out)
+    torch.cuda.synchronize()
+    assert torch.equal(out, want)
+    assert int(workspace[:split_k.SPLIT_K_COUNTER_BYTES].max()) == 0
+    monkeypatch.setenv('YAN_SPLIT_K', '0')
+    eager_before = dict(split_k._book.eager)
+    unsplit = torch.zeros_like(out)
+    yan.gemm_fp8_fp8_bf16_nt((a8, sa), (b8, sb), unsplit)
+    torch.cuda.synchronize()
+    assert split_k._book.eager == eager_before
+    ref = testing.dequant_lhs(a8, sa) @ testing.dequant_rhs(b8, sb).t()
+    assert float(yan.calc_diff(unsplit.float(), ref)) < 1e-5 and float(yan.calc_diff(unsplit.float(), want.float())) < 1e-8
+
+
 def test_capi_seeded_random_shapes_against_device_references():
     """Breadth: 240 seeded random shapes through the C entries (every tile variant, ragged edges, k tails, leading
     dimensions), each against an fp32 / fp64 product of the same operands on the device. The oracle-based tests above

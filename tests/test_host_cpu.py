@@ -421,3 +421,36 @@ def test_compare_tensors_verdicts(capsys):
     assert compare_tensors(y, x, mode='similarity', diff_tolerance=1e-9) is False
     assert compare_tensors(torch.zeros(3), torch.zeros(3), mode='similarity') is True
     assert compare_tensors(x, x[:2]) is False and compare_tensors(x, x, mode='cosine') is False
+
+
+def test_split_k_workspaces_are_kept_per_stream_and_per_capture():
+    """Bookkeeping of the Python entries' split-K workspaces: eager launches share a workspace per (device, stream), at
+    most `max_eager` are kept; every capture gets its own, never shared with eager launches or another capture and never
+    dropped; a workspace whose launch failed is cleared before its next use."""
+    from yan_amd.jit_kernels.split_k import WorkspaceBook
+    made, cleared = [], []
+    book = WorkspaceBook(make=lambda: made.append(object()) or made[-1], clear=cleared.append, max_eager=3)
+    w0 = book.get(0, 111)
+    assert book.get(0, 111) is w0 and len(made) == 1
+    w1 = book.get(0, 222)
+    w2 = book.get(1, 111)
+    assert len({id(w) for w in (w0, w1, w2)}) == 3
+    # captures: keyed by the capture's id, not by the stream that records it
+    c7 = book.get(0, 111, capture=7)
+    assert c7 is not w0 and book.get(0, 111, capture=7) is c7 and book.get(0, 999, capture=7) is c7
+    c8 = book.get(0, 111, capture=8)
+    assert c8 is not c7 and book.get(1, 111, capture=7) is not c7
+    assert len(made) == 6 and not cleared
+    # a failed launch: cleared once, at the next use
+    book.launch_failed(0, 222)
+    assert not cleared
+    assert book.get(0, 222) is w1 and cleared == [w1]
+    assert book.get(0, 222) is w1 and cleared == [w1]
+    book.launch_failed(0, 111, capture=7)           # the graph's own first node zeroes a capture's workspace
+    assert book.get(0, 111, capture=7) is c7 and cleared == [w1]
+    # eviction: the oldest eager workspace goes, captures stay
+    book.launch_failed(0, 111)
+    w3 = book.get(2, 5)
+    assert (0, 111) not in book.eager and len(book.eager) == 3 and (0, 111) not in book.suspect
+    assert book.get(0, 111) is not w0 and cleared == [w1]       # a fresh one: nothing to clear
+    assert len(book.captures) == 3 and book.get(0, 1, capture=8) is c8 and w3 is book.get(2, 5)

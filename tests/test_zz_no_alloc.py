@@ -43,3 +43,37 @@ def test_static_scratch_entry_point_matches_the_workspace_entry_point():
         if free_before is not None:
             assert free_now == free_before
         free_before = free_now
+
+
+def test_reset_clears_the_arrival_counters_of_a_workspace():
+    """yan_gemm_split_k_reset: counters that something left dirty (here: written by hand) are zero again after the call,
+    for a caller's workspace and, with a null workspace, for the library's own array; the next split-K call on either
+    gives the bits of a clean run, and the reset itself allocates nothing."""
+    torch.cuda.set_device(0)
+    lib = capi.load()
+    counter_bytes = lib.yan_gemm_split_k_counter_bytes()
+    lhs, rhs, out = testing.make_fp8_case(64, 4096, 7168, seed=41, device='cuda', gen_device='cuda')
+    assert capi.select_split_k(64, 4096, 7168, 256) is not None
+    workspace = capi.split_k_workspace()
+    assert capi.gemm_fp8_fp8_bf16_nt_split_k(lhs, rhs, out, workspace) == 0
+    torch.cuda.synchronize()
+    want = out.clone()
+    assert int(workspace[:counter_bytes].max()) == 0
+    print('[case] reset of a dirty workspace', flush=True)
+    workspace[:counter_bytes].fill_(1)
+    free_before = torch.cuda.mem_get_info()[0]
+    assert capi.split_k_reset(workspace) == 0
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free_before
+    assert int(workspace[:counter_bytes].max()) == 0
+    assert int(workspace[counter_bytes:counter_bytes + 4096].max()) > 0         # partial sums are left alone
+    out.zero_()
+    assert capi.gemm_fp8_fp8_bf16_nt_split_k(lhs, rhs, out, workspace) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(out, want)
+    print('[case] reset of the static array', flush=True)
+    assert capi.split_k_reset(None) == 0
+    out.zero_()
+    assert capi.gemm_fp8_fp8_bf16_nt_static(lhs, rhs, out) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(out, want)

@@ -11,7 +11,7 @@ _lib = None
 SYMBOLS = ('yan_gemm_bf16_tn', 'yan_gemm_fp16_tn', 'yan_gemm_float_nt', 'yan_gemm_fp8_fp8_bf16_nt', 'yan_m_grouped_gemm_fp8_fp8_bf16_nt_contiguous',
            'yan_m_grouped_gemm_fp8_fp8_bf16_nt_masked', 'yan_per_token_cast_to_fp8', 'yan_per_block_cast_to_fp8',
            'yan_gemm_select_tile', 'yan_gemm_fp8_fp8_bf16_nt_split_k', 'yan_gemm_fp8_fp8_bf16_nt_static', 'yan_gemm_bf16_tn_split_k', 'yan_gemm_fp16_tn_split_k', 'yan_gemm_select_split_k',
-           'yan_gemm_split_k_workspace_bytes', 'yan_gemm_split_k_counter_bytes', 'yan_gemm_version')
+           'yan_gemm_split_k_reset', 'yan_gemm_split_k_workspace_bytes', 'yan_gemm_split_k_counter_bytes', 'yan_gemm_version')
 
 
 def load() -> ctypes.CDLL:
@@ -32,6 +32,7 @@ def load() -> ctypes.CDLL:
         lib.yan_gemm_fp8_fp8_bf16_nt_split_k.argtypes = [vp, vp, ll, ll, vp, vp, vp, ci, ci, ci, vp, ci, vp, ll]
         lib.yan_gemm_select_split_k.argtypes = [ci, ci, ci, ci, ci, ctypes.POINTER(ci), ctypes.POINTER(ci), ctypes.POINTER(ci)]
         lib.yan_gemm_bf16_tn_split_k.argtypes = lib.yan_gemm_fp16_tn_split_k.argtypes = [ci, ci, ci, vp, vp, vp, vp, vp, ll]
+        lib.yan_gemm_split_k_reset.argtypes = [vp, vp]
         lib.yan_gemm_split_k_workspace_bytes.argtypes = lib.yan_gemm_split_k_counter_bytes.argtypes = []
         for name in SYMBOLS[:-1]:
             getattr(lib, name).restype = ci
@@ -91,6 +92,11 @@ def gemm_fp8_fp8_bf16_nt_static(lhs, rhs, out: torch.Tensor, num_sms: int = 0) -
     (m, k), n = a8.shape, b8.shape[0]
     return load().yan_gemm_fp8_fp8_bf16_nt_static(a8.data_ptr(), sa.data_ptr(), sa.stride(0), sa.stride(1), b8.data_ptr(),
                                                   sb.data_ptr(), out.data_ptr(), m, n, k, _stream_handle(), num_sms)
+
+
+def split_k_reset(workspace: torch.Tensor = None) -> int:
+    """Arrival counters of `workspace` (None: the library's own array on the current GPU) back to zero, on the current stream."""
+    return load().yan_gemm_split_k_reset(None if workspace is None else workspace.data_ptr(), _stream_handle())
 
 
 def gemm_bf16_tn_split_k(a: torch.Tensor, b: torch.Tensor, c: torch.Tensor, workspace: torch.Tensor) -> int:

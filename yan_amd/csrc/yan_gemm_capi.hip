@@ -294,6 +294,12 @@ int yan_gemm_fp8_fp8_bf16_nt_static(const void* lhs, const float* lhs_scales, lo
                      workspace, yan::kSplitKWorkspaceBytes);
 }
 
+// Arrival counters of a split-K workspace (the library's own array when `workspace` is null) back to zero, on `stream`.
+int yan_gemm_split_k_reset(void* workspace, void* stream) {
+    if (!workspace) workspace = static_scratch();
+    return int(yan::launch_split_k_reset(workspace, yan::kSplitKCounterBytes, static_cast<hipStream_t>(stream)));
+}
+
 int yan_m_grouped_gemm_fp8_fp8_bf16_nt_contiguous(const void* lhs, const float* lhs_scales, long long lhs_scales_stride_m,
                                                   long long lhs_scales_stride_k, const void* rhs, const float* rhs_scales,
                                                   void* out, const int* m_indices, int num_groups, int m, int n, int k,

@@ -159,6 +159,23 @@ meet_partials(Sums&& sums, float* __restrict__ partials, unsigned* __restrict__ 
     return true;
 }
 
+// Puts the arrival counters at the start of a split-K workspace back to zero: what a caller does once for a fresh
+// workspace, and again after anything that may have left a launch half done (a launch that reported an error, launches
+// that overlapped on one workspace). A fill kernel rather than a memset node, so the call may be captured into a graph.
+template <int = 0>      // a template so that only code that launches it carries it
+__global__ void __launch_bounds__(256) split_k_reset_kernel(unsigned* __restrict__ counters, int count) {
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i < count) __hip_atomic_store(counters + i, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+template <int V = 0>
+inline hipError_t launch_split_k_reset(void* workspace, size_t counter_bytes, hipStream_t stream) {
+    if (!workspace) return hipErrorInvalidValue;
+    const int count = int(counter_bytes / 4);
+    hipLaunchKernelGGL(split_k_reset_kernel<V>, dim3(ceil_div(count, 256)), dim3(256), 0, stream, static_cast<unsigned*>(workspace), count);
+    return hipGetLastError();
+}
+
 // Byte offset, relative to the first row of an R-row atom that starts at a multiple of 16 tile rows, of logical
 // chunk `chunk` of the row this lane owns.
 template <int R>

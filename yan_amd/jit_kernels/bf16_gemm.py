@@ -14,6 +14,7 @@ import torch
 
 from .heuristics import (get_best_dense_config, get_dense_num_stages, get_dense_tile_space, get_skinny_dense_config,
                          get_split_k_dense_config, tuning_enabled)
+from .split_k import SPLIT_K_WORKSPACE_BYTES, split_k_launch_failed, split_k_workspace
 from .tuner import FrozenKeys, jit_tuner
 from .utils import current_raw_stream, get_num_sms, get_num_sms_cap
 
@@ -97,20 +98,23 @@ def _gemm_16bit_tn(a: torch.Tensor, b: torch.Tensor, c: torch.Tensor, dtype: tor
 
     stream = current_raw_stream()
     args = (m, n, k, a, b, c, stream)
-    code_template = template
+    code_template, workspace_token = template, None
     if tuning_enabled() and not get_skinny_dense_config(m, n, k, get_num_sms()):
         name, keys, space, arg_defs = dense_tuning_plan(m, n, k, dtype, get_num_sms(), get_num_sms_cap())
     else:
         (name, keys, arg_defs), space = dense_kernel_plan(m, n, k, dtype, get_num_sms(), get_num_sms_cap()), ()
         split = dense_split_k_plan(m, n, k, dtype, get_num_sms())
         if split is not None:
-            from .gemm import SPLIT_K_WORKSPACE_BYTES, split_k_workspace
-            name, keys, arg_defs = split
-            code_template = split_k_template
-            args += (split_k_workspace(c.device, stream), SPLIT_K_WORKSPACE_BYTES)
+            workspace, workspace_token = split_k_workspace(c.device, stream)
+            if workspace is not None:
+                name, keys, arg_defs = split
+                code_template = split_k_template
+                args += (workspace, SPLIT_K_WORKSPACE_BYTES)
     runtime = jit_tuner.compile_and_tune(name=name, keys=keys, space=space, includes=includes,
                                          arg_defs=arg_defs, template=code_template, args=args)
     rc = runtime(*args)
+    if rc != 0 and workspace_token is not None:
+        split_k_launch_failed(workspace_token)
     assert rc == 0, f'{name} failed with HIP error {rc}'
 
 

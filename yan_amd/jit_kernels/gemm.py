@@ -17,6 +17,7 @@ import torch
 
 from .heuristics import (get_best_fp8_config, get_fp8_num_stages, get_fp8_tile_space, get_skinny_fp8_config,
                          get_split_k_fp8_config, tuning_enabled)
+from .split_k import SPLIT_K_COUNTER_BYTES, SPLIT_K_WORKSPACE_BYTES, split_k_launch_failed, split_k_workspace
 from .tuner import FrozenKeys, jit_tuner
 from .utils import current_raw_stream, get_num_sms, ceil_div, get_col_major_tensor, scales_for_kernel
 
@@ -84,26 +85,6 @@ split_k_template = _keys_block + _token_contiguous_scales + _split_k_launch
 split_k_strided_template = _keys_block + _split_k_launch
 split_k_arg_defs = arg_defs + (('workspace', torch.uint8), ('workspace_bytes', int))
 split_k_strided_arg_defs = split_k_arg_defs + (('lhs_scales_stride_m', int), ('lhs_scales_stride_k', int))
-# kSplitKCounterBytes and kSplitKWorkspaceBytes of gemm/fp8_gemm.hpp: arrival counters, then the partial sums of the
-# largest plan get_split_k_fp8_config makes.
-SPLIT_K_COUNTER_BYTES = 16 * 1024
-SPLIT_K_WORKSPACE_BYTES = SPLIT_K_COUNTER_BYTES + 256 * 128 * 128 * 4
-_split_k_workspaces = {}
-
-
-def split_k_workspace(device: torch.device, stream) -> torch.Tensor:
-    """The workspace split-K launches on `stream` (a Stream or its bare handle) share: one per device and stream, made (and
-    zeroed, on the current stream) at the first call and kept. Launches on one stream run one after the other, which is what sharing needs; the
-    counters at its start are zero again after every launch."""
-    key = (device.index, stream if isinstance(stream, int) else stream.cuda_stream)
-    workspace = _split_k_workspaces.get(key)
-    if workspace is None:
-        if len(_split_k_workspaces) >= 64:      # streams come and go: the oldest workspace returns to torch's allocator,
-            _split_k_workspaces.pop(next(iter(_split_k_workspaces)))      # which hands it out again in stream order
-        workspace = torch.zeros(SPLIT_K_WORKSPACE_BYTES, dtype=torch.uint8, device=device)
-        _split_k_workspaces[key] = workspace
-    return workspace
-
 
 @functools.lru_cache(maxsize=None)
 def fp8_kernel_plan(m: int, n: int, k: int, num_cus: int, token_contiguous_scales: bool = True):
@@ -189,7 +170,7 @@ def gemm_fp8_fp8_bf16_nt(lhs: Tuple[torch.Tensor, torch.Tensor],
     name, keys, defs, smem_size, code_template = fp8_kernel_plan(m, n, k, num_sms, token_contiguous)
     stream = current_raw_stream()
     args = (lhs, lhs_scales, rhs, rhs_scales, out, m, stream, num_sms, smem_size)
-    space = ()
+    space, workspace_token = (), None
     if tuning_enabled():
         tuning = fp8_tuning_plan(m, n, k, num_sms, token_contiguous)
         if tuning is not None:
@@ -197,11 +178,15 @@ def gemm_fp8_fp8_bf16_nt(lhs: Tuple[torch.Tensor, torch.Tensor],
     else:
         split = fp8_split_k_plan(m, n, k, num_sms, token_contiguous)
         if split is not None:
-            name, keys, defs, code_template = split
-            args += (split_k_workspace(out.device, stream), SPLIT_K_WORKSPACE_BYTES)
+            workspace, workspace_token = split_k_workspace(out.device, stream)
+            if workspace is not None:
+                name, keys, defs, code_template = split
+                args += (workspace, SPLIT_K_WORKSPACE_BYTES)
     if not token_contiguous:
         args += (stride_m, stride_k)
     runtime = jit_tuner.compile_and_tune(name=name, keys=keys, space=space, includes=includes,
                                          arg_defs=defs, template=code_template, args=args)
     rc = runtime(*args)
+    if rc != 0 and workspace_token is not None:
+        split_k_launch_failed(workspace_token)
     assert rc == 0, f'{name} failed with HIP error {rc}'
