@@ -219,6 +219,9 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
+    # The same measurement without the settle phase, coming from an idle chip: what a caller gets for its first launches.
+    time.sleep(0.5)
+    idle_kernel_ms, idle_wall_ms = _event_time_ms(step, args.steps, args.warmup, 0)
     kernel_ms, wall_ms = _event_time_ms(step, args.steps, args.warmup, settle['cfg3'])
     # validity of what was timed: sampled rows against an fp32 matmul of the dequantised operands
     diff = _sampled_fp8_diff(yan, harness, a8, sa, b8, sb, out)
@@ -240,6 +243,9 @@ def main():
                    'settle_launches': settle['cfg3'],
                    'settle': 'untimed launches of the same kernel before the warm-up: the power controller takes ~100 launches '
                              'to settle after an idle period',
+                   'tflops_from_idle': round(2.0 * m * n * k / (idle_wall_ms * 1e-3) / 1e12, 1),
+                   'kernel_us_from_idle': round(idle_kernel_ms * 1e3, 2),
+                   'from_idle': 'the same warm-up and timed steps after half a second of idle and no settle launches; `value` is the settled figure',
                    'calc_diff_sampled_rows': diff},
         'roofline': {'bound': 'mfma', 'achieved': round(tflops_kernel, 1), 'peak': PEAK_FP8_TFLOPS, 'unit': 'TFLOP/s',
                      'frac': round(tflops_kernel / PEAK_FP8_TFLOPS, 4), 'traffic': traffic,
@@ -332,7 +338,24 @@ def main():
                                             'frac_of_hbm_peak_warm': round(byt / t_warm / 1e9 / PEAK_HBM_GBPS, 4),
                                             'frac_of_hbm_peak_cold': round(byt / t_cold / 1e9 / PEAK_HBM_GBPS, 4),
                                             'calc_diff': d}
-        del x8, sx, w8, sw, o
+        # The same decode step from bf16 activations: the quantiser and the GEMM as two entry calls, and as the one call of the
+        # entry that enqueues both from one `launch` (same kernels, same bits; what differs is the host's share).
+        xb = torch.randn(mm, kk, device='cuda', generator=torch.Generator(device='cuda').manual_seed(42)).bfloat16()
+        two_calls = lambda: yan.gemm_fp8_fp8_bf16_nt(yan.per_token_cast_to_fp8(xb, col_major_scales=True), (w8, sw), o)
+        one_call = lambda: yan.gemm_bf16_fp8_bf16_nt(xb, (w8, sw), o)
+        two_calls()
+        torch.cuda.synchronize()
+        expect = o.clone()
+        one_call()
+        torch.cuda.synchronize()
+        assert torch.equal(o, expect), 'the chained entry lost the bits of quantiser + GEMM'
+        _, wall_two = _event_time_ms(two_calls, 500, 50, 0)
+        _, wall_one = _event_time_ms(one_call, 500, 50, 0)
+        t_cast = yan.bench_kineto(one_call, 'per_token_cast', suppress_kineto_output=True)
+        extra['fp8_decode_64x4096x7168']['from_bf16_activations'] = {
+            'call_to_call_us_quantiser_then_gemm_two_calls': round(wall_two * 1e3, 2),
+            'call_to_call_us_one_call': round(wall_one * 1e3, 2), 'quantiser_kernel_us': round(t_cast * 1e6, 2), 'same_bits': True}
+        del x8, sx, w8, sw, o, xb
         # configs[4]: FP8 16384^3, uniform[-4, 4] sources with 1 % of the entries x 50
         mm, nn, kk = harness.BASELINE_FP8['cfg5']
         (x8, sx), (w8, sw), o = harness.make_fp8_case(mm, nn, kk, seed=42, dist='outlier', device='cuda', gen_device='cuda')

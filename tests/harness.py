@@ -211,6 +211,10 @@ FP8_SPLIT_K_PLAN_OF_SHAPE = {
     (300, 4100, 6144): (128, 128, 2), (200, 4100, 5376): (128, 128, 3), (129, 4096, 7168): (128, 128, 4),
     (64, 4096, 7168): (64, 64, 4), (128, 4096, 7168): (64, 128, 4), (5, 3076, 6144): (32, 32, 2), (1, 4096, 7168): (32, 32, 2),
 }
+# bf16 activations through the entry that chains the quantiser and the GEMM in one `launch`: a split-K plan, the weight-
+# streaming kernel, unsplit tiles, rows that are no multiple of anything, and one whose codes do not fit the entry's scratch
+# (two entry calls instead).
+CAST_CHAIN_SHAPES = [(64, 4096, 7168), (1, 4096, 7168), (33, 2112, 5376), (7, 96, 640), (300, 2112, 1024), (512, 4096, 2048), (1100, 512, 4096)]
 FP8_SPLIT_K_SHAPES = [s for s in FP8_SPLIT_K_PLAN_OF_SHAPE if s not in ((64, 4096, 7168), (128, 4096, 7168), (1, 4096, 7168))]
 # The same for the dense GEMMs: the three tiles split-K plans use, every factor, ragged m and n, n that is no multiple of 8,
 # k tails (3080 = 48 k-tiles and 8 elements, 7176), a dozen rows (where a plan goes before the weight-streaming kernel), six and
@@ -322,6 +326,18 @@ def jit_kernels_in_use(num_cus: int = 256):
             if split is not None:
                 name, keys, arg_defs, code_template = split
                 add(name, arg_defs, gemm.includes, code_template, keys)
+    for m, n, k in CAST_CHAIN_SHAPES:
+        chain = gemm.fp8_cast_chain_plan(m, n, k, num_cus)
+        if chain is not None:
+            name, keys, arg_defs, code_template, _ = chain
+            add(name, arg_defs, gemm.cast_includes, code_template, keys)
+        # what two entry calls run for the same sizes
+        name, keys, arg_defs, _, code_template = gemm.fp8_kernel_plan(m, n, k, num_cus, True)
+        add(name, arg_defs, gemm.includes, code_template, keys)
+        split = gemm.fp8_split_k_plan(m, n, k, num_cus, True)
+        if split is not None:
+            name, keys, arg_defs, code_template = split
+            add(name, arg_defs, gemm.includes, code_template, keys)
     for m, n, k in CAPPED_SHAPES:
         for cus, cap in ((num_cus, 0), (num_cus, NUM_SMS_CAP), (NUM_SMS_CAP, NUM_SMS_CAP)):
             name, keys, arg_defs = bf16_gemm.dense_kernel_plan(m, n, k, torch.bfloat16, cus, cap)

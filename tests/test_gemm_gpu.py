@@ -1242,6 +1242,40 @@ def test_a_workspace_whose_launch_failed_is_cleared_before_its_next_use(monkeypa
     assert float(yan.calc_diff(unsplit.float(), ref)) < 1e-5 and float(yan.calc_diff(unsplit.float(), want.float())) < 1e-8
 
 
+@pytest.mark.parametrize('m,n,k', testing.CAST_CHAIN_SHAPES)
+def test_bf16_activation_entry_gives_the_bits_of_quantiser_then_gemm(m, n, k):
+    """gemm_bf16_fp8_bf16_nt: one call, one `launch` that enqueues the quantiser and the GEMM, the codes in the entry's own
+    scratch: the bits of per_token_cast_to_fp8 followed by gemm_fp8_fp8_bf16_nt, within the FP8 bar of the oracle's
+    quantise-then-multiply on the same bf16 inputs, rows past m untouched, and nothing allocated per call."""
+    from yan_amd.jit_kernels import gemm as fp8_entry
+    _announce('bf16 activations', m, n, k)
+    g = torch.Generator().manual_seed(97 + m)
+    x = torch.randn(m, k, generator=g).bfloat16()
+    w = torch.randn(n, k, generator=g).bfloat16()
+    b8, sb = testing.per_block_cast_to_fp8(w.float())
+    xd, b8d, sbd = x.cuda(), b8.cuda(), sb.cuda()
+    chained = fp8_entry.fp8_cast_chain_plan(m, n, k, yan.get_num_sms()) is not None
+    assert chained == ((m, n, k) != (1100, 512, 4096))
+    two = torch.zeros(m, n, dtype=torch.bfloat16, device='cuda')
+    yan.gemm_fp8_fp8_bf16_nt(yan.per_token_cast_to_fp8(xd, col_major_scales=True), (b8d, sbd), two)
+    one = torch.full((m + 3, n), 7.0, dtype=torch.bfloat16, device='cuda')
+    yan.gemm_bf16_fp8_bf16_nt(xd, (b8d, sbd), one[:m])
+    torch.cuda.synchronize()
+    assert torch.equal(one[:m], two) and bool((one[m:] == 7.0).all())
+    a8, sa = oracle.per_token_cast_to_fp8(x.float().numpy())
+    ref = oracle.gemm_fp8_block_scaled_ref(a8, sa, _np(b8), _np(sb))
+    assert oracle.calc_diff(_np(one[:m]), ref) < FP8_TOL
+    if chained:
+        target = one[:m]
+        yan.gemm_bf16_fp8_bf16_nt(xd, (b8d, sbd), target)
+        torch.cuda.synchronize()
+        allocated = torch.cuda.memory_allocated()
+        for _ in range(3):
+            yan.gemm_bf16_fp8_bf16_nt(xd, (b8d, sbd), target)
+        torch.cuda.synchronize()
+        assert torch.cuda.memory_allocated() == allocated and torch.equal(target, two)
+
+
 def test_capi_seeded_random_shapes_against_device_references():
     """Breadth: 240 seeded random shapes through the C entries (every tile variant, ragged edges, k tails, leading
     dimensions), each against an fp32 / fp64 product of the same operands on the device. The oracle-based tests above

@@ -454,3 +454,28 @@ def test_split_k_workspaces_are_kept_per_stream_and_per_capture():
     assert (0, 111) not in book.eager and len(book.eager) == 3 and (0, 111) not in book.suspect
     assert book.get(0, 111) is not w0 and cleared == [w1]       # a fresh one: nothing to clear
     assert len(book.captures) == 3 and book.get(0, 1, capture=8) is c8 and w3 is book.get(2, 5)
+
+
+def test_the_bf16_activation_entry_chains_the_quantiser_in_front_of_whatever_the_gemm_entry_runs():
+    """`fp8_cast_chain_plan`: the keys of the GEMM plan the FP8 entry uses for the sizes (split-K plan, weight-streaming kernel
+    or tiles) plus the scratch offset, a `launch` whose arguments are the GEMM's without the quantised operands, and code
+    that calls the quantiser before the GEMM's launch; None when the codes do not fit the scratch."""
+    import harness as testing
+    from yan_amd.jit import cpp_format
+    from yan_amd.jit_kernels.split_k import SPLIT_K_WORKSPACE_BYTES, WORKSPACE_ALLOCATION_BYTES
+    assert WORKSPACE_ALLOCATION_BYTES == SPLIT_K_WORKSPACE_BYTES + gemm.CAST_SCRATCH_BYTES
+    for m, n, k in testing.CAST_CHAIN_SHAPES:
+        plan = gemm.fp8_cast_chain_plan(m, n, k, 256)
+        if m * k + m * (k // 128) * 4 + 256 > gemm.CAST_SCRATCH_BYTES:
+            assert plan is None
+            continue
+        name, keys, arg_defs, code_template, smem_size = plan
+        split = gemm.fp8_split_k_plan(m, n, k, 256, True)
+        inner_keys, inner_defs = (split[1], split[2]) if split is not None else gemm.fp8_kernel_plan(m, n, k, 256, True)[1:3]
+        assert name == 'gemm_bf16_fp8_bf16_nt' and dict(keys) == {**inner_keys, 'SCRATCH_OFFSET': SPLIT_K_WORKSPACE_BYTES}
+        assert [d[0] for d in arg_defs] == ['x', 'buffer', 'scratch_bytes'] + [d[0] for d in inner_defs if d[0] not in ('lhs', 'lhs_scales')]
+        code = cpp_format(code_template, keys)
+        assert code.index('launch_per_token_cast(') < code.index('__return_code = static_cast<int>(', code.index('launch_per_token_cast(') + 1)
+        assert '{' + 'SCRATCH_OFFSET' + '}' not in code and smem_size > 0
+    # without split-K (YAN_SPLIT_K=0 leaves the entries without memory of their own) the entry makes two calls; the plan for it is not asked
+    assert gemm.fp8_cast_chain_plan(64, 4096, 7168, 256, False)[1].get('SPLIT_K') is None

@@ -66,6 +66,21 @@ __return_code = static_cast<int>(GemmType::run_split_k<{SPLIT_K}>(out, lhs, lhs_
                                                                   rhs, rhs_scales, m, N, K, stream, workspace, workspace_bytes));
 """
 
+# bf16 activations: the quantiser and the GEMM enqueued by one `launch` (gemm_bf16_fp8_bf16_nt below). The codes and their
+# token-contiguous scales go to the scratch area behind the split-K workspace proper; the GEMM launch is one of the three above.
+_cast_prologue = """
+// Quantise the activations into the scratch area behind the split-K workspace: codes [m, K], then scales with element (i, kb) at kb * m + i
+static_assert(K % 128 == 0);
+if (scratch_bytes < int64_t(m) * K + 256 + int64_t(m) * (K / 128) * 4) { __return_code = static_cast<int>(hipErrorInvalidValue); return; }
+uint8_t* scratch = buffer + {SCRATCH_OFFSET};
+__hip_fp8_e4m3* lhs = reinterpret_cast<__hip_fp8_e4m3*>(scratch);
+float* lhs_scales = reinterpret_cast<float*>(scratch + ((int64_t(m) * K + 255) / 256) * 256);
+__return_code = static_cast<int>(launch_per_token_cast(reinterpret_cast<const __bf16*>(x), lhs, lhs_scales, 1, m, m, K, stream));
+if (__return_code != 0) return;
+"""
+_cast_arg_defs_head = (('x', torch.bfloat16), ('buffer', torch.uint8), ('scratch_bytes', int))
+cast_includes = includes + ('"gemm/fp8_cast.hpp"', )
+
 # The reference's keys and run-time names, nothing else (yan/jit_kernels/gemm.py:9-30): code that formats this template
 # with `N, K, BLOCK_M, BLOCK_N, NUM_STAGES, NUM_TMA_MULTICAST` and builds it with `arg_defs` gets the kernel for
 # token-contiguous activation scales.
@@ -188,5 +203,74 @@ def gemm_fp8_fp8_bf16_nt(lhs: Tuple[torch.Tensor, torch.Tensor],
                                          arg_defs=defs, template=code_template, args=args)
     rc = runtime(*args)
     if rc != 0 and workspace_token is not None:
+        split_k_launch_failed(workspace_token)
+    assert rc == 0, f'{name} failed with HIP error {rc}'
+
+
+# Scratch of the chained entry: behind the 16 MB of the split-K workspace, room for the codes and scales of up to
+# CAST_SCRATCH_BYTES / (k + k / 32) rows (64 rows of K = 65536, 1024 rows of K = 4096).
+CAST_SCRATCH_BYTES = 4 << 20
+
+
+@functools.lru_cache(maxsize=None)
+def fp8_cast_chain_plan(m: int, n: int, k: int, num_cus: int, split_k_allowed: bool = True):
+    """(name, keys, arg_defs, template, smem_size) of the kernel.so whose `launch` enqueues the per-token quantiser and then the
+    GEMM the FP8 entry would run for these sizes (split-K plan, weight-streaming kernel or tiles), or None when the codes
+    and scales of `m` rows do not fit the scratch area; needs no GPU."""
+    if m <= 0 or m * k + m * (k // 128) * 4 + 256 > CAST_SCRATCH_BYTES:
+        return None
+    split = fp8_split_k_plan(m, n, k, num_cus, True) if split_k_allowed else None
+    if split is not None:
+        _, keys, defs, code_template = split
+        smem_size = keys['NUM_STAGES'] * (keys['BLOCK_M'] + keys['BLOCK_N']) * 128
+    else:
+        _, keys, defs, smem_size, code_template = fp8_kernel_plan(m, n, k, num_cus, True)
+    # the inner templates start with the keys block and the stride definitions; the prologue goes between those and the launch
+    head = _keys_block + _token_contiguous_scales
+    assert code_template.startswith(head)
+    chained = head + _cast_prologue + code_template[len(head):]
+    inner = tuple(d for d in defs if d[0] not in ('lhs', 'lhs_scales'))
+    keys = FrozenKeys({**keys, 'SCRATCH_OFFSET': SPLIT_K_WORKSPACE_BYTES})
+    return 'gemm_bf16_fp8_bf16_nt', keys, _cast_arg_defs_head + inner, chained, smem_size
+
+
+def gemm_bf16_fp8_bf16_nt(x: torch.Tensor, rhs: Tuple[torch.Tensor, torch.Tensor], out: torch.Tensor) -> None:
+    """`gemm_fp8_fp8_bf16_nt(per_token_cast_to_fp8(x, col_major_scales=True), rhs, out)` for bf16 activations `x` `[m, k]`,
+    bit for bit (the same two kernels), as ONE call: one trip through Python and one `launch`, which enqueues the quantiser and
+    the GEMM back to back; the codes and scales live in scratch memory the entry keeps per stream, so nothing is allocated
+    per call. What a decode step saves is host time: two entry calls cost 18-22 us of Python, which is more than both
+    kernels take on the device (64 x 4096 x 7168: 21.7 -> about 13 us call to call). The reference names only the GEMM's
+    operands (`yan/jit_kernels/gemm.py:23-30`); the chain of torch ops its callers put in front of it is what this takes
+    out of the decode latency. Quantising inside the GEMM kernel itself was built and measured, and is slower than the two
+    kernels: every one of the 64 workgroups that share a K range repeats the quantisation of its 64 x 1792 activations,
+    9.6 us of vector arithmetic per workgroup against 2.5 us for the quantiser kernel spread over the chip (21.5 us in one
+    kernel against 3 + 9.7 us in two; same bits). Problems whose codes do not fit the scratch area (or with
+    `YAN_SPLIT_K=0`, which means no memory kept by the entries) run the two entries one after the other."""
+    from .fp8_cast import per_token_cast_to_fp8
+    from .split_k import split_k_enabled
+    rhs_q, rhs_scales = rhs
+    m, k = x.shape
+    n, k_ = rhs_q.shape
+    assert x.dtype == torch.bfloat16 and out.dtype == torch.bfloat16 and rhs_q.dtype == torch.float8_e4m3fn and rhs_scales.dtype == torch.float32
+    assert out.shape == (m, n) and k == k_ and n % 4 == 0 and k % 128 == 0
+    assert rhs_scales.shape == (ceil_div(n, 128), ceil_div(k, 128))
+    assert x.is_contiguous() and rhs_q.is_contiguous() and out.is_contiguous() and rhs_scales.is_contiguous()
+    if m == 0:
+        return
+    num_sms = get_num_sms()
+    plan = fp8_cast_chain_plan(m, n, k, num_sms) if split_k_enabled() and not tuning_enabled() else None
+    if plan is None:
+        gemm_fp8_fp8_bf16_nt(per_token_cast_to_fp8(x, col_major_scales=True), rhs, out)
+        return
+    name, keys, defs, code_template, smem_size = plan
+    stream = current_raw_stream()
+    workspace, workspace_token = split_k_workspace(out.device, stream)
+    values = {'x': x, 'buffer': workspace, 'scratch_bytes': CAST_SCRATCH_BYTES, 'rhs': rhs_q, 'rhs_scales': rhs_scales,
+              'out': out, 'm': m, 'stream': stream, 'num_sms': num_sms, 'smem_size': smem_size, 'workspace': workspace,
+              'workspace_bytes': SPLIT_K_WORKSPACE_BYTES}
+    args = tuple(values[d[0]] for d in defs)
+    runtime = jit_tuner.compile_and_tune(name=name, keys=keys, space=(), includes=cast_includes, arg_defs=defs, template=code_template, args=args)
+    rc = runtime(*args)
+    if rc != 0:
         split_k_launch_failed(workspace_token)
     assert rc == 0, f'{name} failed with HIP error {rc}'

@@ -23,6 +23,9 @@ import torch
 # largest plan the heuristics make.
 SPLIT_K_COUNTER_BYTES = 16 * 1024
 SPLIT_K_WORKSPACE_BYTES = SPLIT_K_COUNTER_BYTES + 256 * 128 * 128 * 4
+# what the entries allocate per workspace: the split-K workspace proper, then scratch for the chained quantiser + GEMM entry
+# (codes and scales of the activations: gemm.CAST_SCRATCH_BYTES)
+WORKSPACE_ALLOCATION_BYTES = SPLIT_K_WORKSPACE_BYTES + (4 << 20)
 MAX_EAGER_WORKSPACES = 8
 
 
@@ -70,7 +73,7 @@ class WorkspaceBook:
 
 
 def _make_workspace() -> torch.Tensor:
-    workspace = torch.empty(SPLIT_K_WORKSPACE_BYTES, dtype=torch.uint8, device='cuda')
+    workspace = torch.empty(WORKSPACE_ALLOCATION_BYTES, dtype=torch.uint8, device='cuda')
     workspace[:SPLIT_K_COUNTER_BYTES].zero_()         # a fill kernel: may be recorded into a graph
     return workspace
 
@@ -113,15 +116,30 @@ def capture_id(stream: int) -> Optional[int]:
     return int(ident.value) if status.value == 1 else None         # hipStreamCaptureStatusActive
 
 
+_is_capturing = getattr(torch._C, '_cuda_isCurrentStreamCapturing', None) or torch.cuda.is_current_stream_capturing
+_last = (None, None)            # (token, workspace) of the latest eager launch: the usual next one
+
+
 def split_k_workspace(device: torch.device, stream: int):
     """(workspace, token) for a split-K launch on `stream` (the bare handle of the current stream), or (None, None) when
     split-K is switched off. Hand `token` to `split_k_launch_failed` if the launch reports an error."""
-    if not split_k_enabled():
+    global _last
+    if os.environ.get('YAN_SPLIT_K', '1') in ('', '0'):
         return None, None
-    capture = capture_id(stream) if torch.cuda.is_current_stream_capturing() else None
-    index = device.index if device.index is not None else torch.cuda.current_device()
-    return _book.get(index, stream, capture), (index, stream, capture)
+    capture = capture_id(stream) if _is_capturing() else None
+    index = device.index
+    if index is None:
+        index = torch.cuda.current_device()
+    token = (index, stream, capture)
+    if token == _last[0]:
+        return _last[1], token
+    workspace = _book.get(index, stream, capture)
+    if capture is None:
+        _last = (token, workspace)
+    return workspace, token
 
 
 def split_k_launch_failed(token) -> None:
+    global _last
+    _last = (None, None)
     _book.launch_failed(*token)
