@@ -412,7 +412,9 @@ def main():
         del x8, sx, w8, sw, o, idx
         # groups whose boundaries fall in the middle of 256-row tiles (every other one): 8 groups of 896 and 1152 rows, next to
         # 8 groups of 1024 rows
-        for label, rows in (('8x896_1152', (896, 1152) * 4), ('8x1024', (1024,) * 8)):
+        # and groups of a few hundred rows, which run the kernel that picks its tile height on the device: 256 x 256 tiles when every
+        # boundary falls on a multiple of 256 rows (16 groups of 512), 128 x 256 when not (16 groups of 384 and 640)
+        for label, rows in (('8x896_1152', (896, 1152) * 4), ('8x1024', (1024,) * 8), ('16x512', (512,) * 16), ('16x384_640', (384, 640) * 8)):
             (x8, sx), (w8, sw), o, idx = harness.make_grouped_contiguous_case(rows, nn, kk, seed=42, device='cuda', gen_device='cuda')
             sx = yan.get_col_major_tensor(sx)
             ms, _ = _event_time_ms(lambda: yan.m_grouped_gemm_fp8_fp8_bf16_nt_contiguous((x8, sx), (w8, sw), o, idx), 30, 5, 150)

@@ -242,7 +242,13 @@ GROUPED_CONTIGUOUS_TEST_CASES = [
     # long groups whose boundaries fall in the middle of 256-row tiles (two-pass tiles), with a trailing padding block
     ((1150, 900, 1300, 1100), 512, 512, 1),
     ((128, 128), 192, 256, 1),                       # the committed fixture
+    # groups of a few hundred rows run the kernel that picks its tile height on the device: every boundary on a multiple of 256 rows
+    # (it takes 256 x 256 tiles), every other one in the middle of such a tile (128 x 256 tiles)
+    ((512,) * 16, 4096, 1024, 0), ((384, 640) * 8, 4096, 1024, 1),
 ]
+# The same kernel built for small problems through explicit keys (the cost table gives those to smaller tiles): whole
+# 256-row tiles, two groups in every other tile row, and a padding block in the middle with one boundary off.
+GROUPED_ROWS_ON_DEVICE_CASES = [((512,) * 6, 768, 512, 0), ((384, 640) * 3, 768, 512, 1), ((512, 256, -128, 500, 512), 768, 384, 0)]
 GROUPED_MASKED_TEST_CASES = [
     (3, 200, 320, 384, (200, 0, 77), 128), (4, 256, 4096, 1024, (1, 256, 130, 64), 64), (2, 64, 200, 128, (64, 3), 32),
     (4, 1024, 4096, 7168, (1024, 900, 512, 1), 1024),
@@ -293,6 +299,15 @@ def fp8_explicit_tile_plan(block_m: int, block_n: int, n: int, k: int):
     keys = {'N': n, 'K': k, 'BLOCK_M': block_m, 'BLOCK_N': block_n, 'NUM_STAGES': get_fp8_num_stages(block_m, block_n),
             'NUM_TMA_MULTICAST': 1}
     return 'gemm_fp8_fp8_bf16_nt', keys, gemm.arg_defs, gemm.template
+
+
+def grouped_rows_on_device_plan(num_groups: int, n: int, k: int):
+    """(name, keys, arg_defs, template) of the contiguous grouped kernel that picks its tile height on the device, whatever the
+    cost table would give the problem."""
+    from yan_amd.jit_kernels import m_grouped_gemm
+    keys = {'N': n, 'K': k, 'BLOCK_M': 256, 'BLOCK_N': 256, 'NUM_GROUPS': num_groups, 'NUM_STAGES': 2, 'NUM_TMA_MULTICAST': 1,
+            'GEMM_TYPE': 'GroupedContiguous', 'ROWS': 'picked on the device'}
+    return 'm_grouped_gemm_fp8_fp8_bf16_nt_rows_on_device', keys, m_grouped_gemm.arg_defs, m_grouped_gemm.rows_on_device_template
 
 
 def jit_kernels_in_use(num_cus: int = 256):
@@ -368,14 +383,21 @@ def jit_kernels_in_use(num_cus: int = 256):
     for rows, n, k, pad_blocks in GROUPED_CONTIGUOUS_TEST_CASES:
         m = sum((abs(r) + 127) // 128 * 128 for r in rows) + 128 * pad_blocks
         name, keys, arg_defs, _ = m_grouped_gemm.grouped_kernel_plan('GroupedContiguous', sum(1 for r in rows if r > 0), m, n, k, num_cus)
-        add(name, arg_defs, m_grouped_gemm.includes, m_grouped_gemm.template, keys)
+        add(name, arg_defs, m_grouped_gemm.includes, m_grouped_gemm.rows_on_device_template if 'ROWS' in keys else m_grouped_gemm.template, keys)
     for groups, m_max, n, k, _, expected_m in GROUPED_MASKED_TEST_CASES:
         name, keys, arg_defs, _ = m_grouped_gemm.grouped_kernel_plan('GroupedMasked', groups, min(expected_m, m_max), n, k, num_cus)
         add(name, arg_defs, m_grouped_gemm.includes, m_grouped_gemm.template, keys)
+    # contiguous layouts only the benchmark's --also legs run
+    for rows, n, k in (((896, 1152) * 4, 4096, 7168), ((1024,) * 8, 4096, 7168), ((512,) * 16, 4096, 7168), ((384, 640) * 8, 4096, 7168)):
+        name, keys, arg_defs, _ = m_grouped_gemm.grouped_kernel_plan('GroupedContiguous', len(rows), sum(rows), n, k, num_cus)
+        add(name, arg_defs, m_grouped_gemm.includes, m_grouped_gemm.rows_on_device_template if 'ROWS' in keys else m_grouped_gemm.template, keys)
+    for rows, n, k, _ in GROUPED_ROWS_ON_DEVICE_CASES:
+        name, keys, arg_defs, code_template = grouped_rows_on_device_plan(sum(1 for r in rows if r > 0), n, k)
+        add(name, arg_defs, m_grouped_gemm.includes, code_template, keys)
     # the grouped layouts under the compute-unit cap: tiles chosen for NUM_SMS_CAP units
     rows, n, k, pad_blocks = GROUPED_TWO_GROUP_ROWS_FIRST_CASE
     name, keys, arg_defs, _ = m_grouped_gemm.grouped_kernel_plan('GroupedContiguous', len(rows), sum(rows) + 128 * pad_blocks, n, k, NUM_SMS_CAP)
-    add(name, arg_defs, m_grouped_gemm.includes, m_grouped_gemm.template, keys)
+    add(name, arg_defs, m_grouped_gemm.includes, m_grouped_gemm.rows_on_device_template if 'ROWS' in keys else m_grouped_gemm.template, keys)
     groups, m_max, n, k, _, expected_m = GROUPED_MASKED_TEST_CASES[6]
     name, keys, arg_defs, _ = m_grouped_gemm.grouped_kernel_plan('GroupedMasked', groups, min(expected_m, m_max), n, k, NUM_SMS_CAP)
     add(name, arg_defs, m_grouped_gemm.includes, m_grouped_gemm.template, keys)

@@ -47,10 +47,14 @@ def test_version_and_tile_selection_match_python(lib):
         for cus in (256, 128, 80):
             assert capi.select_tile(0, m, n, k, cus) == heuristics.get_dense_tile(m, n, k, cus), (m, n, k, cus)
             assert capi.select_tile(1, m, n, k, cus) == heuristics.get_fp8_tile(m, n, k, cus), (m, n, k, cus)
-    for m, n in [(4096, 4096), (32768, 4096), (128, 7168), (256, 200), (1024, 24576)]:
+    picked_on_device = 0
+    for m, n in [(4096, 4096), (32768, 4096), (128, 7168), (256, 200), (1024, 24576), (8192, 4096), (8192, 7168), (6144, 2112), (16384, 4096)]:
         for cus in (256, 80):
-            for groups in (1, 4, 64):
+            for groups in (1, 4, 8, 16, 64):
                 assert capi.select_tile(2, m, n, groups, cus) == heuristics.get_best_grouped_fp8_config(m, n, 1024, cus, 1, 128, groups)
+                assert capi.select_tile(4, m, n, groups, cus) == ((256, 256) if heuristics.get_contiguous_rows_on_device(m, n, 1024, cus, groups) else (0, 0))
+                picked_on_device += heuristics.get_contiguous_rows_on_device(m, n, 1024, cus, groups)
+    assert picked_on_device >= 6
     for m, n in [(128, 2112), (128, 24576), (128, 32768), (128, 7168), (4096, 7168), (4096, 2112), (4096, 32768), (128, 64), (5120, 2048),
                  (256, 256), (512, 4096), (1024, 1024), (2048, 2048), (256, 32768)]:
         for cus in (256, 80):

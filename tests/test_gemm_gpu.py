@@ -977,6 +977,9 @@ def test_grouped_contiguous_parity(rows, n, k, pad_blocks):
         halves = blocks[:len(blocks) // 2 * 2].view(-1, 2)
         two = ((halves[:, 0] != halves[:, 1]) & (halves >= 0).all(1)).nonzero().flatten()
         assert len(two) == 8 and int(two.min()) < 64 <= int(two.max()) and (m + 255) // 256 > 64
+    if rows in ((512,) * 16, (384, 640) * 8):
+        from yan_amd.jit_kernels.m_grouped_gemm import grouped_kernel_plan
+        assert grouped_kernel_plan('GroupedContiguous', len(group_rows), m, n, k, 256)[1].get('ROWS') == 'picked on the device'
     a8d, sad, b8d, sbd, idxd = a8.cuda(), sa.cuda(), b8.cuda(), sb.cuda(), idx.cuda()
     got = out.cuda()
     assert yan.m_grouped_gemm_fp8_fp8_bf16_nt_contiguous((a8d, sad), (b8d, sbd), got, idxd) is None
@@ -1016,6 +1019,38 @@ def test_grouped_contiguous_parity(rows, n, k, pad_blocks):
     plain = torch.zeros(r0, n, dtype=torch.bfloat16, device='cuda')
     yan.gemm_fp8_fp8_bf16_nt((a8d[:r0], sad[:r0].contiguous()), (b8d[0], sbd[0]), plain)
     assert float(yan.calc_diff(plain.float(), got[:r0].float())) < 1e-9
+
+
+@pytest.mark.parametrize('rows,n,k,pad_blocks', testing.GROUPED_ROWS_ON_DEVICE_CASES)
+def test_grouped_contiguous_kernel_that_picks_its_tile_height_on_the_device(rows, n, k, pad_blocks):
+    """fp8_gemm_contiguous_rows_kernel on problems small enough for the oracle in full: with every group boundary on a
+    multiple of 256 rows it runs 256 x 256 tiles, otherwise 128 x 256 ones; either way the oracle's result, the bits of the
+    entry (which gives problems this small to other tiles: all tiles form the same sums), padding blocks untouched, and
+    the same again under a compute-unit cap, where workgroups walk several tiles."""
+    _announce('grouped rows on device', rows, n, k)
+    (a8, sa), (b8, sb), out, idx = testing.make_grouped_contiguous_case(rows, n, k, seed=21, padding_blocks=pad_blocks)
+    m, groups = a8.size(0), sum(1 for r in rows if r > 0)
+    blocks = idx.view(-1, 128)[:, 0]
+    halves = blocks[:len(blocks) // 2 * 2].view(-1, 2)
+    two_group_rows = int(((halves[:, 0] != halves[:, 1]) & (halves >= 0).all(1)).sum())
+    assert (two_group_rows == 0) == (rows == (512,) * 6)              # the first case is the one that runs 256-row tiles
+    name, keys, arg_defs, code_template = testing.grouped_rows_on_device_plan(groups, n, k)
+    from yan_amd.jit_kernels import m_grouped_gemm
+    kernel = jit.build(name, arg_defs, jit.generate(m_grouped_gemm.includes, arg_defs, jit.cpp_format(code_template, keys)))
+    a8d, sad, b8d, sbd, idxd = a8.cuda(), sa.cuda(), b8.cuda(), sb.cuda(), idx.cuda()
+    ref = torch.from_numpy(oracle.m_grouped_gemm_contiguous_ref(_np_codes(a8), sa.numpy(), _np_codes(b8), sb.numpy(), idx.numpy(),
+                                                                out_init=out.float().numpy()))
+    via_entry = out.cuda()
+    yan.m_grouped_gemm_fp8_fp8_bf16_nt_contiguous((a8d, sad), (b8d, sbd), via_entry, idxd)
+    for cap in (yan.get_num_sms(), 8):
+        got = out.cuda()
+        assert kernel(a8d, sad, b8d, sbd, got, idxd, m, torch.cuda.current_stream(), cap, 0, sad.stride(0), sad.stride(1), 0, 0) == 0
+        torch.cuda.synchronize()
+        assert float(yan.calc_diff(got.float().cpu(), ref)) < 1e-3
+        real = idx >= 0
+        assert torch.equal(got.cpu()[~real], out[~real])
+        assert bool(((got.float().cpu() - ref).abs() <= ref.abs() * 2.0 ** -7 + 1e-4 * ref.abs().max())[real].all())
+        assert torch.equal(got, via_entry)
 
 
 @pytest.mark.parametrize('groups,m_max,n,k,masked,expected_m', testing.GROUPED_MASKED_TEST_CASES)

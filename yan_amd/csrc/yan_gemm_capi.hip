@@ -55,6 +55,26 @@ void pick_grouped(int m, int n, int num_cus, int groups, int m_alignment, int gr
     }
 }
 
+// Whether a contiguous grouped GEMM runs the kernel that picks its tile height on the device (get_contiguous_rows_on_device in
+// heuristics.py): groups of 256 to 1023 rows on average that get 128 x 256 tiles but would get 256 x 256 ones if none held two groups.
+bool rows_on_device(int m, int n, int num_cus, int groups_in_m) {
+    if (groups_in_m <= 0 || (long long)m < 256ll * groups_in_m || (long long)m >= 1024ll * groups_in_m) return false;
+    int bm = 0, bn = 0;
+    pick_grouped(m, n, num_cus, 1, 128, groups_in_m, &bm, &bn);
+    if (bm != 128 || bn != 256) return false;
+    // the same table with every tile height allowed
+    double best = -1;
+    int tm = 0, tn = 0;
+    for (const TileCost& t : kFp8Tiles) {
+        if ((t.bn != 64 && t.bn != 128 && t.bn != 256) || (t.bm != 64 && t.bm != 128 && t.bm != 256)) continue;
+        const long long count  = (long long)((m + t.bm - 1) / t.bm) * ((n + t.bn - 1) / t.bn);
+        const long long rounds = (count + num_cus - 1) / num_cus;
+        const double cost = double(rounds) * t.bm * t.bn * t.per_area;
+        if (best < 0 || cost < best || (cost == best && (t.bm < tm || (t.bm == tm && t.bn < tn)))) { best = cost; tm = t.bm; tn = t.bn; }
+    }
+    return tm == 256 && tn == 256;
+}
+
 // Activation atoms of the weight-streaming kernel, or 0 for the tiled kernel (get_skinny_fp8_config in heuristics.py).
 int skinny_atoms(int m, int n, int num_cus) {
     return (m > 0 && m <= 16 && n >= 16 && n <= 16 * num_cus) ? 1 : 0;
@@ -309,6 +329,10 @@ int yan_m_grouped_gemm_fp8_fp8_bf16_nt_contiguous(const void* lhs, const float* 
     const long long last = (long long)(m - 1) * lhs_scales_stride_m + (long long)(k / 128 - 1) * lhs_scales_stride_k;
     if (lhs_scales_stride_m < 0 || lhs_scales_stride_k < 0 || last >= (1ll << 28)) return int(hipErrorInvalidValue);
     const int cus = (num_sms > 0 && num_sms < device_cus()) ? num_sms : device_cus();
+    if (rows_on_device(m, n, cus, num_groups))
+        return int(yan::Gemm<0, 0, 256, 256, 128, 1, 2, 1, yan::GemmType::GroupedContiguous>::run_grouped_rows_on_device(
+            static_cast<__hip_bfloat16*>(out), lhs, lhs_scales, int(lhs_scales_stride_m), int(lhs_scales_stride_k), rhs, rhs_scales, m_indices,
+            num_groups, m, n, k, static_cast<hipStream_t>(stream), num_sms));
     int bm = 0, bn = 0;
     pick_grouped(m, n, cus, 1, 128, num_groups, &bm, &bn);
 #define YAN_GROUPED_CASE(BM, BN)                                                                                     \
@@ -371,6 +395,7 @@ int yan_gemm_select_tile(int op, int m, int n, int k, int num_cus, int* block_m,
     }
     else if (op == 2) pick_grouped(m, n, num_cus, 1, 128, k, block_m, block_n);
     else if (op == 3) { const yan::FloatTile t = yan::pick_float_tile(m, n, num_cus); *block_m = t.block_m; *block_n = t.block_n; }
+    else if (op == 4) { const bool device = rows_on_device(m, n, num_cus, k); *block_m = device ? 256 : 0; *block_n = device ? 256 : 0; }
     else return 1;
     return 0;
 }
@@ -383,6 +408,6 @@ int yan_gemm_select_split_k(int op, int m, int n, int k, int num_cus, int* block
     return 0;
 }
 
-const char* yan_gemm_version(void) { return "yan-gemm gfx950 11 dense + 22 split-K dense + 2 weight-streaming dense + 7 fp32 + 10 fp8 tile variants + 15 split-K fp8 variants + 1 weight-streaming fp8 variant + 12 grouped fp8 variants + 4 quantiser kernels"; }
+const char* yan_gemm_version(void) { return "yan-gemm gfx950 11 dense + 22 split-K dense + 2 weight-streaming dense + 7 fp32 + 10 fp8 tile variants + 15 split-K fp8 variants + 1 weight-streaming fp8 variant + 13 grouped fp8 variants + 4 quantiser kernels"; }
 
 } // extern "C"

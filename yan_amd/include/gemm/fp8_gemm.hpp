@@ -264,13 +264,16 @@ contiguous_row_at(const int* __restrict__ grouped_layout, int m, int tiles_m, in
 
 // STAGES: 2 = two LDS stages with the next k-tile's scales in registers; 3.. = a ring of that many stages.
 // One output tile (one slot of the launch: `bid` is what blockIdx.x would be with a workgroup per slot).
-template <int SHAPE_N, int SHAPE_K, int BLOCK_M, int BLOCK_N, GemmType kGemmType, int STAGES, int SPLIT_K = 1>
+// EXTERNAL_RING: the ring of a tile with STAGES > 2 lives in `ring_lds` (LDS the caller declared, 1024-byte aligned, at least
+// STAGES * Fp8TileConfig::RING_STAGE_BYTES) instead of an array of this function's own: for kernels that hold two kinds of
+// tile and run one of them (fp8_gemm_contiguous_rows_kernel).
+template <int SHAPE_N, int SHAPE_K, int BLOCK_M, int BLOCK_N, GemmType kGemmType, int STAGES, int SPLIT_K = 1, bool EXTERNAL_RING = false>
 __device__ __forceinline__ void
 fp8_gemm_tile(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_scales,
               const uint8_t* __restrict__ rhs, const float* __restrict__ rhs_scales,
               __bf16* __restrict__ out, int m, int n_rt, int k_rt, int sa_stride_m, int sa_stride_k,
               const int* __restrict__ grouped_layout, int sa_stride_g, int bid, int num_groups, int expected_m, Fp8TwoStages two_stages,
-              float* __restrict__ partials = nullptr, unsigned* __restrict__ counters = nullptr) {
+              float* __restrict__ partials = nullptr, unsigned* __restrict__ counters = nullptr, uint8_t* ring_lds = nullptr) {
     using Cfg  = Fp8TileConfig<BLOCK_M, BLOCK_N>;
     using Atom = MfmaFP8_16x16x128;
     // NW waves compute (and copy); LW are launched: the extra ones of the decode tiles only copy.
@@ -503,7 +506,11 @@ fp8_gemm_tile(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_sca
     constexpr int STAGE_BYTES = Cfg::RING_STAGE_BYTES, A_BYTES = Cfg::LDS_ROWS_A * kRowBytes, TILE_BYTES = A_BYTES + Cfg::LDS_ROWS_B * kRowBytes;
     constexpr int OPS = StA::PASSES + StB::PASSES + 1, SCALE_PARTS = BLOCK_M >= 64 ? BLOCK_M / 64 : 1;
     static_assert(Cfg::RING_CAPABLE && (fp8_ring_group(BLOCK_M, BLOCK_N, STAGES) > 1 || (STAGES - 2) * OPS <= 63) && STAGES * STAGE_BYTES <= 160 * 1024);
-    __shared__ __attribute__((aligned(1024))) uint8_t ring[STAGES * STAGE_BYTES];
+    uint8_t* ring = ring_lds;
+    if constexpr (!EXTERNAL_RING) {
+        __shared__ __attribute__((aligned(1024))) uint8_t own_ring[STAGES * STAGE_BYTES];
+        ring = own_ring;
+    }
     const uint32_t scale_voff = uint32_t(m0 + lane) * sa_stride_m * 4;
     auto issue_op = [&](int d, int kb, uint8_t* stage) {
         const bool live = kb < kb_hi;
@@ -887,6 +894,54 @@ fp8_gemm_kernel(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_s
     }
 }
 
+// Contiguous groups of a few hundred rows: whether 256-row tiles pay is in the caller's layout, on the device. A 256-row tile
+// whose halves belong to two groups makes two passes over K and costs about 1.7 tiles, so 256 x 256 tiles win when group
+// boundaries fall on multiples of 256 rows (16 groups of 512 rows, 4096 x 7168 weights: 222 against 264 us on 128 x 256 tiles;
+// 16 of 256 rows: 133 against 152) and lose when every other boundary does not (groups of 384 and 640 rows: 291 against 279 us). The host cannot look; this kernel
+// holds both tiles, every workgroup counts the tile rows that hold two groups (two loads per lane and a ballot) and all
+// take the same decision: 256 x 256 tiles when no tile row holds two groups, else 128 x 256 (with two such rows of 32 the tall
+// tiles already lose 5 %: their tiles take 1.7 tile times and whoever runs one finishes last). It is
+// launched with the slots of the 128-row tiling, the larger number: in the 256-row case the workgroups beyond its slots
+// leave at once, behind everyone else in the launch order. One pool of LDS serves either tile. Same bits either way.
+template <int SHAPE_N, int SHAPE_K, int BLOCK_N>
+__global__ void __launch_bounds__(8 * kWaveSize)
+fp8_gemm_contiguous_rows_kernel(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_scales,
+                                const uint8_t* __restrict__ rhs, const float* __restrict__ rhs_scales,
+                                __bf16* __restrict__ out, int m, int n_rt, int k_rt, int sa_stride_m, int sa_stride_k,
+                                const int* __restrict__ grouped_layout, int num_groups) {
+    using Tall = Fp8TileConfig<256, BLOCK_N>;
+    using Flat = Fp8TileConfig<128, BLOCK_N>;
+    constexpr int FLAT_STAGES = Flat::MAX_RING_STAGES;
+    constexpr int TALL_BYTES = 2 * (Tall::LDS_ROWS_A + Tall::LDS_ROWS_B) * kRowBytes, FLAT_BYTES = FLAT_STAGES * Flat::RING_STAGE_BYTES;
+    static_assert(FLAT_STAGES >= 3 && fp8_launch_waves(256, BLOCK_N, 2) == 8 && fp8_launch_waves(128, BLOCK_N, FLAT_STAGES) == 8);
+    __shared__ __attribute__((aligned(1024))) uint8_t pool[TALL_BYTES > FLAT_BYTES ? TALL_BYTES : FLAT_BYTES];
+    const int N = SHAPE_N ? SHAPE_N : n_rt;
+    const int tall_rows = ceil_div(m, 256);
+    const int two_group_rows = count_two_group_rows(grouped_layout, m, tall_rows, get_lane_id());
+    const int grid = gridDim.x;
+    if (two_group_rows == 0) {
+        const int slots = int(ContiguousSlots::num_slots(m, N, 256, BLOCK_N));
+        uint8_t* const a0 = pool;
+        uint8_t* const b0 = a0 + Tall::LDS_ROWS_A * kRowBytes;
+        uint8_t* const a1 = b0 + Tall::LDS_ROWS_B * kRowBytes;
+        uint8_t* const b1 = a1 + Tall::LDS_ROWS_A * kRowBytes;
+        for (int slot = blockIdx.x; slot < slots; slot += grid) {
+            fp8_gemm_tile<SHAPE_N, SHAPE_K, 256, BLOCK_N, GemmType::GroupedContiguous, 2>(
+                lhs, lhs_scales, rhs, rhs_scales, out, m, n_rt, k_rt, sa_stride_m, sa_stride_k, grouped_layout, 0, slot, num_groups, 0,
+                Fp8TwoStages{a0, b0, a1, b1});
+            if (slot + grid < slots) __syncthreads();
+        }
+    } else {
+        const int slots = XcdTileScheduler<>(m, N, 128, BLOCK_N).grid_size();
+        for (int slot = blockIdx.x; slot < slots; slot += grid) {
+            fp8_gemm_tile<SHAPE_N, SHAPE_K, 128, BLOCK_N, GemmType::GroupedContiguous, FLAT_STAGES, 1, true>(
+                lhs, lhs_scales, rhs, rhs_scales, out, m, n_rt, k_rt, sa_stride_m, sa_stride_k, grouped_layout, 0, slot, num_groups, 0,
+                Fp8TwoStages{nullptr, nullptr, nullptr, nullptr}, nullptr, nullptr, pool);
+            if (slot + grid < slots) __syncthreads();
+        }
+    }
+}
+
 // The same tiles with K split SPLIT_K ways: launch slot s is part s % SPLIT_K of tile slot s / SPLIT_K.
 template <int SHAPE_N, int SHAPE_K, int BLOCK_M, int BLOCK_N, int STAGES, int SPLIT_K>
 __global__ void __launch_bounds__((fp8_launch_waves(BLOCK_M, BLOCK_N, STAGES) * kWaveSize))
@@ -954,6 +1009,31 @@ public:
                            static_cast<const uint8_t*>(rhs), rhs_scales, reinterpret_cast<__bf16*>(out), m, n, k,
                            lhs_scales_stride_m, lhs_scales_stride_k, grouped_layout, lhs_scales_stride_g, int(slots), num_groups,
                            expected_m);
+        return hipGetLastError();
+    }
+
+    // The contiguous layout with the tile height chosen on the device (fp8_gemm_contiguous_rows_kernel): 256 x BLOCK_N tiles when
+    // few tile rows hold two groups, else 128 x BLOCK_N. For groups of a few hundred rows; arguments as run_grouped.
+    static hipError_t run_grouped_rows_on_device(__hip_bfloat16* out, const void* lhs, const float* lhs_scales, int lhs_scales_stride_m,
+                                                 int lhs_scales_stride_k, const void* rhs, const float* rhs_scales,
+                                                 const int* grouped_layout, int num_groups, int m, int n, int k, hipStream_t stream,
+                                                 int num_sms = 0) {
+        static_assert(kGemmType == GemmType::GroupedContiguous && BLOCK_M == 256 && kNumStages == 2);
+        if (m == 0 || n == 0 || num_groups == 0) return hipSuccess;
+        if (m < 0 || n < 0 || k <= 0 || num_groups < 0 || (n % 4) != 0 || (k % 128) != 0 || (m % 128) != 0) return hipErrorInvalidValue;
+        if ((SHAPE_N && n != int(SHAPE_N)) || (SHAPE_K && k != int(SHAPE_K))) return hipErrorInvalidValue;
+        if (kNumGroups > 1 && num_groups != int(kNumGroups)) return hipErrorInvalidValue;
+        if (!out || !lhs || !lhs_scales || !rhs || !rhs_scales || !grouped_layout) return hipErrorInvalidValue;
+        const uint64_t m_pad = uint64_t(ceil_div<uint32_t>(m, BLOCK_M)) * BLOCK_M, n_pad = uint64_t(ceil_div<uint32_t>(n, BLOCK_N)) * BLOCK_N;
+        if (m_pad * k >= kOutOfRange || n_pad * k >= kOutOfRange || uint64_t(BLOCK_M) * n * 2 >= kOutOfRange) return hipErrorInvalidValue;
+        // the slots of the 128-row tiling, which are at least those of the 256-row one
+        const long long flat_slots = XcdTileScheduler<>(m, n, 128, BLOCK_N).grid_size(), tall_slots = ContiguousSlots::num_slots(m, n, 256, BLOCK_N);
+        const long long slots = flat_slots > tall_slots ? flat_slots : tall_slots;
+        if (slots >= kOutOfRange) return hipErrorInvalidValue;
+        const int grid = capped_grid(int(slots), num_sms, device_cu_count());
+        hipLaunchKernelGGL((fp8_gemm_contiguous_rows_kernel<SHAPE_N, SHAPE_K, BLOCK_N>), dim3(grid), dim3(8 * kWaveSize), 0, stream,
+                           static_cast<const uint8_t*>(lhs), lhs_scales, static_cast<const uint8_t*>(rhs), rhs_scales,
+                           reinterpret_cast<__bf16*>(out), m, n, k, lhs_scales_stride_m, lhs_scales_stride_k, grouped_layout, num_groups);
         return hipGetLastError();
     }
 

@@ -103,6 +103,20 @@ def get_best_grouped_fp8_config(m: int, n: int, k: int, num_cus: int, groups: in
     return rank_tiles(max(m, 1), n, num_cus, table, groups)[0][1]
 
 
+def get_contiguous_rows_on_device(m: int, n: int, k: int, num_cus: int, groups_in_m: int) -> bool:
+    """Whether a contiguous grouped GEMM runs the kernel that picks its tile height on the device
+    (`fp8_gemm_contiguous_rows_kernel`): groups of 256 to 1023 rows on average for which the cost table takes 128 x 256
+    tiles but would take 256 x 256 ones if no tile held two groups. Which of the two a call is stands in `m_indices`: with
+    every group boundary on a multiple of 256 rows the tall tiles are 13-17 % faster (16 groups of 512 rows x 4096 x 7168:
+    222 against 264 us), with a single boundary elsewhere they start to lose. Same rule as `rows_on_device` in
+    yan_amd/csrc/yan_gemm_capi.hip."""
+    if groups_in_m <= 0 or not 256 * groups_in_m <= m < 1024 * groups_in_m:
+        return False
+    table = {t: c for t, c in _FP8_TILES.items() if t[1] in (64, 128, 256) and t[0] in (64, 128, 256)}
+    return (get_best_grouped_fp8_config(m, n, k, num_cus, 1, 128, groups_in_m) == (128, 256) and
+            rank_tiles(m, n, num_cus, table)[0][1] == (256, 256))
+
+
 def get_skinny_fp8_config(m: int, n: int, k: int, num_cus: int) -> int:
     """Number of 16-row activation atoms (1) when the weight-streaming kernel should run instead of the tiled one, else 0:
     up to 16 activation rows, and few enough weight rows that its n/16 workgroups fit the chip in one round. Measured

@@ -13,7 +13,7 @@ from typing import Tuple
 import torch
 
 from .gemm import includes
-from .heuristics import get_best_grouped_fp8_config, get_fp8_num_stages
+from .heuristics import get_best_grouped_fp8_config, get_contiguous_rows_on_device, get_fp8_num_stages
 from .tuner import FrozenKeys, jit_tuner
 from .utils import ceil_div, current_raw_stream, get_m_alignment_for_contiguous_layout, get_num_sms, scales_for_kernel
 
@@ -37,6 +37,16 @@ __return_code = static_cast<int>(GemmType::run_grouped(out, lhs, lhs_scales, lhs
                                                        kNumGroups, m, N, K, stream, num_sms, expected_m));
 """
 
+# Contiguous groups of a few hundred rows: the kernel that holds 256 x 256 and 128 x 256 tiles and picks on the device
+# (Gemm::run_grouped_rows_on_device in gemm/fp8_gemm.hpp); same keys and arguments.
+rows_on_device_template = template.replace(
+    """GemmType::run_grouped(out, lhs, lhs_scales, lhs_scales_stride_m, lhs_scales_stride_k,
+                                                       lhs_scales_stride_g, rhs, rhs_scales, grouped_layout,
+                                                       kNumGroups, m, N, K, stream, num_sms, expected_m)""",
+    """GemmType::run_grouped_rows_on_device(out, lhs, lhs_scales, lhs_scales_stride_m, lhs_scales_stride_k,
+                                                                      rhs, rhs_scales, grouped_layout, kNumGroups, m, N, K, stream, num_sms)""")
+assert rows_on_device_template != template
+
 arg_defs = (('lhs', torch.float8_e4m3fn), ('lhs_scales', torch.float),
             ('rhs', torch.float8_e4m3fn), ('rhs_scales', torch.float),
             ('out', torch.bfloat16), ('grouped_layout', torch.int), ('m', int),
@@ -52,6 +62,11 @@ def grouped_kernel_plan(gemm_type: str, num_groups: int, m: int, n: int, k: int,
     if gemm_type == 'GroupedContiguous':
         block_m, block_n = get_best_grouped_fp8_config(m, n, k, num_cus, 1, get_m_alignment_for_contiguous_layout(), num_groups)
         name = 'm_grouped_gemm_fp8_fp8_bf16_nt'
+        if get_contiguous_rows_on_device(m, n, k, num_cus, num_groups):
+            # both tile heights in one kernel, named by the taller one
+            keys = FrozenKeys({'N': n, 'K': k, 'BLOCK_M': 256, 'BLOCK_N': 256, 'NUM_GROUPS': num_groups, 'NUM_STAGES': 2,
+                               'NUM_TMA_MULTICAST': 1, 'GEMM_TYPE': gemm_type, 'ROWS': 'picked on the device'})
+            return name + '_rows_on_device', keys, arg_defs, 2 * (256 + 256) * 128
     else:
         block_m, block_n = get_best_grouped_fp8_config(m, n, k, num_cus, num_groups)
         name = 'm_grouped_gemm_fp8_fp8_bf16_nt'
@@ -66,8 +81,8 @@ def _launch(gemm_type, num_groups, plan_m, m, n, k, lhs, lhs_scales, rhs, rhs_sc
     num_sms = get_num_sms()
     name, keys, defs, smem_size = grouped_kernel_plan(gemm_type, num_groups, plan_m, n, k, num_sms)
     args = (lhs, lhs_scales, rhs, rhs_scales, out, layout, m, current_raw_stream(), num_sms, smem_size, *strides)
-    runtime = jit_tuner.compile_and_tune(name=name, keys=keys, space=(), includes=includes,
-                                         arg_defs=defs, template=template, args=args)
+    runtime = jit_tuner.compile_and_tune(name=name, keys=keys, space=(), includes=includes, arg_defs=defs,
+                                         template=rows_on_device_template if 'ROWS' in keys else template, args=args)
     rc = runtime(*args)
     assert rc == 0, f'{name} failed with HIP error {rc}'
 
