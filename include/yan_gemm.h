@@ -136,8 +136,8 @@ YAN_API int yan_gemm_split_k_reset(void* workspace, void* stream);
  * contiguous: lhs [m,k] holds the rows of all groups one after the other, every group padded to a multiple of 128 rows
  *   (get_m_alignment_for_contiguous_layout, yan/jit_kernels/utils.py:46-55), so m % 128 == 0; m_indices[i] (device,
  *   int32 [m]) is the group of row i, constant over each aligned block of 128 rows; a negative value marks a block of
- *   padding rows, whose rows of `out` are not written. Groups that pad to multiples of 256 rows run up to 17 % faster when
- *   they hold a few hundred rows each (256-row tiles; see yan_gemm_select_tile op 4). */
+ *   padding rows, whose rows of `out` are not written. Groups of a few hundred rows that are padded to multiples of 256 rows
+ *   run up to 17 % faster than others (no 256-row tile then holds two groups; see yan_gemm_select_tile op 4). */
 YAN_API int yan_m_grouped_gemm_fp8_fp8_bf16_nt_contiguous(const void* lhs, const float* lhs_scales, long long lhs_scales_stride_m,
                                                   long long lhs_scales_stride_k, const void* rhs, const float* rhs_scales,
                                                   void* out, const int* m_indices, int num_groups, int m, int n, int k,
@@ -168,8 +168,8 @@ YAN_API int yan_per_block_cast_to_fp8(const void* w, int w_is_fp32, void* q, flo
 /* Macro tile the library uses for a problem: op 0 = dense 16-bit, 1 = FP8 block-scaled, 2 = FP8 grouped contiguous
  * (m = total rows, and `k` carries the number of groups instead of the depth), 3 = fp32. Writes BLOCK_M / BLOCK_N.
  * op 4 (m, `k` as for op 2): 256 x 256 when the contiguous entry point runs the kernel that holds 256 x 256 and 128 x 256
- * tiles and picks between them on the device (groups of 256 to 1023 rows on average: 256-row tiles when every group
- * boundary in m_indices falls on a multiple of 256 rows), 0 x 0 when it runs the tile op 2 names.
+ * tiles and decides on the device, from m_indices, which tile rows run as which (groups of 256 to 2047 rows on average),
+ * 0 x 0 when it runs the tile op 2 names.
  * For ops 0 and 1 with few activation rows the answer is (16 * atoms, 16): the weight-streaming kernels.
  * Host-only (no device call). Stands where the reference leaves tile choice to the caller's keys
  * (yan/jit_kernels/cute_gemm.py:41, yan/jit_kernels/gemm.py:13-16). Returns 0, or 1 for an unknown op. */

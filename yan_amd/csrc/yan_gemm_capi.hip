@@ -55,13 +55,11 @@ void pick_grouped(int m, int n, int num_cus, int groups, int m_alignment, int gr
     }
 }
 
-// Whether a contiguous grouped GEMM runs the kernel that picks its tile height on the device (get_contiguous_rows_on_device in
-// heuristics.py): groups of 256 to 1023 rows on average that get 128 x 256 tiles but would get 256 x 256 ones if none held two groups.
+// Whether a contiguous grouped GEMM runs the kernel that decides on the device what its 256-row tiles do about group boundaries
+// (get_contiguous_rows_on_device in heuristics.py): groups of 256 to 2047 rows on average that get 256 x 256 tiles when every
+// tile height is allowed.
 bool rows_on_device(int m, int n, int num_cus, int groups_in_m) {
-    if (groups_in_m <= 0 || (long long)m < 256ll * groups_in_m || (long long)m >= 1024ll * groups_in_m) return false;
-    int bm = 0, bn = 0;
-    pick_grouped(m, n, num_cus, 1, 128, groups_in_m, &bm, &bn);
-    if (bm != 128 || bn != 256) return false;
+    if (groups_in_m <= 0 || (long long)m < 256ll * groups_in_m || (long long)m >= 2048ll * groups_in_m) return false;
     // the same table with every tile height allowed
     double best = -1;
     int tm = 0, tn = 0;

@@ -267,7 +267,10 @@ contiguous_row_at(const int* __restrict__ grouped_layout, int m, int tiles_m, in
 // EXTERNAL_RING: the ring of a tile with STAGES > 2 lives in `ring_lds` (LDS the caller declared, 1024-byte aligned, at least
 // STAGES * Fp8TileConfig::RING_STAGE_BYTES) instead of an array of this function's own: for kernels that hold two kinds of
 // tile and run one of them (fp8_gemm_contiguous_rows_kernel).
-template <int SHAPE_N, int SHAPE_K, int BLOCK_M, int BLOCK_N, GemmType kGemmType, int STAGES, int SPLIT_K = 1, bool EXTERNAL_RING = false>
+// EXPLICIT_TILE: `bid` names the tile itself, row-major over the tile grid (m_idx * tiles_n + n_idx), for callers that order the
+// tiles themselves.
+template <int SHAPE_N, int SHAPE_K, int BLOCK_M, int BLOCK_N, GemmType kGemmType, int STAGES, int SPLIT_K = 1, bool EXTERNAL_RING = false,
+          bool EXPLICIT_TILE = false>
 __device__ __forceinline__ void
 fp8_gemm_tile(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_scales,
               const uint8_t* __restrict__ rhs, const float* __restrict__ rhs_scales,
@@ -304,7 +307,10 @@ fp8_gemm_tile(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_sca
     // contiguous groups of equal size start on band boundaries when the bands are as tall as a group (or divide one)
     if constexpr (kGemmType == GemmType::GroupedContiguous) sched.fit_bands_to_groups(sched.tiles_m / max(num_groups, 1));
     TileCoord tile;
-    if constexpr (kGemmType == GemmType::GroupedMasked) {
+    if constexpr (EXPLICIT_TILE) {
+        static_assert(kGemmType != GemmType::GroupedMasked);
+        tile = TileCoord{bid / sched.tiles_n, bid % sched.tiles_n, bid >= 0 && bid < sched.total};
+    } else if constexpr (kGemmType == GemmType::GroupedMasked) {
         int group;
         tile = MaskedSlots(num_groups, m, N, BLOCK_M, BLOCK_N, expected_m).tile_of(bid, &group);
         lhs        += size_t(group) * m * K;
@@ -894,15 +900,23 @@ fp8_gemm_kernel(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_s
     }
 }
 
-// Contiguous groups of a few hundred rows: whether 256-row tiles pay is in the caller's layout, on the device. A 256-row tile
-// whose halves belong to two groups makes two passes over K and costs about 1.7 tiles, so 256 x 256 tiles win when group
-// boundaries fall on multiples of 256 rows (16 groups of 512 rows, 4096 x 7168 weights: 222 against 264 us on 128 x 256 tiles;
-// 16 of 256 rows: 133 against 152) and lose when every other boundary does not (groups of 384 and 640 rows: 291 against 279 us). The host cannot look; this kernel
-// holds both tiles, every workgroup counts the tile rows that hold two groups (two loads per lane and a ballot) and all
-// take the same decision: 256 x 256 tiles when no tile row holds two groups, else 128 x 256 (with two such rows of 32 the tall
-// tiles already lose 5 %: their tiles take 1.7 tile times and whoever runs one finishes last). It is
-// launched with the slots of the 128-row tiling, the larger number: in the 256-row case the workgroups beyond its slots
-// leave at once, behind everyone else in the launch order. One pool of LDS serves either tile. Same bits either way.
+// Contiguous groups on 256-row tiles, with what a tile row that holds two groups costs decided on the device. Which rows
+// those are is in the caller's layout; the host cannot look. A 256-row tile whose halves belong to two groups makes two
+// passes over K and takes about 1.7 tile times (fp8_gemm_tile's two-pass path); as two 128 x BLOCK_N tiles on the ring its
+// halves take 1.2 to 1.3 together and can go to two workgroups, but a launch that ends on half tiles ends raggedly.
+// This kernel holds both tiles over one pool of LDS; every workgroup counts the tile rows that hold two groups (two
+// loads per lane and a ballot: `two` of `rows`) and all number the slots alike, one of three ways (measured with
+// 4096 x 7168 weights; all three give the same bits):
+//   * two * 20 < rows (long groups, or every boundary on a multiple of 256 rows): 256-row tiles throughout, the two-pass
+//     tiles first (ContiguousSlots). 16 groups of 512 rows: 225 us against 264 on 128 x 256 tiles; groups of 1920 to 2176 rows
+//     with one such row in 32: 223 against 238 for the next way;
+//   * up to a quarter of the rows: the whole 256-row tiles of the other rows first, in band order dealt to the XCDs in
+//     patches, then the half tiles of the two-group rows, the shorter jobs, which fill the end of the launch. 8 groups of
+//     896 and 1152 rows: 230 us against 251 with two-pass tiles; 16 of 384 and 640: 271 against 284 on 128-row tiles;
+//   * more than a quarter (groups of less than two tile rows: a 256-row tile has no neighbour to share its weight panel
+//     with): 128 x BLOCK_N tiles throughout. 16 groups of 384 rows: 205 us against 216 for the second way.
+// It is launched with eight slots more than the 128-row tiling has, which covers every case; workgroups beyond the last
+// slot leave at once.
 template <int SHAPE_N, int SHAPE_K, int BLOCK_N>
 __global__ void __launch_bounds__(8 * kWaveSize)
 fp8_gemm_contiguous_rows_kernel(const uint8_t* __restrict__ lhs, const float* __restrict__ lhs_scales,
@@ -915,30 +929,66 @@ fp8_gemm_contiguous_rows_kernel(const uint8_t* __restrict__ lhs, const float* __
     constexpr int TALL_BYTES = 2 * (Tall::LDS_ROWS_A + Tall::LDS_ROWS_B) * kRowBytes, FLAT_BYTES = FLAT_STAGES * Flat::RING_STAGE_BYTES;
     static_assert(FLAT_STAGES >= 3 && fp8_launch_waves(256, BLOCK_N, 2) == 8 && fp8_launch_waves(128, BLOCK_N, FLAT_STAGES) == 8);
     __shared__ __attribute__((aligned(1024))) uint8_t pool[TALL_BYTES > FLAT_BYTES ? TALL_BYTES : FLAT_BYTES];
+    uint8_t* const a0 = pool;
+    uint8_t* const b0 = a0 + Tall::LDS_ROWS_A * kRowBytes;
+    uint8_t* const a1 = b0 + Tall::LDS_ROWS_B * kRowBytes;
+    uint8_t* const b1 = a1 + Tall::LDS_ROWS_A * kRowBytes;
     const int N = SHAPE_N ? SHAPE_N : n_rt;
-    const int tall_rows = ceil_div(m, 256);
-    const int two_group_rows = count_two_group_rows(grouped_layout, m, tall_rows, get_lane_id());
+    const int lane = get_lane_id();
+    const int tall_rows = ceil_div(m, 256), tiles_n = ceil_div(N, BLOCK_N);
+    const int two_group_rows = count_two_group_rows(grouped_layout, m, tall_rows, lane);
+    // tile (row, column) of the 256-row / 128-row grid
+    auto tall_tile = [&](int row, int n_idx) {
+        fp8_gemm_tile<SHAPE_N, SHAPE_K, 256, BLOCK_N, GemmType::GroupedContiguous, 2, 1, false, true>(
+            lhs, lhs_scales, rhs, rhs_scales, out, m, n_rt, k_rt, sa_stride_m, sa_stride_k, grouped_layout, 0, row * tiles_n + n_idx, num_groups, 0,
+            Fp8TwoStages{a0, b0, a1, b1});
+    };
+    auto flat_tile = [&](int row, int n_idx) {
+        fp8_gemm_tile<SHAPE_N, SHAPE_K, 128, BLOCK_N, GemmType::GroupedContiguous, FLAT_STAGES, 1, true, true>(
+            lhs, lhs_scales, rhs, rhs_scales, out, m, n_rt, k_rt, sa_stride_m, sa_stride_k, grouped_layout, 0, row * tiles_n + n_idx, num_groups, 0,
+            Fp8TwoStages{nullptr, nullptr, nullptr, nullptr}, nullptr, nullptr, pool);
+    };
+    const int mode = two_group_rows * 20 < tall_rows ? 0 : (two_group_rows * 4 <= tall_rows ? 1 : 2);
+    // the rows that hold one group (or one group and padding), as a grid of their own (mode 1)
+    XcdTileScheduler<> whole((tall_rows - two_group_rows) * 256, N, 256, BLOCK_N);
+    whole.fit_bands_to_groups((tall_rows - two_group_rows) / max(num_groups, 1));
+    XcdTileScheduler<> flat(m, N, 128, BLOCK_N);
+    flat.fit_bands_to_groups(flat.tiles_m / max(num_groups, 1));
+    const ContiguousSlots two_pass_first(m, N, 256, BLOCK_N, num_groups, two_group_rows);
+    const int whole_slots = whole.grid_size();
+    const int slots = mode == 0 ? int(ContiguousSlots::num_slots(m, N, 256, BLOCK_N))
+                                : (mode == 1 ? whole_slots + 2 * two_group_rows * tiles_n : flat.grid_size());
+    // Either tile's code appears once (the compiler gives each copy of it its own registers, and four copies spill).
+    auto run_slot = [&](int slot) {
+        TileCoord t{0, 0, false};       // of the 256-row grid, or of the 128-row grid when `half_tile`
+        bool half_tile = false;
+        if (mode == 0) {
+            t = two_pass_first.tile_of(slot);
+            if (t.valid && two_group_rows) t.m_idx = contiguous_row_at(grouped_layout, m, tall_rows, two_group_rows, t.m_idx, lane);
+        } else if (mode == 2) {
+            t = flat.tile_of(slot);
+            half_tile = true;
+        } else if (slot < whole_slots) {
+            t = whole.dealt_band_tile_of(slot);
+            if (t.valid) t.m_idx = contiguous_row_at(grouped_layout, m, tall_rows, two_group_rows, two_group_rows + t.m_idx, lane);
+        } else {
+            const int h = slot - whole_slots, within = h % (2 * tiles_n);
+            t = TileCoord{2 * contiguous_row_at(grouped_layout, m, tall_rows, two_group_rows, h / (2 * tiles_n), lane) + (within & 1), within / 2, true};
+            half_tile = true;
+        }
+        if (!t.valid) return;
+        if (half_tile) flat_tile(t.m_idx, t.n_idx);
+        else tall_tile(t.m_idx, t.n_idx);
+    };
     const int grid = gridDim.x;
-    if (two_group_rows == 0) {
-        const int slots = int(ContiguousSlots::num_slots(m, N, 256, BLOCK_N));
-        uint8_t* const a0 = pool;
-        uint8_t* const b0 = a0 + Tall::LDS_ROWS_A * kRowBytes;
-        uint8_t* const a1 = b0 + Tall::LDS_ROWS_B * kRowBytes;
-        uint8_t* const b1 = a1 + Tall::LDS_ROWS_A * kRowBytes;
-        for (int slot = blockIdx.x; slot < slots; slot += grid) {
-            fp8_gemm_tile<SHAPE_N, SHAPE_K, 256, BLOCK_N, GemmType::GroupedContiguous, 2>(
-                lhs, lhs_scales, rhs, rhs_scales, out, m, n_rt, k_rt, sa_stride_m, sa_stride_k, grouped_layout, 0, slot, num_groups, 0,
-                Fp8TwoStages{a0, b0, a1, b1});
-            if (slot + grid < slots) __syncthreads();
-        }
-    } else {
-        const int slots = XcdTileScheduler<>(m, N, 128, BLOCK_N).grid_size();
-        for (int slot = blockIdx.x; slot < slots; slot += grid) {
-            fp8_gemm_tile<SHAPE_N, SHAPE_K, 128, BLOCK_N, GemmType::GroupedContiguous, FLAT_STAGES, 1, true>(
-                lhs, lhs_scales, rhs, rhs_scales, out, m, n_rt, k_rt, sa_stride_m, sa_stride_k, grouped_layout, 0, slot, num_groups, 0,
-                Fp8TwoStages{nullptr, nullptr, nullptr, nullptr}, nullptr, nullptr, pool);
-            if (slot + grid < slots) __syncthreads();
-        }
+    // a workgroup per slot (no cap): the tile without a loop around it
+    if (grid >= slots) {
+        if (int(blockIdx.x) < slots) run_slot(blockIdx.x);
+        return;
+    }
+    for (int slot = blockIdx.x; slot < slots; slot += grid) {
+        run_slot(slot);
+        if (slot + grid < slots) __syncthreads();
     }
 }
 
@@ -1012,8 +1062,8 @@ public:
         return hipGetLastError();
     }
 
-    // The contiguous layout with the tile height chosen on the device (fp8_gemm_contiguous_rows_kernel): 256 x BLOCK_N tiles when
-    // few tile rows hold two groups, else 128 x BLOCK_N. For groups of a few hundred rows; arguments as run_grouped.
+    // The contiguous layout with the tile height chosen on the device, tile row by tile row (fp8_gemm_contiguous_rows_kernel):
+    // 256 x BLOCK_N tiles where a tile row holds one group, 128 x BLOCK_N where it holds two. Arguments as run_grouped.
     static hipError_t run_grouped_rows_on_device(__hip_bfloat16* out, const void* lhs, const float* lhs_scales, int lhs_scales_stride_m,
                                                  int lhs_scales_stride_k, const void* rhs, const float* rhs_scales,
                                                  const int* grouped_layout, int num_groups, int m, int n, int k, hipStream_t stream,
@@ -1026,9 +1076,8 @@ public:
         if (!out || !lhs || !lhs_scales || !rhs || !rhs_scales || !grouped_layout) return hipErrorInvalidValue;
         const uint64_t m_pad = uint64_t(ceil_div<uint32_t>(m, BLOCK_M)) * BLOCK_M, n_pad = uint64_t(ceil_div<uint32_t>(n, BLOCK_N)) * BLOCK_N;
         if (m_pad * k >= kOutOfRange || n_pad * k >= kOutOfRange || uint64_t(BLOCK_M) * n * 2 >= kOutOfRange) return hipErrorInvalidValue;
-        // the slots of the 128-row tiling, which are at least those of the 256-row one
-        const long long flat_slots = XcdTileScheduler<>(m, n, 128, BLOCK_N).grid_size(), tall_slots = ContiguousSlots::num_slots(m, n, 256, BLOCK_N);
-        const long long slots = flat_slots > tall_slots ? flat_slots : tall_slots;
+        // whole tiles (rounded up to the 8 XCDs) plus two half tiles for every other tile: at most the tiles of the 128-row tiling + 8
+        const long long slots = (long long)XcdTileScheduler<>(m, n, 128, BLOCK_N).grid_size() + kNumXCD;
         if (slots >= kOutOfRange) return hipErrorInvalidValue;
         const int grid = capped_grid(int(slots), num_sms, device_cu_count());
         hipLaunchKernelGGL((fp8_gemm_contiguous_rows_kernel<SHAPE_N, SHAPE_K, BLOCK_N>), dim3(grid), dim3(8 * kWaveSize), 0, stream,

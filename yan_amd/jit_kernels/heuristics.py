@@ -104,17 +104,18 @@ def get_best_grouped_fp8_config(m: int, n: int, k: int, num_cus: int, groups: in
 
 
 def get_contiguous_rows_on_device(m: int, n: int, k: int, num_cus: int, groups_in_m: int) -> bool:
-    """Whether a contiguous grouped GEMM runs the kernel that picks its tile height on the device
-    (`fp8_gemm_contiguous_rows_kernel`): groups of 256 to 1023 rows on average for which the cost table takes 128 x 256
-    tiles but would take 256 x 256 ones if no tile held two groups. Which of the two a call is stands in `m_indices`: with
-    every group boundary on a multiple of 256 rows the tall tiles are 13-17 % faster (16 groups of 512 rows x 4096 x 7168:
-    222 against 264 us), with a single boundary elsewhere they start to lose. Same rule as `rows_on_device` in
-    yan_amd/csrc/yan_gemm_capi.hip."""
-    if groups_in_m <= 0 or not 256 * groups_in_m <= m < 1024 * groups_in_m:
+    """Whether a contiguous grouped GEMM runs the kernel that decides on the device what its 256-row tiles do about group
+    boundaries (`fp8_gemm_contiguous_rows_kernel`): groups of 256 to 2047 rows on average for which the cost table, with
+    256-row tiles allowed, takes 256 x 256 tiles. Which tile rows hold two groups stands in `m_indices`: with none (every
+    boundary on a multiple of 256 rows) 256-row tiles are 13-17 % faster than 128 x 256 ones (16 groups of 512 rows x 4096 x
+    7168: 225 against 264 us), with a few the kernel runs those rows as 128-row tiles at the end of the launch (8 groups
+    of 896 and 1152 rows: 230 against 250 us with two-pass tiles), with many it runs 128-row tiles throughout. Longer groups keep
+    the fixed 256-row tiles (within 2 % either way, and the fixed kernel is the faster when no row holds two groups). Same
+    rule as `rows_on_device` in yan_amd/csrc/yan_gemm_capi.hip."""
+    if groups_in_m <= 0 or not 256 * groups_in_m <= m < 2048 * groups_in_m:
         return False
     table = {t: c for t, c in _FP8_TILES.items() if t[1] in (64, 128, 256) and t[0] in (64, 128, 256)}
-    return (get_best_grouped_fp8_config(m, n, k, num_cus, 1, 128, groups_in_m) == (128, 256) and
-            rank_tiles(m, n, num_cus, table)[0][1] == (256, 256))
+    return rank_tiles(m, n, num_cus, table)[0][1] == (256, 256)
 
 
 def get_skinny_fp8_config(m: int, n: int, k: int, num_cus: int) -> int:
