@@ -535,6 +535,245 @@ dense_gemm_body_8w(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
     }
 }
 
+// The 256 x 256 tile with 4 waves (one per SIMD), each with a 128 x 128 slab of 16x16x32 atoms: 256 sums per lane, pinned in
+// the accumulation registers, and two thirds of the LDS fragment reads the 8-wave layout needs per k-tile (128 KB against
+// 192 KB), which is what counts where the chip's power limit sets the pace. A lone wave per SIMD has nobody to hide behind:
+// whatever it issues besides MFMAs has to fit the shadow of the MFMA in front of it, so
+//   * every copy, fragment read and scalar update sits behind an MFMA of its own, at most one between two MFMAs;
+//   * the fragments of a whole k-half (8 + 8 of them) are double-buffered in registers: a k-half is read out of LDS while
+//     the k-half before it is multiplied, three reads per row of 8 MFMAs, all of them back when the k-half ends;
+//   * LDS is a ring of five 32 KB units, a unit being one operand's k-tile: between the two k-halves of k-tile t every wave
+//     has read all of t (its two units are free) and t + 1 has landed; the copies of t + 2 go out one per row of MFMAs
+//     (a wave gets one copy instruction through per ~100 cycles, a row lasts 128), A during the first k-half of t into the
+//     fifth unit, B during the second into the unit A of t has left. A copy has one k-tile (B) or two (A) to land, and the
+//     wait in front of the barrier leaves the eight youngest copies in flight;
+//   * the lane offsets of the copies are the same for both operands and every tile (8 registers); the tile's first row and
+//     the place along K ride in the scalar offset, which the hardware adds before its bounds check.
+// Persistent like the 8-wave kernel, same walk, same K rotation per XCD, same order of summation, same bits: from the last but
+// one k-tile of a tile on the copies fetch the next tile; the epilogue turns the slab round through the fifth unit and its
+// stores drain under the next tile. For k % 64 == 0, k >= 128, n % 8 == 0; the launcher sends everything else to the
+// 8-wave kernel.
+template <typename Elem>
+__device__ __forceinline__ void
+dense_gemm_body_4w(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, Elem* __restrict__ C, int m, int n, int k) {
+    constexpr int BLOCK_M = 256, BLOCK_N = 256, TN = 8, TM = 8, WTN = 128, WTM = 128, UNITS = 5, UNIT_BYTES = 256 * kRowBytes;
+    using Frag = typename MfmaBF16_16x16x32::Frag;
+    static_assert(sizeof(Elem) == 2 && sizeof(typename MfmaF16_16x16x32::Frag) == sizeof(Frag));
+    __shared__ __attribute__((aligned(1024))) uint8_t ring[UNITS * UNIT_BYTES];
+
+    const XcdTileScheduler<> sched(m, n, BLOCK_M, BLOCK_N, (long long)k * sizeof(Elem));
+    const int num_slots = sched.grid_size();
+    const int lane = get_lane_id();
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWaveSize);
+    const int wn = wave % 2, wm = wave / 2;
+    const int g = lane / 16, col = lane % 16;
+    const uint32_t ld_bytes = uint32_t(k) * 2;
+    const __amdgpu_buffer_rsrc_t rsrc_a = make_rsrc(A, uint32_t(m) * ld_bytes);
+    const __amdgpu_buffer_rsrc_t rsrc_b = make_rsrc(B, uint32_t(n) * ld_bytes);
+    // as the 8-wave kernel: an even number of k-tiles per tile (an odd count gets one k-tile of zeros), the walk over K
+    // starting at a k-tile that depends on the tile's XCD and wrapping round
+    const int num_k_tiles = k / 64, k_tiles_run = (num_k_tiles + 1) & ~1;
+    const uint32_t k_wrap = uint32_t(k_tiles_run) * kRowBytes;
+    const int koff[2] = {frag_offset<16>(lane, 2 * g), frag_offset<16>(lane, 2 * g + 1)};
+    const int a_lane = wm * WTM * kRowBytes, b_lane = wn * WTN * kRowBytes;
+    const bool stream_out = size_t(m) * n * sizeof(Elem) > (size_t(32) << 20);
+
+    // Wave w copies rows 64 w .. 64 w + 63 of either operand's k-tile, 8 rows per pass.
+    uint32_t voff[8];
+    {
+        const int sub = lane >> 3, slot = lane & 7;
+#pragma unroll
+        for (int j = 0; j < 8; ++j)     // logical chunk: slot ^ swizzle_of_row(8 (8 w + j) + sub)
+            voff[j] = uint32_t(wave * 64 + j * 8 + sub) * ld_bytes + (slot ^ sub ^ (j & 1)) * kChunk;
+    }
+    // Where the next copies fetch: the first rows of the tile they belong to (kOutOfRange: no such tile, they move zeros),
+    // the byte along K, and the two put together (kOutOfRange for the k-tile of zeros).
+    uint32_t base_a, base_b, kpos, at_a, at_b;
+    auto aim = [&] {
+        at_a = kpos < ld_bytes ? base_a + kpos : kOutOfRange;
+        at_b = kpos < ld_bytes ? base_b + kpos : kOutOfRange;
+    };
+    auto aim_at = [&](TileCoord t, int slot) {
+        base_a = t.valid ? uint32_t(t.m_idx * BLOCK_M) * ld_bytes : kOutOfRange;
+        base_b = t.valid ? uint32_t(t.n_idx * BLOCK_N) * ld_bytes : kOutOfRange;
+        kpos = uint32_t((slot % kNumXCD) * (k_tiles_run / kNumXCD)) * kRowBytes;
+        aim();
+    };
+    // pass `r` of an operand's next k-tile into the ring unit at byte offset `unit`
+    auto copy_a = [&](int r, int unit) __attribute__((always_inline)) {
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, YAN_LDS_PTR(ring + unit + (wave * 8 + r) * 8 * kRowBytes), kChunk, voff[r], at_a, 0, 0);
+    };
+    auto copy_b = [&](int r, int unit) __attribute__((always_inline)) {
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, YAN_LDS_PTR(ring + unit + (wave * 8 + r) * 8 * kRowBytes), kChunk, voff[r], at_b, 0, 0);
+    };
+
+    f32x4 acc[TN][TM];
+    Frag nf[2][TN], mf[2][TM];
+
+    // acc[i][j] (+)= weight fragment i x activation fragment j of fragment buffer KH; FIRST: the sums start here
+    auto mma = [&](auto first_c, auto kh_c, int i, int j) __attribute__((always_inline)) {
+        constexpr int KH = decltype(kh_c)::value;
+        if constexpr (decltype(first_c)::value) {
+            if constexpr (__is_same(Elem, __bf16))
+                asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, 0" : "=a"(acc[i][j]) : "v"(nf[KH][i]), "v"(mf[KH][j]));
+            else
+                asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, 0" : "=a"(acc[i][j]) : "v"(nf[KH][i]), "v"(mf[KH][j]));
+        } else {
+            if constexpr (__is_same(Elem, __bf16))
+                asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc[i][j]) : "v"(nf[KH][i]), "v"(mf[KH][j]));
+            else
+                asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc[i][j]) : "v"(nf[KH][i]), "v"(mf[KH][j]));
+        }
+    };
+    // fragment number x of a k-half (the 8 activation fragments, then the 8 weight fragments) into buffer KH
+    auto read = [&](auto kh_c, const uint8_t* pa, const uint8_t* pb, int x) __attribute__((always_inline)) {
+        constexpr int KH = decltype(kh_c)::value;
+        if (x < TM) mf[KH][x % TM] = *reinterpret_cast<const Frag*>(pa + (x % TM) * 16 * kRowBytes);
+        else if (x < TM + TN) nf[KH][(x - TM) % TN] = *reinterpret_cast<const Frag*>(pb + ((x - TM) % TN) * 16 * kRowBytes);
+    };
+    // One k-half: 8 rows of 8 MFMAs on fragment buffer KH; the reads of the next k-half (units ua, ub; chunk set RK) go into
+    // buffer KH ^ 1, three a row; `copy(row)` and `tail(row)` once per row.
+    auto half_step = [&](auto kh_c, auto rk_c, auto first_c, int ua, int ub, auto&& copy, auto&& tail) __attribute__((always_inline)) {
+        constexpr int KH = decltype(kh_c)::value, RK = decltype(rk_c)::value;
+        using Other = std::integral_constant<int, KH ^ 1>;
+        const uint8_t* pa = ring + ua + a_lane + koff[RK];
+        const uint8_t* pb = ring + ub + b_lane + koff[RK];
+#pragma unroll
+        for (int i = 0; i < TN; ++i) {
+            mma(first_c, kh_c, i, 0); copy(i);
+            __builtin_amdgcn_sched_barrier(0);
+            mma(first_c, kh_c, i, 1); read(Other{}, pa, pb, 3 * i);
+            __builtin_amdgcn_sched_barrier(0);
+            mma(first_c, kh_c, i, 2); mma(first_c, kh_c, i, 3); read(Other{}, pa, pb, 3 * i + 1);
+            __builtin_amdgcn_sched_barrier(0);
+            mma(first_c, kh_c, i, 4); mma(first_c, kh_c, i, 5); read(Other{}, pa, pb, 3 * i + 2);
+            __builtin_amdgcn_sched_barrier(0);
+            mma(first_c, kh_c, i, 6); mma(first_c, kh_c, i, 7); tail(i);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    using Half0 = std::integral_constant<int, 0>;
+    using Half1 = std::integral_constant<int, 1>;
+
+    auto seek = [&](int slot) {
+        while (slot < num_slots && !sched.tile_of(slot).valid) slot += gridDim.x;
+        return slot;
+    };
+    int slot = seek(blockIdx.x);
+    TileCoord cur = slot < num_slots ? sched.tile_of(slot) : TileCoord{0, 0, false};
+    if (!cur.valid) return;
+    aim_at(cur, slot);
+    auto advance = [&] {
+        kpos += kRowBytes;
+        if (kpos == k_wrap) kpos = 0;
+        aim();
+    };
+    // the first two k-tiles of the first tile into units 0 .. 3
+#pragma unroll
+    for (int r = 0; r < 8; ++r) copy_a(r, 0 * UNIT_BYTES);
+#pragma unroll
+    for (int r = 0; r < 8; ++r) copy_b(r, 1 * UNIT_BYTES);
+    advance();
+#pragma unroll
+    for (int r = 0; r < 8; ++r) copy_a(r, 2 * UNIT_BYTES);
+#pragma unroll
+    for (int r = 0; r < 8; ++r) copy_b(r, 3 * UNIT_BYTES);
+    advance();
+    __builtin_amdgcn_s_waitcnt(waitcnt_imm(16, kNoWaitLgkm));
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    {
+        const uint8_t* pa = ring + a_lane + koff[0];
+        const uint8_t* pb = ring + UNIT_BYTES + b_lane + koff[0];
+#pragma unroll
+        for (int j = 0; j < TM; ++j) mf[0][j] = *reinterpret_cast<const Frag*>(pa + j * 16 * kRowBytes);
+#pragma unroll
+        for (int i = 0; i < TN; ++i) nf[0][i] = *reinterpret_cast<const Frag*>(pb + i * 16 * kRowBytes);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+
+    // byte offsets of the units that hold A and B of the current k-tile, of the next one, and of the fifth unit
+    int oa = 0, ob = UNIT_BYTES, oa1 = 2 * UNIT_BYTES, ob1 = 3 * UNIT_BYTES, o5 = 4 * UNIT_BYTES;
+    while (true) {
+        const int next_slot = seek(slot + gridDim.x);
+        const TileCoord nxt = next_slot < num_slots ? sched.tile_of(next_slot) : TileCoord{0, 0, false};
+        auto k_tile = [&](auto first_c, int kt) __attribute__((always_inline)) {
+            if (kt == k_tiles_run - 2) aim_at(nxt, next_slot);
+            half_step(Half0{}, Half1{}, first_c, oa, ob, [&](int r) __attribute__((always_inline)) { copy_a(r, o5); }, [](int) {});
+            // k-tile kt + 1 has landed (the 8 copies just issued may still be on their way); every wave is done reading k-tile kt
+            __builtin_amdgcn_s_waitcnt(waitcnt_imm(8, 0));
+            asm volatile("" ::: "memory");
+            __builtin_amdgcn_s_barrier();
+            asm volatile("" ::: "memory");
+            // behind the last copy of the k-tile the copies move on along K and the units change roles, a row apart
+            half_step(Half1{}, Half0{}, std::false_type{}, oa1, ob1, [&](int r) __attribute__((always_inline)) { copy_b(r, oa); },
+                      [&](int r) __attribute__((always_inline)) {
+                          if (r == 7) {
+                              advance();
+                              const int ta = oa, tb = ob;
+                              oa = oa1; ob = ob1; oa1 = o5; ob1 = ta; o5 = tb;
+                          }
+                      });
+        };
+        k_tile(std::true_type{}, 0);
+        for (int kt = 1; kt < k_tiles_run; ++kt) k_tile(std::false_type{}, kt);
+        asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");      // the last MFMAs retire before the epilogue reads the sums
+
+        // Epilogue: the 4 registers of atom (i, j) are n = n_slab + 16 i + 4 g + {0..3} of row m = m_slab + 16 j + col. Each wave
+        // turns its slab round through the fifth unit (B of the last k-tile: every wave left it at the last barrier, the next
+        // copies into it come behind the barrier below), 16 rows at a time, rows 2 * WTN + 16 bytes apart, and stores 4 rows x
+        // 256 bytes per instruction: lane offset fixed, the row group in the scalar offset. Rows past m fall off the end of
+        // the descriptor, lanes past n are sent there.
+        auto epilogue = [&](auto policy_c) __attribute__((always_inline)) {
+            constexpr int PITCH = 2 * WTN + 16, LANES_PER_ROW = WTN / 8, ROWS_PER_STORE = kWaveSize / LANES_PER_ROW;
+            uint8_t* region = ring + o5 + wave * (16 * PITCH);
+            const int m0 = cur.m_idx * BLOCK_M, n0 = cur.n_idx * BLOCK_N;
+            const size_t left = (size_t(m - m0) * n - n0) * sizeof(Elem);
+            const __amdgpu_buffer_rsrc_t rsrc_c = make_rsrc(C + size_t(m0) * n + n0, left < kOutOfRange ? uint32_t(left) : kOutOfRange);
+            const int r_in = lane / LANES_PER_ROW, c = lane % LANES_PER_ROW;
+            const uint32_t lane_off = n0 + wn * WTN + 8 * c < n ? uint32_t((wm * WTM + r_in) * n + wn * WTN + 8 * c) * 2u : kOutOfRange;
+            const uint32_t group_bytes = uint32_t(n) * 2u * ROWS_PER_STORE;
+#pragma unroll
+            for (int j = 0; j < TM; ++j) {
+#pragma unroll
+                for (int i = 0; i < TN; ++i) {
+                    // the sums come out of the accumulation registers here and nowhere earlier (left to the register allocator
+                    // it moves all 256 at once and spills what else is live)
+                    f32x4 sums;
+                    asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(sums[0]) : "a"(acc[i][j][0]));
+                    asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(sums[1]) : "a"(acc[i][j][1]));
+                    asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(sums[2]) : "a"(acc[i][j][2]));
+                    asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(sums[3]) : "a"(acc[i][j][3]));
+                    *reinterpret_cast<decltype(pack4(sums, Elem{}))*>(region + col * PITCH + (16 * i + 4 * g) * 2) = pack4(sums, Elem{});
+                }
+#pragma unroll
+                for (int q = 0; q < 16 / ROWS_PER_STORE; ++q) {
+                    const i32x4 v = *reinterpret_cast<const i32x4*>(region + (ROWS_PER_STORE * q + r_in) * PITCH + c * 16);
+                    __builtin_amdgcn_raw_buffer_store_b128(v, rsrc_c, lane_off, (j * (16 / ROWS_PER_STORE) + q) * group_bytes, decltype(policy_c)::value);
+                }
+            }
+        };
+        // an output larger than the L2s together is stored with the non-temporal hint (see the 8-wave kernel)
+        if (stream_out) epilogue(std::integral_constant<int, 2>{});
+        else epilogue(std::integral_constant<int, 0>{});
+        if (!nxt.valid) break;
+        cur = nxt;
+        slot = next_slot;
+        // every wave is out of the fifth unit before the next copies go into it
+        __builtin_amdgcn_s_waitcnt(waitcnt_imm(kNoWaitVm, 0));
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+    }
+}
+
+template <typename Elem>
+__global__ void __launch_bounds__(4 * kWaveSize)
+dense_gemm_mfma_4w(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, Elem* __restrict__ C, int m, int n, int k) {
+    dense_gemm_body_4w<Elem>(A, B, C, m, n, k);
+}
+
 template <typename Atom, typename Elem, int BLOCK_M, int BLOCK_N>
 __global__ void __launch_bounds__(8 * kWaveSize)
 dense_gemm_mfma_8w(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, Elem* __restrict__ C, int m, int n, int k) {
@@ -587,6 +826,11 @@ fp16_gemm_cute_split_k(const uint8_t* __restrict__ A, const uint8_t* __restrict_
     dense_gemm_body<MfmaF16_32x32x16, _Float16, BLOCK_M, BLOCK_N, STAGES, SPLIT_K>(A, B, C, m, n, k, int(blockIdx.x), partials, counters);
 }
 
+__global__ void __launch_bounds__(4 * kWaveSize)
+fp16_gemm_cute_4w(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, _Float16* __restrict__ C, int m, int n, int k) {
+    dense_gemm_body_4w<_Float16>(A, B, C, m, n, k);
+}
+
 template <int BLOCK_M, int BLOCK_N>
 __global__ void __launch_bounds__(8 * kWaveSize)
 fp16_gemm_cute_8w(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, _Float16* __restrict__ C, int m, int n, int k) {
@@ -607,19 +851,30 @@ inline hipError_t check_dense_args(int m, int n, int k, const void* a, const voi
 }
 
 // `num_sms`: the caller's compute-unit cap (0 = none), see capped_grid in scheduler.hpp.
-template <typename Atom, typename Elem, int BLOCK_M, int BLOCK_N, int STAGES = DenseTileConfig<BLOCK_M, BLOCK_N>::MAX_STAGES>
+// WAVES: 0 lets the launcher choose between the two kernels of the 256 x 256 tile, 8 names the 8-wave one (for comparisons).
+template <typename Atom, typename Elem, int BLOCK_M, int BLOCK_N, int STAGES = DenseTileConfig<BLOCK_M, BLOCK_N>::MAX_STAGES, int WAVES = 0>
 inline hipError_t launch_dense(int m, int n, int k, const void* a, const void* b, void* c, hipStream_t stream, int num_sms = 0) {
     if (m == 0 || n == 0) return hipSuccess;
     if (hipError_t e = check_dense_args(m, n, k, a, b, c, BLOCK_M, BLOCK_N); e != hipSuccess) return e;
     const XcdTileScheduler<> sched(m, n, BLOCK_M, BLOCK_N);
     const int slots = sched.grid_size();
     if constexpr (BLOCK_M == 256 && STAGES == 2) {
-        // The largest tile runs the 8-wave kernel on 16x16x32 atoms: level with the 4-wave one where the chip's power
-        // limit sets the pace (8192^3), 13 % faster at 4096^3.
         // persistent: one workgroup per CU (a multiple of the 8 XCDs, so a workgroup's tiles stay on one XCD's range),
         // or as many as the caller's cap allows
         const int cus = device_cu_count() / kNumXCD * kNumXCD;
         const int grid = capped_grid(slots < cus ? slots : cus, num_sms, device_cu_count());
+        // The 256 x 256 tile has two kernels that give the same bits: 4 waves with 128 x 128 slabs where its conditions hold
+        // (whole k-tiles, output rows of whole 16-byte segments) and K is long enough for it to pay (level at k = 256,
+        // 5 to 14 % faster from k = 1024 on), 8 waves with 128 x 64 slabs otherwise and for the narrower tiles.
+        if (WAVES == 0 && BLOCK_N == 256 && k % 64 == 0 && k >= 256 && n % 8 == 0) {
+            if constexpr (__is_same(Elem, _Float16))
+                hipLaunchKernelGGL(fp16_gemm_cute_4w, dim3(grid), dim3(4 * kWaveSize), 0, stream,
+                                   static_cast<const uint8_t*>(a), static_cast<const uint8_t*>(b), static_cast<Elem*>(c), m, n, k);
+            else
+                hipLaunchKernelGGL((dense_gemm_mfma_4w<Elem>), dim3(grid), dim3(4 * kWaveSize), 0, stream,
+                                   static_cast<const uint8_t*>(a), static_cast<const uint8_t*>(b), static_cast<Elem*>(c), m, n, k);
+            return hipGetLastError();
+        }
         if constexpr (__is_same(Elem, _Float16))
             hipLaunchKernelGGL((fp16_gemm_cute_8w<BLOCK_M, BLOCK_N>), dim3(grid), dim3(8 * kWaveSize), 0, stream,
                                static_cast<const uint8_t*>(a), static_cast<const uint8_t*>(b), static_cast<Elem*>(c), m, n, k);
@@ -674,12 +929,12 @@ inline hipError_t launch_dense_split_k(int m, int n, int k, const void* a, const
 
 // bf16 in, fp32 accumulate, bf16 out. NUM_STAGES is the number of LDS stages (2 .. DenseTileConfig::MAX_STAGES; two
 // 256x256x64 stages are 128 KB of the 160 KB, smaller tiles can hold a deeper ring).
-template <int BLOCK_M, int BLOCK_N, int NUM_STAGES>
+template <int BLOCK_M, int BLOCK_N, int NUM_STAGES, int WAVES = 0>
 inline hipError_t gemm_tn(int m, int n, int k, const __hip_bfloat16* A, const __hip_bfloat16* B, __hip_bfloat16* C,
                           hipStream_t stream, int num_sms = 0) {
     // BLOCK_N == 16 names the weight-streaming kernel for up to BLOCK_M activation rows (bf16_gemm_skinny.hpp)
     if constexpr (BLOCK_N == 16) return yan::launch_dense_skinny<yan::MfmaBF16_16x16x32, __bf16, BLOCK_M / 16, 8>(m, n, k, A, B, C, stream);
-    else return yan::launch_dense<yan::MfmaBF16_32x32x16, __bf16, BLOCK_M, BLOCK_N, NUM_STAGES>(m, n, k, A, B, C, stream, num_sms);
+    else return yan::launch_dense<yan::MfmaBF16_32x32x16, __bf16, BLOCK_M, BLOCK_N, NUM_STAGES, WAVES>(m, n, k, A, B, C, stream, num_sms);
 }
 
 // fp16 in, fp32 accumulate, fp16 out.
@@ -695,8 +950,8 @@ inline hipError_t gemm_tn_split_k(int m, int n, int k, const __half* A, const __
     return yan::launch_dense_split_k<yan::MfmaF16_32x32x16, _Float16, BLOCK_M, BLOCK_N, SPLIT_K, NUM_STAGES>(m, n, k, A, B, C, stream, workspace, workspace_bytes);
 }
 
-template <int BLOCK_M, int BLOCK_N, int NUM_STAGES>
+template <int BLOCK_M, int BLOCK_N, int NUM_STAGES, int WAVES = 0>
 inline hipError_t gemm_tn(int m, int n, int k, const __half* A, const __half* B, __half* C, hipStream_t stream, int num_sms = 0) {
     if constexpr (BLOCK_N == 16) return yan::launch_dense_skinny<yan::MfmaF16_16x16x32, _Float16, BLOCK_M / 16, 8>(m, n, k, A, B, C, stream);
-    else return yan::launch_dense<yan::MfmaF16_32x32x16, _Float16, BLOCK_M, BLOCK_N, NUM_STAGES>(m, n, k, A, B, C, stream, num_sms);
+    else return yan::launch_dense<yan::MfmaF16_32x32x16, _Float16, BLOCK_M, BLOCK_N, NUM_STAGES, WAVES>(m, n, k, A, B, C, stream, num_sms);
 }

@@ -12,14 +12,19 @@ from typing import List, Optional, Tuple
 from .utils import ceil_div
 
 # (BLOCK_M, BLOCK_N): relative time per unit of tile area. Bigger tiles reuse operands better.
-# Dense tiles: 256 rows x {256, 224, 192, 160} columns run the 8-wave kernel (two LDS stages), the others the 4-wave kernel
-# with a ring of stages. Costs of the tiles from 128 x 128 up are measured: time per output of a problem that fills four
-# whole rounds of 256 compute units with the tile (8192 x 32 BLOCK_N x 8192), relative to 256 x 256.
+# Dense tiles: 256 x 256 runs the 4-wave kernel with a ring of five LDS units (the 8-wave kernel for short or ragged K), 256 rows
+# x {224, 192, 160} columns the 8-wave kernel (two LDS stages), the others the 4-wave kernel with a ring of stages. Costs of
+# the tiles from 128 x 128 up are measured: time per output of a problem that fills four whole rounds of 256 compute units
+# with the tile (8192 x 32 BLOCK_N x 8192), relative to 256 x 256. 256 x 224, which the 8-wave kernel supports, measures
+# 1.09 there and is not in the table: where it would compete, n = 7168, the 32 tile columns it fills exactly lose to 28
+# columns of 256 x 256 tiles whose last round is partly empty (4096 x 7168 x 16384: 733 against 646 us; 8192 x 7168 x 7168:
+# 586 against 559), and a per-area cost above 256 / 224 never wins a round count.
 # 128 x 192 and 64 x 192 (ring kernel, wave slabs 96 columns wide) are for problems that leave most compute units idle with
 # 256-wide tiles and need two rounds with 128-wide ones (2048 x 2112 x 7168: 144 tiles of 128 x 256 run 85 us, 176 of 128 x 192 68 us).
-# With this table the pick is within 2 % of the fastest tile on 67 shapes swept with every tile forced in turn.
-_DENSE_TILES = {(256, 256): 1.00, (256, 224): 1.05, (256, 192): 1.10, (256, 160): 1.19, (256, 128): 1.29, (128, 256): 1.28,
-                (128, 192): 1.39, (128, 128): 1.46, (64, 192): 1.9, (64, 128): 1.94, (64, 64): 2.7}
+# With this table the pick is the fastest tile or within 1 % of it on 65 of 67 shapes swept with every tile forced in turn
+# (the others: 2048 x 5120 x 5120 7 %, 512 x 24576 x 1536 2 %).
+_DENSE_TILES = {(256, 256): 1.00, (256, 192): 1.12, (256, 160): 1.22, (256, 128): 1.32, (128, 256): 1.31,
+                (128, 192): 1.43, (128, 128): 1.51, (64, 192): 1.96, (64, 128): 2.0, (64, 64): 2.78}
 # FP8 tiles: measured over 74 shapes (m = 17 ... 8192, n = 2048 ... 32768, k = 512 ... 16384) with every tile forced in turn;
 # with these costs the model's pick is within 1 % of the fastest tile on all of them. 256 x 192 and 256 x 160 are there for
 # problems whose 256 x 256 tiles leave a round of compute units partly empty (4096 x 5120 x 5120: 320 tiles, against 512
@@ -64,11 +69,11 @@ def get_best_fp8_config(m: int, n: int, k: int, num_cus: int) -> Tuple[int, int]
 
 
 def get_dense_num_stages(block_m: int, block_n: int) -> int:
-    """LDS stages of the dense kernel for a tile: 2 for the tiles of the 8-wave kernel (256 rows, more than 128 columns),
-    else as many as the 160 KB LDS holds, at most 8 (`DenseTileConfig::MAX_STAGES` in bf16_gemm.hpp): 3 for 128 x 256,
-    ... 8 for 64 x 64."""
+    """LDS stages of the dense kernel for a tile: 2 names the persistent kernels of the tiles with 256 rows and more than 128
+    columns (8 waves on two stages, or 4 waves on a ring of five operand units for 256 x 256: the launcher chooses), else as
+    many as the 160 KB LDS holds, at most 8 (`DenseTileConfig::MAX_STAGES` in bf16_gemm.hpp): 3 for 128 x 256, ... 8 for 64 x 64."""
     if block_m == 256 and block_n > 128:
-        return 2            # the 8-wave kernel, whatever the width
+        return 2            # the persistent kernels, whatever the width
     return min(8, 160 * 1024 // ((block_m + block_n) * 128))
 
 
