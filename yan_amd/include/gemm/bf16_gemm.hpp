@@ -568,8 +568,12 @@ dense_gemm_body_4w(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
     const int wn = wave % 2, wm = wave / 2;
     const int g = lane / 16, col = lane % 16;
     const uint32_t ld_bytes = uint32_t(k) * 2;
-    const __amdgpu_buffer_rsrc_t rsrc_a = make_rsrc(A, uint32_t(m) * ld_bytes);
-    const __amdgpu_buffer_rsrc_t rsrc_b = make_rsrc(B, uint32_t(n) * ld_bytes);
+    // Four consecutive passes of a wave's copies share one LDS base (M0) and differ in the instruction's immediate offset,
+    // which the hardware adds on the LDS side and on the global side alike: the lane offsets take it back out, and the
+    // descriptors start kCopyBias bytes early so that no lane offset goes below zero.
+    constexpr uint32_t kCopyBias = 3 * 8 * kRowBytes;
+    const __amdgpu_buffer_rsrc_t rsrc_a = make_rsrc(A - kCopyBias, uint32_t(m) * ld_bytes + kCopyBias);
+    const __amdgpu_buffer_rsrc_t rsrc_b = make_rsrc(B - kCopyBias, uint32_t(n) * ld_bytes + kCopyBias);
     // as the 8-wave kernel: an even number of k-tiles per tile (an odd count gets one k-tile of zeros), the walk over K
     // starting at a k-tile that depends on the tile's XCD and wrapping round
     const int num_k_tiles = k / 64, k_tiles_run = (num_k_tiles + 1) & ~1;
@@ -584,7 +588,7 @@ dense_gemm_body_4w(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
         const int sub = lane >> 3, slot = lane & 7;
 #pragma unroll
         for (int j = 0; j < 8; ++j)     // logical chunk: slot ^ swizzle_of_row(8 (8 w + j) + sub)
-            voff[j] = uint32_t(wave * 64 + j * 8 + sub) * ld_bytes + (slot ^ sub ^ (j & 1)) * kChunk;
+            voff[j] = uint32_t(wave * 64 + j * 8 + sub) * ld_bytes + (slot ^ sub ^ (j & 1)) * kChunk + kCopyBias - (j & 3) * 8 * kRowBytes;
     }
     // Where the next copies fetch: the first rows of the tile they belong to (kOutOfRange: no such tile, they move zeros),
     // the byte along K, and the two put together (kOutOfRange for the k-tile of zeros).
@@ -600,12 +604,17 @@ dense_gemm_body_4w(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
         aim();
     };
     // pass `r` of an operand's next k-tile into the ring unit at byte offset `unit`
-    auto copy_a = [&](int r, int unit) __attribute__((always_inline)) {
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, YAN_LDS_PTR(ring + unit + (wave * 8 + r) * 8 * kRowBytes), kChunk, voff[r], at_a, 0, 0);
+    auto copy = [&](__amdgpu_buffer_rsrc_t rsrc, uint32_t at, int r, int unit) __attribute__((always_inline)) {
+        auto* base = YAN_LDS_PTR(ring + unit + (wave * 8 + (r & 4)) * 8 * kRowBytes);
+        switch (r & 3) {        // the immediate offset is part of the instruction
+            case 0: __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, base, kChunk, voff[r], at, 0 * 8 * kRowBytes, 0); break;
+            case 1: __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, base, kChunk, voff[r], at, 1 * 8 * kRowBytes, 0); break;
+            case 2: __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, base, kChunk, voff[r], at, 2 * 8 * kRowBytes, 0); break;
+            default: __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, base, kChunk, voff[r], at, 3 * 8 * kRowBytes, 0); break;
+        }
     };
-    auto copy_b = [&](int r, int unit) __attribute__((always_inline)) {
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, YAN_LDS_PTR(ring + unit + (wave * 8 + r) * 8 * kRowBytes), kChunk, voff[r], at_b, 0, 0);
-    };
+    auto copy_a = [&](int r, int unit) __attribute__((always_inline)) { copy(rsrc_a, at_a, r, unit); };
+    auto copy_b = [&](int r, int unit) __attribute__((always_inline)) { copy(rsrc_b, at_b, r, unit); };
 
     f32x4 acc[TN][TM];
     Frag nf[2][TN], mf[2][TM];
@@ -706,14 +715,17 @@ dense_gemm_body_4w(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
             asm volatile("" ::: "memory");
             __builtin_amdgcn_s_barrier();
             asm volatile("" ::: "memory");
-            // behind the last copy of the k-tile the copies move on along K and the units change roles, a row apart
-            half_step(Half1{}, Half0{}, std::false_type{}, oa1, ob1, [&](int r) __attribute__((always_inline)) { copy_b(r, oa); },
+            // the copies move on along K and, behind the last copy of the k-tile, the units change roles: a few scalar
+            // instructions a row, so that they ride under the MFMAs
+            uint32_t next_b;
+            const int into = oa;
+            half_step(Half1{}, Half0{}, std::false_type{}, oa1, ob1, [&](int r) __attribute__((always_inline)) { copy_b(r, into); },
                       [&](int r) __attribute__((always_inline)) {
-                          if (r == 7) {
-                              advance();
-                              const int ta = oa, tb = ob;
-                              oa = oa1; ob = ob1; oa1 = o5; ob1 = ta; o5 = tb;
-                          }
+                          if (r == 3) { kpos += kRowBytes; if (kpos == k_wrap) kpos = 0; }
+                          if (r == 4) at_a = kpos < ld_bytes ? base_a + kpos : kOutOfRange;
+                          if (r == 5) next_b = kpos < ld_bytes ? base_b + kpos : kOutOfRange;
+                          if (r == 6) { const int ta = oa1; oa1 = o5; o5 = ob; ob = ob1; ob1 = oa; oa = ta; }
+                          if (r == 7) at_b = next_b;
                       });
         };
         k_tile(std::true_type{}, 0);
@@ -866,7 +878,10 @@ inline hipError_t launch_dense(int m, int n, int k, const void* a, const void* b
         // The 256 x 256 tile has two kernels that give the same bits: 4 waves with 128 x 128 slabs where its conditions hold
         // (whole k-tiles, output rows of whole 16-byte segments) and K is long enough for it to pay (level at k = 256,
         // 5 to 14 % faster from k = 1024 on), 8 waves with 128 x 64 slabs otherwise and for the narrower tiles.
-        if (WAVES == 0 && BLOCK_N == 256 && k % 64 == 0 && k >= 256 && n % 8 == 0) {
+        // (its copies address the operands 3 KB above their descriptors' start: that much less than 2 GiB per operand)
+        const uint64_t m_pad = uint64_t(ceil_div(m, BLOCK_M)) * BLOCK_M, n_pad = uint64_t(ceil_div(n, BLOCK_N)) * BLOCK_N;
+        const bool in_reach = (m_pad > n_pad ? m_pad : n_pad) * k * 2 + 4096 < kOutOfRange;
+        if (WAVES == 0 && BLOCK_N == 256 && k % 64 == 0 && k >= 256 && n % 8 == 0 && in_reach) {
             if constexpr (__is_same(Elem, _Float16))
                 hipLaunchKernelGGL(fp16_gemm_cute_4w, dim3(grid), dim3(4 * kWaveSize), 0, stream,
                                    static_cast<const uint8_t*>(a), static_cast<const uint8_t*>(b), static_cast<Elem*>(c), m, n, k);
