@@ -363,6 +363,55 @@ def test_tied_accumulators_of_the_8_wave_kernel_stay_where_the_mfmas_left_them(t
     assert sum(1 for line in after[:first_use] if line == 's_nop 15') >= 2, 'the sums are read before the last MFMAs have retired'
 
 
+@pytest.mark.parametrize('dtype_name', ['bfloat16', 'half'])
+def test_the_4_wave_dense_kernel_keeps_its_sums_in_place_and_one_instruction_behind_each_mfma(tmp_path, dtype_name):
+    """The 4-wave kernel of the 256 x 256 tile has one wave per SIMD: a spill, a sum that wanders, or two memory instructions
+    back to back in its main loop leave the matrix core idle. Checked on the generated code (compiled for the device only):
+    no scratch; every MFMA adds into the accumulation registers it reads (or starts them from zero), 256 of them; in the
+    main loop an MFMA sits between any two copies or fragment reads; the epilogue reads
+    the sums behind the wait states written in the source."""
+    import re
+    import subprocess
+    from yan_amd.jit import cpp_format, generate
+    from yan_amd.jit.compiler import get_hipcc_compiler, get_jit_include_dir, get_offload_arch
+    from yan_amd.jit_kernels import bf16_gemm
+    dtype = getattr(torch, dtype_name)
+    _, keys, arg_defs = bf16_gemm.dense_kernel_plan(8192, 8192, 8192, dtype, 256, 0)
+    assert (keys['BLOCK_M'], keys['BLOCK_N'], keys['NUM_STAGES']) == (256, 256, 2)
+    src, asm = tmp_path / 'kernel.cu', tmp_path / 'kernel.s'
+    src.write_text(generate(bf16_gemm.includes, arg_defs, cpp_format(bf16_gemm.template, keys)))
+    subprocess.check_call([get_hipcc_compiler()[0], '-x', 'hip', '--cuda-device-only', '-S', '-std=c++20', '-O3',
+                           f'--offload-arch={get_offload_arch()}', '-Xclang', '-target-feature', '-Xclang', '-packed-fp32-ops',
+                           f'-I{get_jit_include_dir()}', str(src), '-o', str(asm)])
+    text = asm.read_text()
+    assert set(re.findall(r'\.private_segment_fixed_size:\s+(\d+)', text)) == {'0'} and 'scratch_' not in text, 'a kernel spills'
+    name = 'dense_gemm_mfma_4w' if dtype == torch.bfloat16 else 'fp16_gemm_cute_4w'
+    start = next(i for i, line in enumerate(text.split('\n')) if re.match(rf'^_ZN3yan\d*{name}\w*:', line))
+    lines = [line.split(';')[0].strip() for line in text.split('\n')[start + 1:]]
+    lines = lines[:lines.index('s_endpgm')]
+    lines = [line for line in lines if line and not line.startswith(('.', '//'))]
+    mfma = re.compile(r'^v_mfma_f32_16x16x32_(?:bf16|f16) (a\[\d+:\d+\]), v\[\d+:\d+\], v\[\d+:\d+\], (a\[\d+:\d+\]|0)$')
+    assert not [line for line in lines if line.startswith('v_mfma') and not mfma.match(line)]
+    sums = set()
+    for line in lines:
+        found = mfma.match(line)
+        if found:
+            assert found.group(2) in (found.group(1), '0'), line
+            lo, hi = map(int, re.match(r'a\[(\d+):(\d+)\]', found.group(1)).groups())
+            sums.update(range(lo, hi + 1))
+    assert sums == set(range(256))
+    # the main loop: from the second barrier (the first opens the first k-tile of the walk) to the last MFMA
+    barriers = [i for i, line in enumerate(lines) if line == 's_barrier']
+    last_mfma = max(i for i, line in enumerate(lines) if mfma.match(line))
+    loop = [line for line in lines[barriers[1] + 1:last_mfma + 1] if not line.startswith('s_') and not line.endswith(':')]
+    heavy = [i for i, line in enumerate(loop) if line.startswith(('buffer_load', 'ds_read'))]
+    assert len(heavy) >= (16 + 32) + (8 + 16)              # a k-tile of the loop and the second k-half of the first one
+    assert all(any(mfma.match(line) for line in loop[i + 1:j]) for i, j in zip(heavy, heavy[1:])), 'two copies or fragment reads with no MFMA between them'
+    after = lines[last_mfma + 1:]
+    first_read = next(i for i, line in enumerate(after) if line.startswith('v_accvgpr_read'))
+    assert sum(1 for line in after[:first_read] if line == 's_nop 15') >= 2
+
+
 @pytest.mark.parametrize('shape', [(4096, 7168, 7168), (64, 4096, 7168), (4096, 5120, 5120)])
 def test_fp8_kernels_of_the_baseline_shapes_do_not_spill(tmp_path, shape):
     """The FP8 main loop keeps 128 running sums, the fragments of a row of atoms and the scales in registers and sits close
