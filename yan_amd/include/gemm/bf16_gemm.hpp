@@ -734,36 +734,58 @@ dense_gemm_body_4w(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
 
         // Epilogue: the 4 registers of atom (i, j) are n = n_slab + 16 i + 4 g + {0..3} of row m = m_slab + 16 j + col. Each wave
         // turns its slab round through the fifth unit (B of the last k-tile: every wave left it at the last barrier, the next
-        // copies into it come behind the barrier below), 16 rows at a time, rows 2 * WTN + 16 bytes apart, and stores 4 rows x
-        // 256 bytes per instruction: lane offset fixed, the row group in the scalar offset. Rows past m fall off the end of
-        // the descriptor, lanes past n are sent there.
+        // copies into it come behind the barrier below), 16 rows x 64 columns (four atoms) at a time through two buffers of
+        // its own: the sums of piece u go into LDS, piece u - 1 comes back out as whole 128-byte row segments, piece u - 2 is
+        // stored, 8 rows x 128 bytes per instruction, so that no step waits for the LDS round trip of its own piece. Rows are
+        // 144 bytes apart in LDS (the 8-byte writes of 16 rows spread over the banks). Lane offsets are fixed, the piece rides
+        // in the scalar offset; rows past m fall off the end of the descriptor, lanes past n are sent there.
         auto epilogue = [&](auto policy_c) __attribute__((always_inline)) {
-            constexpr int PITCH = 2 * WTN + 16, LANES_PER_ROW = WTN / 8, ROWS_PER_STORE = kWaveSize / LANES_PER_ROW;
-            uint8_t* region = ring + o5 + wave * (16 * PITCH);
+            constexpr int PIECE_COLS = 64, PITCH = 2 * PIECE_COLS + 16, PIECE_BYTES = 16 * PITCH, PIECES = TM * (WTN / PIECE_COLS);
+            static_assert(4 * 2 * PIECE_BYTES <= UNIT_BYTES);
+            uint8_t* buffers = ring + o5 + wave * (2 * PIECE_BYTES);
             const int m0 = cur.m_idx * BLOCK_M, n0 = cur.n_idx * BLOCK_N;
             const size_t left = (size_t(m - m0) * n - n0) * sizeof(Elem);
             const __amdgpu_buffer_rsrc_t rsrc_c = make_rsrc(C + size_t(m0) * n + n0, left < kOutOfRange ? uint32_t(left) : kOutOfRange);
-            const int r_in = lane / LANES_PER_ROW, c = lane % LANES_PER_ROW;
-            const uint32_t lane_off = n0 + wn * WTN + 8 * c < n ? uint32_t((wm * WTM + r_in) * n + wn * WTN + 8 * c) * 2u : kOutOfRange;
-            const uint32_t group_bytes = uint32_t(n) * 2u * ROWS_PER_STORE;
+            const int r_in = lane / 8, c = lane % 8;           // a lane stores 16 bytes of row r_in (and r_in + 8) of a piece
+            uint32_t off[WTN / PIECE_COLS];
 #pragma unroll
-            for (int j = 0; j < TM; ++j) {
+            for (int h = 0; h < WTN / PIECE_COLS; ++h)
+                off[h] = n0 + wn * WTN + PIECE_COLS * h + 8 * c < n ? uint32_t((wm * WTM + r_in) * n + wn * WTN + PIECE_COLS * h + 8 * c) * 2u : kOutOfRange;
+            const uint32_t rows8 = uint32_t(n) * 2u * 8;
+            i32x4 back[2][2];
+            auto into_lds = [&](int u) __attribute__((always_inline)) {
+                const int j = u / (WTN / PIECE_COLS), h = u % (WTN / PIECE_COLS);
 #pragma unroll
-                for (int i = 0; i < TN; ++i) {
-                    // the sums come out of the accumulation registers here and nowhere earlier (left to the register allocator
-                    // it moves all 256 at once and spills what else is live)
+                for (int a = 0; a < PIECE_COLS / 16; ++a) {
+                    // the sums come out of the accumulation registers here and nowhere earlier (left to the register
+                    // allocator it moves all 256 at once and spills what else is live)
+                    const int i = h * (PIECE_COLS / 16) + a;
                     f32x4 sums;
                     asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(sums[0]) : "a"(acc[i][j][0]));
                     asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(sums[1]) : "a"(acc[i][j][1]));
                     asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(sums[2]) : "a"(acc[i][j][2]));
                     asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(sums[3]) : "a"(acc[i][j][3]));
-                    *reinterpret_cast<decltype(pack4(sums, Elem{}))*>(region + col * PITCH + (16 * i + 4 * g) * 2) = pack4(sums, Elem{});
+                    *reinterpret_cast<decltype(pack4(sums, Elem{}))*>(buffers + (u & 1) * PIECE_BYTES + col * PITCH + (16 * a + 4 * g) * 2) = pack4(sums, Elem{});
                 }
+            };
+            auto out_of_lds = [&](int u) __attribute__((always_inline)) {
 #pragma unroll
-                for (int q = 0; q < 16 / ROWS_PER_STORE; ++q) {
-                    const i32x4 v = *reinterpret_cast<const i32x4*>(region + (ROWS_PER_STORE * q + r_in) * PITCH + c * 16);
-                    __builtin_amdgcn_raw_buffer_store_b128(v, rsrc_c, lane_off, (j * (16 / ROWS_PER_STORE) + q) * group_bytes, decltype(policy_c)::value);
-                }
+                for (int s = 0; s < 2; ++s)
+                    back[u & 1][s] = *reinterpret_cast<const i32x4*>(buffers + (u & 1) * PIECE_BYTES + (8 * s + r_in) * PITCH + c * 16);
+            };
+            auto store = [&](int u) __attribute__((always_inline)) {
+                const int j = u / (WTN / PIECE_COLS), h = u % (WTN / PIECE_COLS);
+#pragma unroll
+                for (int s = 0; s < 2; ++s)
+                    __builtin_amdgcn_raw_buffer_store_b128(back[u & 1][s], rsrc_c, off[h], (2 * j + s) * rows8, decltype(policy_c)::value);
+            };
+#pragma unroll
+            for (int u = 0; u < PIECES + 2; ++u) {
+                if (u < PIECES) into_lds(u);
+                __builtin_amdgcn_sched_barrier(0);
+                if (u >= 1 && u - 1 < PIECES) out_of_lds(u - 1);
+                if (u >= 2) store(u - 2);
+                __builtin_amdgcn_sched_barrier(0);
             }
         };
         // an output larger than the L2s together is stored with the non-temporal hint (see the 8-wave kernel)
