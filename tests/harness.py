@@ -158,8 +158,11 @@ DENSE_TEST_SHAPES = [
     (2900, 5000, 64),            # same with a single k-tile
     (3000, 5000, 960),           # the 256 x 256 tile on the 4-wave kernel (whole k-tiles, an odd number of them), ragged m and n
     (2900, 5000, 256),           # same with four k-tiles, the fewest it takes
-    # the narrower tiles of the 8-wave kernel: 256 x 160 and 256 x 192, each once whole and once ragged in m, n and k
-    (4096, 5120, 512), (4000, 5000, 520), (4096, 6144, 256), (4090, 6100, 72),
+    # the narrower tiles of 256 rows: 256 x 160, 256 x 224, 256 x 192, each once whole (4-wave kernel) and once ragged in m, n
+    # and k (8-wave kernel)
+    (4096, 5120, 512), (4000, 5000, 520), (2048, 7168, 256), (2047, 7100, 264), (4096, 6144, 256), (4090, 6100, 72),
+    # and ragged in m and n on the 4-wave kernel (whole k-tiles, n a multiple of 8)
+    (4000, 5000, 576), (2047, 7096, 832), (4090, 6104, 320),
     # the 192-wide tiles of the ring kernel (wave slabs of 96 columns), whole and ragged
     (2048, 2112, 264), (2000, 2100, 136), (1024, 2112, 264), (1000, 2100, 72),
     # a handful of rows over up to 4096 weight rows: the weight-streaming kernel with one and two activation atoms, the
@@ -167,27 +170,27 @@ DENSE_TEST_SHAPES = [
     (1, 4096, 7168), (16, 2112, 1024), (7, 1156, 512), (17, 4096, 2048), (32, 272, 4096), (20, 100, 2112),
 ]
 # (shape, tile the cost model must pick): the shapes above exist for these tiles
-DENSE_TILE_OF_SHAPE = {(4096, 5120, 512): (256, 160), (4000, 5000, 520): (256, 160),
-                       (4096, 6144, 256): (256, 192), (4090, 6100, 72): (256, 192),
+DENSE_TILE_OF_SHAPE = {(4096, 5120, 512): (256, 160), (4000, 5000, 520): (256, 160), (2048, 7168, 256): (256, 224),
+                       (2047, 7100, 264): (256, 224), (4096, 6144, 256): (256, 192), (4090, 6100, 72): (256, 192),
+                       (4000, 5000, 576): (256, 160), (2047, 7096, 832): (256, 224), (4090, 6104, 320): (256, 192),
                        (3000, 5000, 1000): (256, 256), (8192, 8192, 8192): (256, 256), (3000, 5000, 960): (256, 256), (2900, 5000, 256): (256, 256),
                        (2048, 2112, 264): (128, 192), (2000, 2100, 136): (128, 192), (1024, 2112, 264): (64, 192), (1000, 2100, 72): (64, 192),
                        (1, 4096, 7168): (16, 16), (7, 1156, 512): (16, 16), (17, 4096, 2048): (32, 16), (20, 100, 2112): (32, 16)}
-# Dense kernels no call selects by itself, built with explicit keys: the 256 x 224 tile of the 8-wave kernel (the cost table
-# no longer holds it: where it fills whole rounds, n = 7168, 256 x 256 tiles with a partly empty last round are faster), whole
-# and ragged; and the 8-wave kernel of the 256 x 256 tile on shapes the launcher gives to the 4-wave kernel, to compare bits.
-DENSE_EXPLICIT_TILE_CASES = [((256, 224), (2048, 7168, 256)), ((256, 224), (2047, 7100, 264))]
-DENSE_BOTH_KERNELS_SHAPES = [(3000, 5000, 960), (2900, 5000, 256), (3840, 4096, 576), (4096, 4096, 2048)]
+# Shapes on which the launcher of the 256-row tiles takes the 4-wave kernel (whole k-tiles, at least four of them, n a multiple
+# of 8), one or two per tile width; the 8-wave kernel of the same tile is built with explicit keys to compare bits.
+DENSE_BOTH_KERNELS_SHAPES = [(3000, 5000, 960), (2900, 5000, 256), (3840, 4096, 576), (4096, 4096, 2048),
+                             (4096, 5120, 512), (4000, 5000, 576), (2047, 7096, 832), (4090, 6104, 320)]
 
 
 def dense_explicit_plan(tile, dtype=torch.bfloat16, eight_waves: bool = False):
-    """(name, keys, arg_defs, template) of a dense kernel with the tile given; `eight_waves` names the 8-wave kernel of the
-    256 x 256 tile whatever the shape."""
+    """(name, keys, arg_defs, template) of a dense kernel with the tile given; `eight_waves` names the 8-wave kernel of a
+    256-row tile whatever the shape."""
     from yan_amd.jit_kernels import bf16_gemm
     from yan_amd.jit_kernels.heuristics import get_dense_num_stages
     keys = {'BLOCK_M': tile[0], 'BLOCK_N': tile[1], 'NUM_STAGES': get_dense_num_stages(*tile), 'NUM_SMS': 0}
     template = bf16_gemm.template
     if eight_waves:
-        assert tile == (256, 256) and 'gemm_tn<BLOCK_M, BLOCK_N, kNumStages>' in template
+        assert tile[0] == 256 and tile[1] >= 160 and 'gemm_tn<BLOCK_M, BLOCK_N, kNumStages>' in template
         template = template.replace('gemm_tn<BLOCK_M, BLOCK_N, kNumStages>', 'gemm_tn<BLOCK_M, BLOCK_N, kNumStages, 8>')
     name = ('gemm_bf16_tn' if dtype == torch.bfloat16 else 'gemm_fp16_tn') + ('_eight_waves' if eight_waves else '')
     return name, keys, bf16_gemm._arg_defs(dtype), template
@@ -353,16 +356,16 @@ def jit_kernels_in_use(num_cus: int = 256):
                 if split is not None:
                     name, keys, arg_defs = split
                     add(name, arg_defs, bf16_gemm.includes, bf16_gemm.split_k_template, keys)
-    for tile, _ in DENSE_EXPLICIT_TILE_CASES:
-        name, keys, arg_defs, code_template = dense_explicit_plan(tile)
-        add(name, arg_defs, bf16_gemm.includes, code_template, keys)
     for dtype in (torch.bfloat16, torch.half):
-        name, keys, arg_defs, code_template = dense_explicit_plan((256, 256), dtype, eight_waves=True)
-        add(name, arg_defs, bf16_gemm.includes, code_template, keys)
         for m, n, k in DENSE_BOTH_KERNELS_SHAPES:
             name, keys, arg_defs = bf16_gemm.dense_kernel_plan(m, n, k, dtype, num_cus)
-            assert (keys['BLOCK_M'], keys['BLOCK_N']) == (256, 256), (m, n, k)
+            assert keys['BLOCK_M'] == 256 and keys['BLOCK_N'] >= 160, (m, n, k)
             add(name, arg_defs, bf16_gemm.includes, bf16_gemm.template, keys)
+            for cap in (7, 100):
+                name, capped_keys, arg_defs = bf16_gemm.dense_kernel_plan(m, n, k, dtype, num_cus, cap)
+                add(name, arg_defs, bf16_gemm.includes, bf16_gemm.template, capped_keys)
+            name, keys, arg_defs, code_template = dense_explicit_plan((keys['BLOCK_M'], keys['BLOCK_N']), dtype, eight_waves=True)
+            add(name, arg_defs, bf16_gemm.includes, code_template, keys)
     for m, n, k in REFERENCE_FLOAT_TEST_SHAPES + FLOAT_TEST_SHAPES + [(5120, 2048, 4096)]:
         name, keys, arg_defs = simple_gemm.float_kernel_plan(m, n, num_cus)
         add(name, arg_defs, simple_gemm.includes, simple_gemm.template, keys)

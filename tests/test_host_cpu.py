@@ -151,21 +151,23 @@ def test_fp8_shapes_of_the_gpu_suite_reach_every_tile_of_the_cost_table():
 
 
 def test_dense_shapes_of_the_gpu_suite_reach_every_tile_of_the_8_wave_kernel():
-    """A change of the cost table must not silently take the 256 x {160, 192} tiles, or the 192-wide ring tiles, out of the
-    parity tests; 256 x 224, which the table no longer holds, is tested with explicit keys."""
+    """A change of the cost table must not silently take the 256 x {160, 192, 224} tiles, or the 192-wide ring tiles, out of the
+    parity tests."""
     import harness
     for shape, tile in harness.DENSE_TILE_OF_SHAPE.items():
         assert shape in harness.DENSE_TEST_SHAPES
         assert heuristics.get_dense_tile(*shape, 256) == tile, shape
         if tile[1] != 16:
             assert heuristics.get_dense_num_stages(*tile) == (2 if tile[0] == 256 else {(128, 192): 4, (64, 192): 5}[tile])
-    assert {t for t in harness.DENSE_TILE_OF_SHAPE.values()} == {(256, 160), (256, 192), (256, 256), (128, 192), (64, 192),
+    assert {t for t in harness.DENSE_TILE_OF_SHAPE.values()} == {(256, 160), (256, 192), (256, 224), (256, 256), (128, 192), (64, 192),
                                                                  (16, 16), (32, 16)}
-    assert (256, 224) not in heuristics._DENSE_TILES and {t for t, _ in harness.DENSE_EXPLICIT_TILE_CASES} == {(256, 224)}
-    # shapes on which the launcher of the 256 x 256 tile takes the 4-wave kernel, and shapes on which it cannot
-    for m, n, k in harness.DENSE_BOTH_KERNELS_SHAPES + [(3000, 5000, 960), (8192, 8192, 8192)]:
-        assert heuristics.get_dense_tile(m, n, k, 256) == (256, 256) and k % 64 == 0 and k >= 256 and n % 8 == 0
-    assert 1000 % 64 != 0 and 5004 % 8 != 0
+    # shapes on which the launcher of the 256-row tiles takes the 4-wave kernel, every width among them, and shapes on which
+    # it cannot
+    for m, n, k in harness.DENSE_BOTH_KERNELS_SHAPES + [(8192, 8192, 8192)]:
+        tile = heuristics.get_dense_tile(m, n, k, 256)
+        assert tile[0] == 256 and tile[1] >= 160 and k % 64 == 0 and k >= 256 and n % 8 == 0
+    assert {heuristics.get_dense_tile(*shape, 256)[1] for shape in harness.DENSE_BOTH_KERNELS_SHAPES} == {160, 192, 224, 256}
+    assert 1000 % 64 != 0 and 5004 % 8 != 0 and 520 % 64 != 0 and 264 % 64 != 0 and 72 < 256
     # the weight-streaming kernel: one round of workgroups, whole K blocks, two atoms only on long K
     assert heuristics.get_skinny_dense_config(16, 4096, 7168, 256) == 1 and heuristics.get_skinny_dense_config(16, 4112, 7168, 256) == 0
     assert heuristics.get_skinny_dense_config(16, 4096, 7176, 256) == 0 and heuristics.get_skinny_dense_config(33, 4096, 7168, 256) == 0

@@ -21,7 +21,7 @@ namespace {
 struct TileCost { int bm, bn; double per_area; };
 
 // Same tables and cost model as yan_amd/jit_kernels/heuristics.py (a CPU test keeps the two in step).
-constexpr TileCost kDenseTiles[] = {{256, 256, 1.00}, {256, 192, 1.12}, {256, 160, 1.22}, {256, 128, 1.32}, {128, 256, 1.31},
+constexpr TileCost kDenseTiles[] = {{256, 256, 1.00}, {256, 224, 1.03}, {256, 192, 1.05}, {256, 160, 1.085}, {256, 128, 1.42}, {128, 256, 1.40},
                                     {128, 192, 1.43}, {128, 128, 1.51}, {64, 192, 1.96}, {64, 128, 2.0}, {64, 64, 2.78}};
 constexpr TileCost kFp8Tiles[]   = {{256, 256, 1.00}, {256, 192, 1.12}, {256, 160, 1.28}, {256, 128, 1.34}, {128, 256, 1.34}, {128, 128, 1.5},
                                     {64, 128, 2.3}, {64, 64, 3.55}, {64, 32, 4.8}, {32, 32, 7.0}};
@@ -191,7 +191,7 @@ int dense(int m, int n, int k, const void* a, const void* b, void* c, void* stre
     pick(kDenseTiles, m, n, device_cus(), &bm, &bn);
 #define YAN_DENSE_CASE(BM, BN) if (bm == BM && bn == BN) return int(yan::launch_dense<Atom, Elem, BM, BN>(m, n, k, a, b, c, s));
 #define YAN_DENSE_CASE_8W(BM, BN) if (bm == BM && bn == BN) return int(yan::launch_dense<Atom, Elem, BM, BN, 2>(m, n, k, a, b, c, s));
-    YAN_DENSE_CASE_8W(256, 256) YAN_DENSE_CASE_8W(256, 192) YAN_DENSE_CASE_8W(256, 160)
+    YAN_DENSE_CASE_8W(256, 256) YAN_DENSE_CASE_8W(256, 224) YAN_DENSE_CASE_8W(256, 192) YAN_DENSE_CASE_8W(256, 160)
     YAN_DENSE_CASE(256, 128) YAN_DENSE_CASE(128, 256) YAN_DENSE_CASE(128, 192) YAN_DENSE_CASE(128, 128) YAN_DENSE_CASE(64, 192)
     YAN_DENSE_CASE(64, 128) YAN_DENSE_CASE(64, 64)
 #undef YAN_DENSE_CASE

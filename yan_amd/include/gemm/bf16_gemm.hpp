@@ -553,10 +553,14 @@ dense_gemm_body_8w(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
 // one k-tile of a tile on the copies fetch the next tile; the epilogue turns the slab round through the fifth unit and its
 // stores drain under the next tile. For k % 64 == 0, k >= 128, n % 8 == 0; the launcher sends everything else to the
 // 8-wave kernel.
-template <typename Elem>
+template <typename Elem, int BLOCK_N>
 __device__ __forceinline__ void
 dense_gemm_body_4w(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, Elem* __restrict__ C, int m, int n, int k) {
-    constexpr int BLOCK_M = 256, BLOCK_N = 256, TN = 8, TM = 8, WTN = 128, WTM = 128, UNITS = 5, UNIT_BYTES = 256 * kRowBytes;
+    // BLOCK_N: 256, or 160, 192, 224 (wave slabs of 80 to 112 columns, 5 to 7 rows of MFMAs per k-half; the weight unit of the
+    // ring is then partly empty)
+    static_assert(BLOCK_N % 32 == 0 && BLOCK_N >= 160 && BLOCK_N <= 256);
+    constexpr int BLOCK_M = 256, TN = BLOCK_N / 32, TM = 8, WTN = BLOCK_N / 2, WTM = 128, UNITS = 5, UNIT_BYTES = 256 * kRowBytes;
+    constexpr int PASSES_A = 8, PASSES_B = BLOCK_N / 32;         // copy instructions per wave and k-tile, 8 rows each
     using Frag = typename MfmaBF16_16x16x32::Frag;
     static_assert(sizeof(Elem) == 2 && sizeof(typename MfmaF16_16x16x32::Frag) == sizeof(Frag));
     __shared__ __attribute__((aligned(1024))) uint8_t ring[UNITS * UNIT_BYTES];
@@ -582,13 +586,20 @@ dense_gemm_body_4w(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
     const int a_lane = wm * WTM * kRowBytes, b_lane = wn * WTN * kRowBytes;
     const bool stream_out = size_t(m) * n * sizeof(Elem) > (size_t(32) << 20);
 
-    // Wave w copies rows 64 w .. 64 w + 63 of either operand's k-tile, 8 rows per pass.
-    uint32_t voff[8];
+    // Wave w copies rows 64 w .. 64 w + 63 of the activation k-tile and rows BLOCK_N / 4 w .. of the weight k-tile, 8 rows per
+    // pass. Pass j of the weights has the lane offsets of pass j of the activations when the tile is 256 wide.
+    uint32_t voff[PASSES_A], voff_b[PASSES_B == PASSES_A ? 1 : PASSES_B];
     {
         const int sub = lane >> 3, slot = lane & 7;
 #pragma unroll
-        for (int j = 0; j < 8; ++j)     // logical chunk: slot ^ swizzle_of_row(8 (8 w + j) + sub)
+        for (int j = 0; j < PASSES_A; ++j)     // logical chunk: slot ^ swizzle_of_row(8 (8 w + j) + sub)
             voff[j] = uint32_t(wave * 64 + j * 8 + sub) * ld_bytes + (slot ^ sub ^ (j & 1)) * kChunk + kCopyBias - (j & 3) * 8 * kRowBytes;
+        if constexpr (PASSES_B != PASSES_A) {
+#pragma unroll
+            for (int j = 0; j < PASSES_B; ++j)
+                voff_b[j] = uint32_t(wave * (BLOCK_N / 4) + j * 8 + sub) * ld_bytes + (slot ^ sub ^ ((wave * PASSES_B + j) & 1)) * kChunk +
+                            kCopyBias - (j & 3) * 8 * kRowBytes;
+        }
     }
     // Where the next copies fetch: the first rows of the tile they belong to (kOutOfRange: no such tile, they move zeros),
     // the byte along K, and the two put together (kOutOfRange for the k-tile of zeros).
@@ -604,17 +615,20 @@ dense_gemm_body_4w(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
         aim();
     };
     // pass `r` of an operand's next k-tile into the ring unit at byte offset `unit`
-    auto copy = [&](__amdgpu_buffer_rsrc_t rsrc, uint32_t at, int r, int unit) __attribute__((always_inline)) {
-        auto* base = YAN_LDS_PTR(ring + unit + (wave * 8 + (r & 4)) * 8 * kRowBytes);
+    auto copy = [&](__amdgpu_buffer_rsrc_t rsrc, uint32_t at, uint32_t lane_off, int first_pass, int r, int unit) __attribute__((always_inline)) {
+        auto* base = YAN_LDS_PTR(ring + unit + (first_pass + (r & 4)) * 8 * kRowBytes);
         switch (r & 3) {        // the immediate offset is part of the instruction
-            case 0: __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, base, kChunk, voff[r], at, 0 * 8 * kRowBytes, 0); break;
-            case 1: __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, base, kChunk, voff[r], at, 1 * 8 * kRowBytes, 0); break;
-            case 2: __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, base, kChunk, voff[r], at, 2 * 8 * kRowBytes, 0); break;
-            default: __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, base, kChunk, voff[r], at, 3 * 8 * kRowBytes, 0); break;
+            case 0: __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, base, kChunk, lane_off, at, 0 * 8 * kRowBytes, 0); break;
+            case 1: __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, base, kChunk, lane_off, at, 1 * 8 * kRowBytes, 0); break;
+            case 2: __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, base, kChunk, lane_off, at, 2 * 8 * kRowBytes, 0); break;
+            default: __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, base, kChunk, lane_off, at, 3 * 8 * kRowBytes, 0); break;
         }
     };
-    auto copy_a = [&](int r, int unit) __attribute__((always_inline)) { copy(rsrc_a, at_a, r, unit); };
-    auto copy_b = [&](int r, int unit) __attribute__((always_inline)) { copy(rsrc_b, at_b, r, unit); };
+    auto copy_a = [&](int r, int unit) __attribute__((always_inline)) { copy(rsrc_a, at_a, voff[r], wave * PASSES_A, r, unit); };
+    auto copy_b = [&](int r, int unit) __attribute__((always_inline)) {
+        if constexpr (PASSES_B == PASSES_A) copy(rsrc_b, at_b, voff[r], wave * PASSES_B, r, unit);
+        else copy(rsrc_b, at_b, voff_b[r], wave * PASSES_B, r, unit);
+    };
 
     f32x4 acc[TN][TM];
     Frag nf[2][TN], mf[2][TM];
@@ -640,8 +654,9 @@ dense_gemm_body_4w(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
         if (x < TM) mf[KH][x % TM] = *reinterpret_cast<const Frag*>(pa + (x % TM) * 16 * kRowBytes);
         else if (x < TM + TN) nf[KH][(x - TM) % TN] = *reinterpret_cast<const Frag*>(pb + ((x - TM) % TN) * 16 * kRowBytes);
     };
-    // One k-half: 8 rows of 8 MFMAs on fragment buffer KH; the reads of the next k-half (units ua, ub; chunk set RK) go into
-    // buffer KH ^ 1, three a row; `copy(row)` and `tail(row)` once per row.
+    // One k-half: TN rows of 8 MFMAs on fragment buffer KH; the reads of the next k-half (units ua, ub; chunk set RK) go into
+    // buffer KH ^ 1, three a row; `copy(row, 0)`, `copy(row, 1)` (the narrower tiles have more activation passes than rows)
+    // and `tail(row)` once per row.
     auto half_step = [&](auto kh_c, auto rk_c, auto first_c, int ua, int ub, auto&& copy, auto&& tail) __attribute__((always_inline)) {
         constexpr int KH = decltype(kh_c)::value, RK = decltype(rk_c)::value;
         using Other = std::integral_constant<int, KH ^ 1>;
@@ -649,13 +664,15 @@ dense_gemm_body_4w(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
         const uint8_t* pb = ring + ub + b_lane + koff[RK];
 #pragma unroll
         for (int i = 0; i < TN; ++i) {
-            mma(first_c, kh_c, i, 0); copy(i);
+            mma(first_c, kh_c, i, 0); copy(i, 0);
             __builtin_amdgcn_sched_barrier(0);
             mma(first_c, kh_c, i, 1); read(Other{}, pa, pb, 3 * i);
             __builtin_amdgcn_sched_barrier(0);
             mma(first_c, kh_c, i, 2); mma(first_c, kh_c, i, 3); read(Other{}, pa, pb, 3 * i + 1);
             __builtin_amdgcn_sched_barrier(0);
-            mma(first_c, kh_c, i, 4); mma(first_c, kh_c, i, 5); read(Other{}, pa, pb, 3 * i + 2);
+            mma(first_c, kh_c, i, 4); copy(i, 1);
+            __builtin_amdgcn_sched_barrier(0);
+            mma(first_c, kh_c, i, 5); read(Other{}, pa, pb, 3 * i + 2);
             __builtin_amdgcn_sched_barrier(0);
             mma(first_c, kh_c, i, 6); mma(first_c, kh_c, i, 7); tail(i);
             __builtin_amdgcn_sched_barrier(0);
@@ -679,16 +696,16 @@ dense_gemm_body_4w(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
     };
     // the first two k-tiles of the first tile into units 0 .. 3
 #pragma unroll
-    for (int r = 0; r < 8; ++r) copy_a(r, 0 * UNIT_BYTES);
+    for (int r = 0; r < PASSES_A; ++r) copy_a(r, 0 * UNIT_BYTES);
 #pragma unroll
-    for (int r = 0; r < 8; ++r) copy_b(r, 1 * UNIT_BYTES);
+    for (int r = 0; r < PASSES_B; ++r) copy_b(r, 1 * UNIT_BYTES);
     advance();
 #pragma unroll
-    for (int r = 0; r < 8; ++r) copy_a(r, 2 * UNIT_BYTES);
+    for (int r = 0; r < PASSES_A; ++r) copy_a(r, 2 * UNIT_BYTES);
 #pragma unroll
-    for (int r = 0; r < 8; ++r) copy_b(r, 3 * UNIT_BYTES);
+    for (int r = 0; r < PASSES_B; ++r) copy_b(r, 3 * UNIT_BYTES);
     advance();
-    __builtin_amdgcn_s_waitcnt(waitcnt_imm(16, kNoWaitLgkm));
+    __builtin_amdgcn_s_waitcnt(waitcnt_imm(PASSES_A + PASSES_B, kNoWaitLgkm));
     asm volatile("" ::: "memory");
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
@@ -709,9 +726,13 @@ dense_gemm_body_4w(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
         const TileCoord nxt = next_slot < num_slots ? sched.tile_of(next_slot) : TileCoord{0, 0, false};
         auto k_tile = [&](auto first_c, int kt) __attribute__((always_inline)) {
             if (kt == k_tiles_run - 2) aim_at(nxt, next_slot);
-            half_step(Half0{}, Half1{}, first_c, oa, ob, [&](int r) __attribute__((always_inline)) { copy_a(r, o5); }, [](int) {});
+            half_step(Half0{}, Half1{}, first_c, oa, ob,
+                      [&](int r, int second) __attribute__((always_inline)) {
+                          if (!second) copy_a(r, o5);
+                          else if (TN + r < PASSES_A) copy_a(TN + r, o5);
+                      }, [](int) {});
             // k-tile kt + 1 has landed (the 8 copies just issued may still be on their way); every wave is done reading k-tile kt
-            __builtin_amdgcn_s_waitcnt(waitcnt_imm(8, 0));
+            __builtin_amdgcn_s_waitcnt(waitcnt_imm(PASSES_A, 0));
             asm volatile("" ::: "memory");
             __builtin_amdgcn_s_barrier();
             asm volatile("" ::: "memory");
@@ -719,13 +740,14 @@ dense_gemm_body_4w(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
             // instructions a row, so that they ride under the MFMAs
             uint32_t next_b;
             const int into = oa;
-            half_step(Half1{}, Half0{}, std::false_type{}, oa1, ob1, [&](int r) __attribute__((always_inline)) { copy_b(r, into); },
+            half_step(Half1{}, Half0{}, std::false_type{}, oa1, ob1,
+                      [&](int r, int second) __attribute__((always_inline)) { if (!second) copy_b(r, into); },
                       [&](int r) __attribute__((always_inline)) {
-                          if (r == 3) { kpos += kRowBytes; if (kpos == k_wrap) kpos = 0; }
-                          if (r == 4) at_a = kpos < ld_bytes ? base_a + kpos : kOutOfRange;
-                          if (r == 5) next_b = kpos < ld_bytes ? base_b + kpos : kOutOfRange;
-                          if (r == 6) { const int ta = oa1; oa1 = o5; o5 = ob; ob = ob1; ob1 = oa; oa = ta; }
-                          if (r == 7) at_b = next_b;
+                          if (r == TN - 5) { kpos += kRowBytes; if (kpos == k_wrap) kpos = 0; }
+                          if (r == TN - 4) at_a = kpos < ld_bytes ? base_a + kpos : kOutOfRange;
+                          if (r == TN - 3) next_b = kpos < ld_bytes ? base_b + kpos : kOutOfRange;
+                          if (r == TN - 2) { const int ta = oa1; oa1 = o5; o5 = ob; ob = ob1; ob1 = oa; oa = ta; }
+                          if (r == TN - 1) at_b = next_b;
                       });
         };
         k_tile(std::true_type{}, 0);
@@ -734,31 +756,35 @@ dense_gemm_body_4w(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
 
         // Epilogue: the 4 registers of atom (i, j) are n = n_slab + 16 i + 4 g + {0..3} of row m = m_slab + 16 j + col. Each wave
         // turns its slab round through the fifth unit (B of the last k-tile: every wave left it at the last barrier, the next
-        // copies into it come behind the barrier below), 16 rows x 64 columns (four atoms) at a time through two buffers of
-        // its own: the sums of piece u go into LDS, piece u - 1 comes back out as whole 128-byte row segments, piece u - 2 is
-        // stored, 8 rows x 128 bytes per instruction, so that no step waits for the LDS round trip of its own piece. Rows are
-        // 144 bytes apart in LDS (the 8-byte writes of 16 rows spread over the banks). Lane offsets are fixed, the piece rides
-        // in the scalar offset; rows past m fall off the end of the descriptor, lanes past n are sent there.
+        // copies into it come behind the barrier below), a piece of 16 rows at a time (half the slab's width for the 256-wide
+        // tile, all of it for the narrower ones) through two buffers of its own: the sums of piece u go into LDS, piece u - 1
+        // comes back out as whole row segments, 16 bytes per lane, piece u - 2 is stored, so that no step waits for the LDS
+        // round trip of its own piece. Rows are a segment and 16 bytes apart in LDS (the 8-byte writes of 16 rows spread over
+        // the banks). Lane offsets are fixed, the piece rides in the scalar offset; rows past m fall off the end of the
+        // descriptor, lanes past n or past the piece's 16 rows are sent there.
         auto epilogue = [&](auto policy_c) __attribute__((always_inline)) {
-            constexpr int PIECE_COLS = 64, PITCH = 2 * PIECE_COLS + 16, PIECE_BYTES = 16 * PITCH, PIECES = TM * (WTN / PIECE_COLS);
-            static_assert(4 * 2 * PIECE_BYTES <= UNIT_BYTES);
+            constexpr int PIECE_COLS = BLOCK_N == 256 ? 64 : WTN, PIECES_PER_GROUP = WTN / PIECE_COLS, PIECES = TM * PIECES_PER_GROUP;
+            constexpr int PITCH = 2 * PIECE_COLS + 16, PIECE_BYTES = 16 * PITCH;
+            constexpr int LANES_PER_ROW = PIECE_COLS / 8, ROWS_PER_STORE = kWaveSize / LANES_PER_ROW, STORES = ceil_div(16, ROWS_PER_STORE);
+            static_assert(4 * 2 * PIECE_BYTES + 8 * PITCH <= UNIT_BYTES);
             uint8_t* buffers = ring + o5 + wave * (2 * PIECE_BYTES);
             const int m0 = cur.m_idx * BLOCK_M, n0 = cur.n_idx * BLOCK_N;
             const size_t left = (size_t(m - m0) * n - n0) * sizeof(Elem);
             const __amdgpu_buffer_rsrc_t rsrc_c = make_rsrc(C + size_t(m0) * n + n0, left < kOutOfRange ? uint32_t(left) : kOutOfRange);
-            const int r_in = lane / 8, c = lane % 8;           // a lane stores 16 bytes of row r_in (and r_in + 8) of a piece
-            uint32_t off[WTN / PIECE_COLS];
+            const int r_in = lane / LANES_PER_ROW, c = lane % LANES_PER_ROW;    // a lane stores 16 bytes of row ROWS_PER_STORE s + r_in
+            uint32_t off[PIECES_PER_GROUP];
 #pragma unroll
-            for (int h = 0; h < WTN / PIECE_COLS; ++h)
-                off[h] = n0 + wn * WTN + PIECE_COLS * h + 8 * c < n ? uint32_t((wm * WTM + r_in) * n + wn * WTN + PIECE_COLS * h + 8 * c) * 2u : kOutOfRange;
-            const uint32_t rows8 = uint32_t(n) * 2u * 8;
-            i32x4 back[2][2];
+            for (int h = 0; h < PIECES_PER_GROUP; ++h)
+                off[h] = r_in < ROWS_PER_STORE && n0 + wn * WTN + PIECE_COLS * h + 8 * c < n
+                             ? uint32_t((wm * WTM + r_in) * n + wn * WTN + PIECE_COLS * h + 8 * c) * 2u : kOutOfRange;
+            const uint32_t row_bytes = uint32_t(n) * 2u;
+            i32x4 back[2][STORES];
             auto into_lds = [&](int u) __attribute__((always_inline)) {
-                const int j = u / (WTN / PIECE_COLS), h = u % (WTN / PIECE_COLS);
+                const int j = u / PIECES_PER_GROUP, h = u % PIECES_PER_GROUP;
 #pragma unroll
                 for (int a = 0; a < PIECE_COLS / 16; ++a) {
                     // the sums come out of the accumulation registers here and nowhere earlier (left to the register
-                    // allocator it moves all 256 at once and spills what else is live)
+                    // allocator it moves all of them at once and spills what else is live)
                     const int i = h * (PIECE_COLS / 16) + a;
                     f32x4 sums;
                     asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(sums[0]) : "a"(acc[i][j][0]));
@@ -770,14 +796,17 @@ dense_gemm_body_4w(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
             };
             auto out_of_lds = [&](int u) __attribute__((always_inline)) {
 #pragma unroll
-                for (int s = 0; s < 2; ++s)
-                    back[u & 1][s] = *reinterpret_cast<const i32x4*>(buffers + (u & 1) * PIECE_BYTES + (8 * s + r_in) * PITCH + c * 16);
+                for (int s = 0; s < STORES; ++s)
+                    back[u & 1][s] = *reinterpret_cast<const i32x4*>(buffers + (u & 1) * PIECE_BYTES + (ROWS_PER_STORE * s + r_in) * PITCH + c * 16);
             };
             auto store = [&](int u) __attribute__((always_inline)) {
-                const int j = u / (WTN / PIECE_COLS), h = u % (WTN / PIECE_COLS);
+                const int j = u / PIECES_PER_GROUP, h = u % PIECES_PER_GROUP;
 #pragma unroll
-                for (int s = 0; s < 2; ++s)
-                    __builtin_amdgcn_raw_buffer_store_b128(back[u & 1][s], rsrc_c, off[h], (2 * j + s) * rows8, decltype(policy_c)::value);
+                for (int s = 0; s < STORES; ++s) {
+                    // the last store of a piece may reach past its 16 rows
+                    const uint32_t lane_off = (16 % ROWS_PER_STORE == 0 || ROWS_PER_STORE * s + r_in < 16) ? off[h] : kOutOfRange;
+                    __builtin_amdgcn_raw_buffer_store_b128(back[u & 1][s], rsrc_c, lane_off, (16 * j + ROWS_PER_STORE * s) * row_bytes, decltype(policy_c)::value);
+                }
             };
 #pragma unroll
             for (int u = 0; u < PIECES + 2; ++u) {
@@ -802,10 +831,10 @@ dense_gemm_body_4w(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
     }
 }
 
-template <typename Elem>
+template <typename Elem, int BLOCK_N>
 __global__ void __launch_bounds__(4 * kWaveSize)
 dense_gemm_mfma_4w(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, Elem* __restrict__ C, int m, int n, int k) {
-    dense_gemm_body_4w<Elem>(A, B, C, m, n, k);
+    dense_gemm_body_4w<Elem, BLOCK_N>(A, B, C, m, n, k);
 }
 
 template <typename Atom, typename Elem, int BLOCK_M, int BLOCK_N>
@@ -860,9 +889,10 @@ fp16_gemm_cute_split_k(const uint8_t* __restrict__ A, const uint8_t* __restrict_
     dense_gemm_body<MfmaF16_32x32x16, _Float16, BLOCK_M, BLOCK_N, STAGES, SPLIT_K>(A, B, C, m, n, k, int(blockIdx.x), partials, counters);
 }
 
+template <int BLOCK_N>
 __global__ void __launch_bounds__(4 * kWaveSize)
 fp16_gemm_cute_4w(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, _Float16* __restrict__ C, int m, int n, int k) {
-    dense_gemm_body_4w<_Float16>(A, B, C, m, n, k);
+    dense_gemm_body_4w<_Float16, BLOCK_N>(A, B, C, m, n, k);
 }
 
 template <int BLOCK_M, int BLOCK_N>
@@ -897,18 +927,20 @@ inline hipError_t launch_dense(int m, int n, int k, const void* a, const void* b
         // or as many as the caller's cap allows
         const int cus = device_cu_count() / kNumXCD * kNumXCD;
         const int grid = capped_grid(slots < cus ? slots : cus, num_sms, device_cu_count());
-        // The 256 x 256 tile has two kernels that give the same bits: 4 waves with 128 x 128 slabs where its conditions hold
-        // (whole k-tiles, output rows of whole 16-byte segments) and K is long enough for it to pay (level at k = 256,
-        // 5 to 14 % faster from k = 1024 on), 8 waves with 128 x 64 slabs otherwise and for the narrower tiles.
+        // The tiles of 256 rows and 160 to 256 columns have two kernels that give the same bits: 4 waves with slabs of 128 rows
+        // where its conditions hold (whole k-tiles, output rows of whole 16-byte segments) and K is long enough for it to pay
+        // (256 x 256: level at k = 256, 5 to 14 % faster from k = 1024 on; the narrower tiles gain 8 to 20 %), 8 waves with
+        // slabs of 64 rows otherwise.
         // (its copies address the operands 3 KB above their descriptors' start: that much less than 2 GiB per operand)
         const uint64_t m_pad = uint64_t(ceil_div(m, BLOCK_M)) * BLOCK_M, n_pad = uint64_t(ceil_div(n, BLOCK_N)) * BLOCK_N;
         const bool in_reach = (m_pad > n_pad ? m_pad : n_pad) * k * 2 + 4096 < kOutOfRange;
-        if (WAVES == 0 && BLOCK_N == 256 && k % 64 == 0 && k >= 256 && n % 8 == 0 && in_reach) {
+        if constexpr (WAVES == 0 && BLOCK_N >= 160)
+        if (k % 64 == 0 && k >= 256 && n % 8 == 0 && in_reach) {
             if constexpr (__is_same(Elem, _Float16))
-                hipLaunchKernelGGL(fp16_gemm_cute_4w, dim3(grid), dim3(4 * kWaveSize), 0, stream,
+                hipLaunchKernelGGL((fp16_gemm_cute_4w<BLOCK_N>), dim3(grid), dim3(4 * kWaveSize), 0, stream,
                                    static_cast<const uint8_t*>(a), static_cast<const uint8_t*>(b), static_cast<Elem*>(c), m, n, k);
             else
-                hipLaunchKernelGGL((dense_gemm_mfma_4w<Elem>), dim3(grid), dim3(4 * kWaveSize), 0, stream,
+                hipLaunchKernelGGL((dense_gemm_mfma_4w<Elem, BLOCK_N>), dim3(grid), dim3(4 * kWaveSize), 0, stream,
                                    static_cast<const uint8_t*>(a), static_cast<const uint8_t*>(b), static_cast<Elem*>(c), m, n, k);
             return hipGetLastError();
         }

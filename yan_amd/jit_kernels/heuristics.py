@@ -12,18 +12,17 @@ from typing import List, Optional, Tuple
 from .utils import ceil_div
 
 # (BLOCK_M, BLOCK_N): relative time per unit of tile area. Bigger tiles reuse operands better.
-# Dense tiles: 256 x 256 runs the 4-wave kernel with a ring of five LDS units (the 8-wave kernel for short or ragged K), 256 rows
-# x {224, 192, 160} columns the 8-wave kernel (two LDS stages), the others the 4-wave kernel with a ring of stages. Costs of
-# the tiles from 128 x 128 up are measured: time per output of a problem that fills four whole rounds of 256 compute units
-# with the tile (8192 x 32 BLOCK_N x 8192), relative to 256 x 256. 256 x 224, which the 8-wave kernel supports, measures
-# 1.09 there and is not in the table: where it would compete, n = 7168, the 32 tile columns it fills exactly lose to 28
-# columns of 256 x 256 tiles whose last round is partly empty (4096 x 7168 x 16384: 733 against 646 us; 8192 x 7168 x 7168:
-# 586 against 559), and a per-area cost above 256 / 224 never wins a round count.
+# Dense tiles: 256 rows x {256, 224, 192, 160} columns run the persistent 4-wave kernel with a ring of five LDS units (the
+# 8-wave kernel on two stages for short or ragged K), the others the 4-wave kernel with a ring of stages. Costs of the 256-row
+# tiles are measured: time per output of a problem that fills four whole rounds of 256 compute units with the tile
+# (8192 x 32 BLOCK_N x 8192), relative to 256 x 256 (1.02-1.04, 1.035-1.06, 1.07-1.10 over three boxes). The ring tiles measure
+# 1.30-1.32 (256 x 128, 128 x 256) and 1.49 (128 x 128) there, but no problem of four rounds ever takes them: where they
+# compete, in launches of one or two rounds, a tile pays its first loads and its epilogue in full, and 1.40 / 1.42 is what
+# makes the table's pick the fastest tile or within 1.2 % of it on all 67 shapes swept with every tile forced in turn (with
+# 1.30, 128 x 256 took eight one-round shapes from 256 x 160, which is 4 to 17 % faster there).
 # 128 x 192 and 64 x 192 (ring kernel, wave slabs 96 columns wide) are for problems that leave most compute units idle with
 # 256-wide tiles and need two rounds with 128-wide ones (2048 x 2112 x 7168: 144 tiles of 128 x 256 run 85 us, 176 of 128 x 192 68 us).
-# With this table the pick is the fastest tile or within 1 % of it on 65 of 67 shapes swept with every tile forced in turn
-# (the others: 2048 x 5120 x 5120 7 %, 512 x 24576 x 1536 2 %).
-_DENSE_TILES = {(256, 256): 1.00, (256, 192): 1.12, (256, 160): 1.22, (256, 128): 1.32, (128, 256): 1.31,
+_DENSE_TILES = {(256, 256): 1.00, (256, 224): 1.03, (256, 192): 1.05, (256, 160): 1.085, (256, 128): 1.42, (128, 256): 1.40,
                 (128, 192): 1.43, (128, 128): 1.51, (64, 192): 1.96, (64, 128): 2.0, (64, 64): 2.78}
 # FP8 tiles: measured over 74 shapes (m = 17 ... 8192, n = 2048 ... 32768, k = 512 ... 16384) with every tile forced in turn;
 # with these costs the model's pick is within 1 % of the fastest tile on all of them. 256 x 192 and 256 x 160 are there for
