@@ -17,7 +17,8 @@
 //     meets one activation row per atom: one sA per lane per atom per K block, and sB is wave-uniform;
 //   * the running sums stay in architectural VGPRs (the VALU cannot address AGPRs): 128 per wave;
 //   * the output leaves through LDS: each wave turns its slab round through the stage that was consumed last and stores
-//     16 bytes per lane in row runs of 2 * WTN bytes (non-temporal when the output is larger than the L2s together);
+//     16 bytes per lane in row runs of 2 * WTN bytes (non-temporal when the output is larger than the L2s together,
+//     except in the persistent walk, whose stores are plain);
 //   * the plain GEMM on the 256-row tiles is a persistent walk: one workgroup per compute unit takes tile after tile and
 //     overlaps the seams (fp8_gemm_walk); every other case runs a workgroup per tile, or a plain loop under a cap;
 //   * problems with long K and fewer tiles than compute units split K over SPLIT_K workgroups per tile on the ring tiles
