@@ -169,6 +169,15 @@ DENSE_TEST_SHAPES = [
     # last workgroup partly past n, fewer K blocks than waves ((1, 64, 64) above), more than one pass over the waves
     (1, 4096, 7168), (16, 2112, 1024), (7, 1156, 512), (17, 4096, 2048), (32, 272, 4096), (20, 100, 2112),
 ]
+# Shapes for every 256-row tile width in turn, with the tile given (whatever the cost model would pick): the edges of what the
+# 4-wave kernel takes (four k-tiles, eight columns, one row) and seeded random ones; n a multiple of 8 and K whole k-tiles.
+def _seeded_dense_shapes(count, seed=7):
+    import random
+    rng = random.Random(seed)
+    return [(rng.randint(1, 6000), 8 * rng.randint(1, 800), 64 * rng.randint(4, 40)) for _ in range(count)]
+
+
+DENSE_SEEDED_BOTH_KERNELS_SHAPES = [(1, 8, 256), (255, 160, 256), (257, 168, 320), (5000, 8, 2560), (1, 6000, 1024), (4097, 4104, 256)] + _seeded_dense_shapes(8)
 # (shape, tile the cost model must pick): the shapes above exist for these tiles
 DENSE_TILE_OF_SHAPE = {(4096, 5120, 512): (256, 160), (4000, 5000, 520): (256, 160), (2048, 7168, 256): (256, 224),
                        (2047, 7100, 264): (256, 224), (4096, 6144, 256): (256, 192), (4090, 6100, 72): (256, 192),
@@ -365,6 +374,10 @@ def jit_kernels_in_use(num_cus: int = 256):
                 name, capped_keys, arg_defs = bf16_gemm.dense_kernel_plan(m, n, k, dtype, num_cus, cap)
                 add(name, arg_defs, bf16_gemm.includes, bf16_gemm.template, capped_keys)
             name, keys, arg_defs, code_template = dense_explicit_plan((keys['BLOCK_M'], keys['BLOCK_N']), dtype, eight_waves=True)
+            add(name, arg_defs, bf16_gemm.includes, code_template, keys)
+    for block_n in (160, 192, 224, 256):           # every width with the tile given, on either kernel (DENSE_SEEDED_BOTH_KERNELS_SHAPES)
+        for eight_waves in (False, True):
+            name, keys, arg_defs, code_template = dense_explicit_plan((256, block_n), torch.bfloat16, eight_waves)
             add(name, arg_defs, bf16_gemm.includes, code_template, keys)
     for m, n, k in REFERENCE_FLOAT_TEST_SHAPES + FLOAT_TEST_SHAPES + [(5120, 2048, 4096)]:
         name, keys, arg_defs = simple_gemm.float_kernel_plan(m, n, num_cus)

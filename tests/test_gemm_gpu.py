@@ -223,6 +223,27 @@ def _explicit_dense_runtime(tile, dtype=torch.bfloat16, eight_waves=False):
     return jit.build(name, defs, jit.generate(bf16_gemm.includes, defs, jit.cpp_format(template, keys)))
 
 
+@pytest.mark.parametrize('m,n,k', testing.DENSE_SEEDED_BOTH_KERNELS_SHAPES)
+def test_both_kernels_agree_on_every_tile_width_for_seeded_shapes(m, n, k):
+    """Every 256-row tile width in turn with the tile given, so that shapes the cost model would never hand to a width reach it
+    too (a single row, eight columns, far fewer tiles than compute units): the 4-wave and the 8-wave kernel give the same
+    bits, nothing outside the matrix is touched, and the result agrees with the oracle."""
+    _announce('dense, both kernels, tile given', torch.bfloat16, m, n, k)
+    a, b, c = testing.make_bf16_case(m, n, k, seed=m + n + k, device='cuda')
+    ref = oracle.gemm_bf16_tn_ref(_np(a), _np(b))
+    for block_n in (160, 192, 224, 256):
+        four, eight = _explicit_dense_runtime((256, block_n)), _explicit_dense_runtime((256, block_n), eight_waves=True)
+        # one allocation with a guard row behind the matrix: the kernels address rows past m through their descriptors
+        whole = torch.full((m + 1, n), float('nan'), dtype=torch.bfloat16, device='cuda')
+        got, want = whole[:m], torch.full_like(c, float('nan'))
+        assert four(m, n, k, a, b, got, torch.cuda.current_stream()) == 0
+        assert eight(m, n, k, a, b, want, torch.cuda.current_stream()) == 0
+        torch.cuda.synchronize()
+        assert torch.equal(got, want), block_n
+        assert bool(torch.isnan(whole[m]).all()), block_n
+        assert oracle.calc_diff(_np(got), ref) < BF16_TOL, block_n
+
+
 @pytest.mark.parametrize('dtype', [torch.bfloat16, torch.half])
 @pytest.mark.parametrize('m,n,k', testing.DENSE_BOTH_KERNELS_SHAPES)
 def test_both_kernels_of_the_256_row_tiles_give_the_same_bits(m, n, k, dtype):
