@@ -111,7 +111,12 @@ __device__ __forceinline__ void
 fp8_compute_k_tile(f32x4 (&acc)[TN][TM], const uint8_t* pa, const uint8_t* pb, const float (&sa)[TM], const float (&sb)[NB],
                    int rows_in_first_block, int off0, int off1, RowHook&& row_hook) {
     using Atom = MfmaFP8_16x16x128;
-    constexpr int T = TN * TM, DEPTH = 2, RING = 4;
+    // A fold three steps behind its MFMA: at two the fold still waits for the MFMA now and then (a build whose folds do not
+    // depend on the MFMAs at all runs 3-4 % faster), at three 1-1.7 % of that is back on the 256-row tiles and 4 % on
+    // 64 x 128 (cfg3 174.4 -> 172.5 us, 8192 x 7168 x 7168 333.0 -> 327.5, 512 x 4096 x 2048 9.83 -> 9.40); four and five
+    // steps, with a ring of eight partial sums, are no better than three.
+    constexpr int T = TN * TM, DEPTH = 3, RING = 4;
+    static_assert(DEPTH < RING);
     i32x8 mf[TM], nf[2];
     nf[0] = fp8_read_frag(pb, off0, off1);
 #pragma unroll
